@@ -1,0 +1,164 @@
+/*
+ * pimhip.h -- C ABI of the MI355X (gfx950) hot path of the PimAiCompiler runtime: the fp16 batch-1
+ * GEMV family and the LSTM cell stack.
+ *
+ * Every entry point replaces one piece of the interface the reference runtime reaches this path
+ * through (paths relative to the reference tree):
+ *   - the PIM SDK calls made by customAtenAddmm / customAtenMatmul
+ *     (runtime/source/executor/op_executor/aten_ops.cpp:609-932), i.e. PimCreateGemmDesc /
+ *     PimCreateBo / PimExecuteGemm / PimDestroy*;
+ *   - the LSTM forward of executeAtenLSTM1/2 and executeMIOpenLSTM1/2
+ *     (runtime/source/executor/op_executor/aten_ops_executor.cpp:2135-2399,
+ *      runtime/source/executor/op_executor/miopen_ops_executor.cpp:22-421);
+ *   - the shape logic gemmBroadcast / getGemmType
+ *     (runtime/source/executor/utils/utils.cpp:293-396).
+ *
+ * Conventions
+ *   - All data pointers are device pointers on the current HIP device unless a parameter says
+ *     "host".  fp16 tensors are IEEE binary16, densely packed unless a leading dimension is given.
+ *   - `stream` is a hipStream_t passed as void* (the reference passes streams the same way,
+ *     aten_ops.h:434-437); NULL means the null stream.  Every entry point enqueues on `stream`
+ *     and returns without synchronising, unless stated otherwise.
+ *   - The caller owns every buffer.  Nothing here allocates the outputs.
+ *   - Return value: PIMHIP_OK (0) or a PimHipStatus error; pimhip_last_error() returns a
+ *     thread-local description of the last failure.  Unsupported arguments are reported, never
+ *     silently ignored (the reference's launchers `return` silently, custom_ops.h:126-129).
+ *   - The library keeps per-device state only (workspaces keyed by device and stream).  Calls on
+ *     different streams may run concurrently; calls on one stream are ordered by that stream.
+ */
+#ifndef PIMHIP_H_
+#define PIMHIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum PimHipStatus {
+    PIMHIP_OK = 0,
+    PIMHIP_ERR_INVALID_ARGUMENT = 1,
+    PIMHIP_ERR_UNSUPPORTED = 2,
+    PIMHIP_ERR_HIP = 3,
+    PIMHIP_ERR_NOT_INITIALIZED = 4,
+    PIMHIP_ERR_TIMEOUT = 5
+} PimHipStatus;
+
+/* Activation fused into the GEMV epilogue.  Mirrors PimActFunc {NONE, ACT_RELU} (aten_ops.cpp:615-624). */
+typedef enum PimHipActFunc { PIMHIP_ACT_NONE = 0, PIMHIP_ACT_RELU = 1 } PimHipActFunc;
+
+/* Operand order of a GEMV.  Mirrors the PIM SDK's I_X_W / W_X_I (aten_ops.cpp:653,686). */
+typedef enum PimHipGemmOrder {
+    PIMHIP_I_X_W = 0, /* y[1,out] = x[1,in] . A[in,out]   ("VM") */
+    PIMHIP_W_X_I = 1  /* y[out,1] = A[out,in] . x[in,1]   ("MV") */
+} PimHipGemmOrder;
+
+/* Shape classes of a matrix product.  Mirrors GEMM_TYPE (runtime/include/executor/utils/utils.h:30-36). */
+typedef enum PimHipGemmType {
+    PIMHIP_GEMM_UNKNOWN = 0,
+    PIMHIP_GEMM_VV = 1,
+    PIMHIP_GEMM_VM = 2,
+    PIMHIP_GEMM_MV = 3,
+    PIMHIP_GEMM_MM = 4
+} PimHipGemmType;
+
+/* ---- init / teardown ------------------------------------------------------------------------ */
+
+/* Replaces PimInitialize(RT_TYPE_HIP, PIM_FP16) (runtime/source/nn_runtime.cpp:32).  Binds the library
+ * to `device` (a HIP ordinal), checks that it is a gfx950 part and creates its per-device state.
+ * May be called once per device; repeated calls are no-ops. */
+int pimhip_initialize(int device);
+
+/* Replaces PimDeinitialize() (runtime/source/nn_runtime.cpp:85).  Synchronises every initialised device
+ * and frees all workspaces and LSTM plans' internal buffers owned by the library. */
+int pimhip_deinitialize(void);
+
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char* pimhip_last_error(void);
+
+/* ---- shape logic (host, integer only) ------------------------------------------------------- */
+
+/* Replaces gemmBroadcast (utils.cpp:293-371): pads two matmul operand shapes towards rank 4.
+ * shape1/shape2 are host arrays with room for 4 entries; rank1/rank2 are in/out.  Shapes the reference
+ * leaves at a rank other than 4 (it would then read out of range in getGemmType) are returned
+ * as they are with PIMHIP_ERR_UNSUPPORTED; ranks above 4 or below 1 give PIMHIP_ERR_INVALID_ARGUMENT. */
+int pimhip_gemm_broadcast(int64_t* shape1, int* rank1, int64_t* shape2, int* rank2);
+
+/* Replaces getGemmType (utils.cpp:373-396) on two rank-4 shapes; writes a PimHipGemmType. */
+int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* other_shape4, int* gemm_type);
+
+/* ---- fp16 GEMV family ----------------------------------------------------------------------- */
+
+/* Replaces PimCreateGemmDesc + 4x PimCreateBo + PimExecuteGemm + destroys for the batch-1 cases
+ * (aten_ops.cpp:647-659, 680-692, 792-802, 828-838).
+ *   order == PIMHIP_W_X_I: weight is [out_w, in_w] row-major with row pitch ld_weight (elements)
+ *   order == PIMHIP_I_X_W: weight is [in_w, out_w] row-major with row pitch ld_weight (elements)
+ * out[out_w] = act(sum_k weight * in[k] + bias[out_w]); bias may be NULL.  fp32 accumulation, one
+ * rounding to fp16 at the store.  As in the reference's VM/MV branches there is no alpha/beta
+ * (aten_ops.cpp:627-628).  ld_weight == 0 selects the dense pitch. */
+int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
+                        int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
+
+/* Replaces the VV branch of customAtenMatmul (aten_ops.cpp:841-882): out[0] = sum_k a[k] * b[k]. */
+int pimhip_execute_dot(void* out, const void* a, const void* b, int64_t in_w, void* stream);
+
+/* Replaces executeMultiStream's N sibling GEMVs on N streams
+ * (runtime/source/executor/op_executor/stream_ops_executor.cpp:27-50) by one grouped launch on one
+ * stream.  All arrays are host arrays of `count` entries (count <= 64); entries follow
+ * pimhip_execute_gemv's meaning and all use order PIMHIP_W_X_I. */
+int pimhip_execute_gemv_group(int count, void* const* outs, const void* const* ins, const void* const* weights,
+                              const void* const* biases, const int64_t* in_ws, const int64_t* out_ws,
+                              const int* acts, void* stream);
+
+/* ---- LSTM ----------------------------------------------------------------------------------- */
+
+typedef struct PimHipLstmPlan PimHipLstmPlan;
+
+/* One-time weight preparation; replaces ModelBuilder::buildLstmParameterVector / reArangeLstmWeights
+ * (runtime/source/builder/model_builder.cpp:158-319) and the per-call MIOpen descriptor and workspace
+ * set-up (miopen_ops_executor.cpp:109-160).
+ *   params: host array of n_params device pointers in LibTorch order, per layer then per direction
+ *           (w_ih [4H, I_l], w_hh [4H, H], then b_ih [4H], b_hh [4H] when has_biases), gate order
+ *           (i, f, g, o); I_0 = input_size, I_l = num_directions * H for l > 0.
+ * The plan keeps the caller's weight pointers (they must outlive the plan), pre-adds b_ih + b_hh, and
+ * owns the internal buffers for up to max_seq_len steps.  Runs on `stream` and synchronises it. */
+int pimhip_lstm_plan_create(PimHipLstmPlan** plan, const void* const* params, int n_params, int has_biases,
+                            int num_layers, int bidirectional, int64_t input_size, int64_t hidden_size,
+                            int64_t max_seq_len, void* stream);
+
+int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan);
+
+/* Replaces atenLstm1 / atenLstm2 with batch 1 (aten_ops.cpp:328-344) and miopenRNNForwardInference
+ * (miopen_ops_executor.cpp:175,230,393,411).  Inference only (dropout is forced to 0 by the reference,
+ * aten_ops.cpp:333,342).
+ *   x  [seq_len, input_size]            (batch 1: the same bytes for [T,1,I], [1,T,I] and packed [T,I])
+ *   h0, c0 [num_layers*num_directions, hidden_size]
+ *   y  [seq_len, num_directions*hidden_size]
+ *   hn, cn [num_layers*num_directions, hidden_size], ordered (l0 fwd, l0 bwd, l1 fwd, ...)
+ * y, hn, cn may not alias x, h0, c0.  Calls sharing one plan must be ordered on one stream. */
+int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn,
+                        void* cn, int64_t seq_len, void* stream);
+
+/* After the stream has been synchronised: 0 if every persistent-kernel wait in the last forward of this plan
+ * completed, PIMHIP_ERR_TIMEOUT if a bounded wait gave up (the outputs are then undefined). */
+int pimhip_lstm_plan_status(PimHipLstmPlan* plan);
+
+/* Upper bound on the polls of one wait inside the persistent kernel (default 2^22, roughly seconds).  A wait
+ * that reaches it gives up, the kernel still runs to its end, and pimhip_lstm_plan_status reports the time-out.
+ * Tests of that error path pass 0 here so that every wait gives up at once. */
+int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limit);
+
+/* Selects how pimhip_lstm_forward runs the recurrence: 0 = automatic, 1 = one fused launch per step,
+ * 2 = persistent sequence kernel (fails with PIMHIP_ERR_UNSUPPORTED if the shape does not fit). */
+int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);
+
+/* The dense input projection of one LSTM layer over all time steps, the only MFMA kernel of the path:
+ * out[T, n_out] (fp32) = x[T, in] (fp16) . w[n_out, in]^T (fp16) + bias[n_out] (fp32, may be NULL). */
+int pimhip_input_projection(void* out, const void* x, const void* w, const void* bias, int64_t seq_len,
+                            int64_t in_w, int64_t n_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PIMHIP_H_ */

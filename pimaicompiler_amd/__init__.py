@@ -1,0 +1,23 @@
+"""MI355X (gfx950) implementation of the PimAiCompiler runtime's memory-bound hot path.
+
+The compute lives in libpimhip.so (hand-written HIP kernels behind the C ABI of include/pimhip.h).
+`pimaicompiler_amd.ops` mirrors the reference runtime's operator interface for this path on torch tensors,
+which are used for device memory and streams only.
+"""
+from . import _lib  # noqa: F401
+from .ops import (  # noqa: F401
+    NNRuntimeException,
+    GemmType,
+    initialize,
+    deinitialize,
+    gemm_broadcast,
+    get_gemm_type,
+    custom_aten_addmm,
+    custom_aten_matmul,
+    aten_linear,
+    aten_lstm1,
+    aten_lstm2,
+    execute_gemv_group,
+    input_projection,
+    LstmPlan,
+)

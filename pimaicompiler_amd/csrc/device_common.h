@@ -1,0 +1,71 @@
+// Device-side helpers shared by the gfx950 kernels: fp16 vector types, fp32-accumulating
+// dot products on v_dot2_f32_f16, and 64-lane wavefront reductions built on DPP.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pimhip
+{
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+static constexpr int kWave = 64;
+
+// acc += sum_{i<8} w[i] * x[i], products and sum in fp32.
+__device__ __forceinline__ float dot8(const half8_t w, const half8_t x, float acc)
+{
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(w, w, 0, 1), __builtin_shufflevector(x, x, 0, 1), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(w, w, 2, 3), __builtin_shufflevector(x, x, 2, 3), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(w, w, 4, 5), __builtin_shufflevector(x, x, 4, 5), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(w, w, 6, 7), __builtin_shufflevector(x, x, 6, 7), acc, false);
+    return acc;
+}
+
+__device__ __forceinline__ float dot4(const half4_t w, const half4_t x, float acc)
+{
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(w, w, 0, 1), __builtin_shufflevector(x, x, 0, 1), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(w, w, 2, 3), __builtin_shufflevector(x, x, 2, 3), acc, false);
+    return acc;
+}
+
+// 16-byte streaming load of weight data that is read exactly once per launch.
+__device__ __forceinline__ half8_t load_stream(const half8_t* p) { return __builtin_nontemporal_load(p); }
+
+// DPP controls (gfx9 encoding).
+static constexpr int kDppQuadXor1 = 0xB1;     // quad_perm:[1,0,3,2]
+static constexpr int kDppQuadXor2 = 0x4E;     // quad_perm:[2,3,0,1]
+static constexpr int kDppRowHalfMirror = 0x141;
+static constexpr int kDppRowMirror = 0x140;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// Sum over the 64 lanes of a wavefront; every lane returns the total.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v += dpp_f32<kDppQuadXor1>(v);
+    v += dpp_f32<kDppQuadXor2>(v);
+    v += dpp_f32<kDppRowHalfMirror>(v);
+    v += dpp_f32<kDppRowMirror>(v);
+    v += __shfl_xor(v, 16, kWave);
+    v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float sigmoid_f32(float v) { return 1.0f / (1.0f + __expf(-v)); }
+
+__device__ __forceinline__ float tanh_f32(float v)
+{
+    // tanh(v) = 1 - 2 / (exp(2v) + 1); exact limits at +-inf, no cancellation near 0 beyond 1 ulp of 1.
+    const float e = __expf(2.0f * v);
+    return 1.0f - 2.0f / (e + 1.0f);
+}
+
+}  // namespace pimhip

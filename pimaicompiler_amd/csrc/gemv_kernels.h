@@ -1,0 +1,331 @@
+// fp16 batch-1 GEMV kernels for gfx950 (fp16 storage, fp32 accumulation, one rounding at the store).
+//
+// Two weight orders exist on this path, named after the operand order of the product:
+//   MV ("W_X_I"): y[out] = W[out,in] . x[in]   -- weight rows contiguous along the reduction
+//   VM ("I_X_W"): y[out] = x[in] . A[in,out]   -- weight rows contiguous along the outputs
+// plus VV, the dot product of two vectors.  Every kernel takes the fused epilogue
+// y = act(acc + bias) that the reference's addmv kernels define
+// (runtime/include/executor/op_executor/custom_ops.h:216-381: bias added after the alpha/beta
+// combination, ReLU applied last).
+//
+// All of them are HBM-bound: each weight element is read from memory exactly once per launch
+// through 16-byte non-temporal loads, x stays cache resident, and the only cross-lane traffic is
+// the final reduction.
+#pragma once
+
+#include "device_common.h"
+
+namespace pimhip
+{
+// ---------------------------------------------------------------------------------------------
+// MV order, vector path.  Requirements checked by the launcher: K % 8 == 0, ldw % 8 == 0,
+// W / x 16-byte aligned.
+//
+// A block holds WAVES wavefronts.  KS consecutive wavefronts share one group of R rows and split
+// the reduction dimension between them in an interleaved fashion (wave ks takes 16-byte chunks
+// ks*64 + lane, then strides by 64*KS), so one block covers (WAVES / KS) * R rows.  Each lane
+// keeps U chunks per row in flight: R*U independent 16-byte weight loads per lane per iteration.
+// ---------------------------------------------------------------------------------------------
+template <int R, int U, int WAVES, int KS>
+__device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, const half_t* __restrict__ x,
+                                                 const half_t* __restrict__ bias, half_t* __restrict__ y, int N,
+                                                 int K, long ldw, int relu, int block)
+{
+    static_assert(WAVES % KS == 0, "KS must divide WAVES");
+    constexpr int RG = WAVES / KS;  // row groups per block
+    __shared__ float red[WAVES][R];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int rg = wave / KS;
+    const int ks = wave % KS;
+    const long row0 = ((long)block * RG + rg) * R;
+
+    float acc[R];
+    const half8_t* wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        acc[r] = 0.0f;
+        long row = row0 + r;
+        if (row > N - 1) row = N - 1;  // out-of-range rows re-read the last row and are never stored
+        wrow[r] = reinterpret_cast<const half8_t*>(W + row * ldw);
+    }
+    const half8_t* xv = reinterpret_cast<const half8_t*>(x);
+    const int nchunks = K >> 3;
+    constexpr int STEP = 64 * KS;
+
+    int c = ks * 64 + lane;
+    // Main loop: U chunks per row in flight, all of them in range.
+    for (; c + (U - 1) * STEP < nchunks; c += U * STEP) {
+        half8_t xr[U];
+        half8_t wr[R][U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) wr[r][u] = load_stream(wrow[r] + c + u * STEP);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) xr[u] = xv[c + u * STEP];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = dot8(wr[r][u], xr[u], acc[r]);
+        }
+    }
+    // Tail: one chunk per row at a time.
+    for (; c < nchunks; c += STEP) {
+        half8_t wr[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) wr[r] = load_stream(wrow[r] + c);
+        const half8_t xr = xv[c];
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = dot8(wr[r], xr, acc[r]);
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+
+    if (KS > 1) {
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) red[wave][r] = acc[r];
+        }
+        __syncthreads();
+        if (ks == 0 && lane < R) {
+            float v = 0.0f;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) v += red[rg * KS + s][lane];
+            const long row = row0 + lane;
+            if (row < N) {
+                if (bias) v += (float)bias[row];
+                if (relu) v = fmaxf(v, 0.0f);
+                y[row] = (half_t)v;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const long row = row0 + r;
+            if (lane == r && row < N) {
+                float v = acc[r];
+                if (bias) v += (float)bias[row];
+                if (relu) v = fmaxf(v, 0.0f);
+                y[row] = (half_t)v;
+            }
+        }
+    }
+}
+
+template <int R, int U, int WAVES, int KS>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_kernel(const half_t* __restrict__ W,
+                                                                 const half_t* __restrict__ x,
+                                                                 const half_t* __restrict__ bias,
+                                                                 half_t* __restrict__ y, int N, int K, long ldw,
+                                                                 int relu)
+{
+    gemv_mv_f16_body<R, U, WAVES, KS>(W, x, bias, y, N, K, ldw, relu, blockIdx.x);
+}
+
+// Several independent MV GEMVs in one launch (sibling projections that the reference issues on separate
+// streams, runtime/source/executor/op_executor/stream_ops_executor.cpp:36-47).  Blocks
+// [block_begin[i], block_begin[i+1]) work on problem i.
+static constexpr int kGemvGroupMax = 32;
+struct GemvGroupArgs {
+    const half_t* W[kGemvGroupMax];
+    const half_t* x[kGemvGroupMax];
+    const half_t* bias[kGemvGroupMax];
+    half_t* y[kGemvGroupMax];
+    int N[kGemvGroupMax];
+    int K[kGemvGroupMax];
+    int relu[kGemvGroupMax];
+    int block_begin[kGemvGroupMax + 1];
+    int count;
+};
+
+template <int R, int U, int WAVES, int KS>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_group_kernel(GemvGroupArgs g)
+{
+    int i = 0;
+    while (i + 1 < g.count && (int)blockIdx.x >= g.block_begin[i + 1]) ++i;
+    gemv_mv_f16_body<R, U, WAVES, KS>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i],
+                                      (int)blockIdx.x - g.block_begin[i]);
+}
+
+// MV order, any K / leading dimension / alignment: one wavefront per row, 2-byte loads.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_generic_kernel(const half_t* __restrict__ W,
+                                                                         const half_t* __restrict__ x,
+                                                                         const half_t* __restrict__ bias,
+                                                                         half_t* __restrict__ y, int N, int K,
+                                                                         long ldw, int relu)
+{
+    const int lane = threadIdx.x & 63;
+    const long row = (long)blockIdx.x * WAVES + (threadIdx.x >> 6);
+    if (row >= N) return;
+    const half_t* w = W + row * ldw;
+    float acc = 0.0f;
+    for (int k = lane; k < K; k += 64) acc = fmaf((float)w[k], (float)x[k], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) {
+        if (bias) acc += (float)bias[row];
+        if (relu) acc = fmaxf(acc, 0.0f);
+        y[row] = (half_t)acc;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// VM order, vector path.  Requirements: N % 8 == 0, lda % 8 == 0, A 16-byte aligned.
+//
+// A block owns 512 adjacent outputs (8 per lane, one 16-byte load per weight row) and a slice
+// [k_begin, k_end) of the reduction; its WAVES wavefronts interleave over the rows of the slice.
+// gridDim.y slices cover K.  With one slice the block finishes the outputs itself; with several,
+// each block writes its 512 partial sums (fp32) to `partial[slice][N]` and takes a ticket from
+// `tickets[blockIdx.x]`; the block that draws the last ticket adds the slices in slice order (so
+// the result does not depend on which block finishes last), applies the epilogue and re-arms the
+// ticket counter for the next launch.
+// ---------------------------------------------------------------------------------------------
+template <int WAVES, int U>
+__global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* __restrict__ x,
+                                                                 const half_t* __restrict__ A,
+                                                                 const half_t* __restrict__ bias,
+                                                                 half_t* __restrict__ y, int K, int N, long lda,
+                                                                 int relu, int k_per_slice,
+                                                                 float* __restrict__ partial,
+                                                                 unsigned int* __restrict__ tickets)
+{
+    __shared__ float red[WAVES][8][64];
+    __shared__ unsigned int s_ticket;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const long col0 = ((long)blockIdx.x * 64 + lane) * 8;
+    const bool col_ok = col0 < N;
+    const int k_begin = blockIdx.y * k_per_slice;
+    const int k_end = min(K, k_begin + k_per_slice);
+
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+
+    if (col_ok) {
+        const half_t* a = A + col0;
+        int k = k_begin + wave;
+        for (; k + (U - 1) * WAVES < k_end; k += U * WAVES) {
+            half8_t ar[U];
+            float xr[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                ar[u] = load_stream(reinterpret_cast<const half8_t*>(a + (long)(k + u * WAVES) * lda));
+#pragma unroll
+            for (int u = 0; u < U; ++u) xr[u] = (float)x[k + u * WAVES];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] = fmaf((float)ar[u][j], xr[u], acc[j]);
+            }
+        }
+        for (; k < k_end; k += WAVES) {
+            const half8_t ar = load_stream(reinterpret_cast<const half8_t*>(a + (long)k * lda));
+            const float xr = (float)x[k];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = fmaf((float)ar[j], xr, acc[j]);
+        }
+    }
+
+    // Combine the WAVES partial sums of each column in LDS; wave 0 ends up with the block's result.
+#pragma unroll
+    for (int j = 0; j < 8; ++j) red[wave][j][lane] = acc[j];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float v = red[0][j][lane];
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) v += red[w][j][lane];
+            acc[j] = v;
+        }
+    }
+
+    const int nslices = gridDim.y;
+    if (nslices == 1) {
+        if (wave == 0 && col_ok) {
+            half8_t out;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float v = acc[j];
+                if (bias) v += (float)bias[col0 + j];
+                if (relu) v = fmaxf(v, 0.0f);
+                out[j] = (half_t)v;
+            }
+            *reinterpret_cast<half8_t*>(y + col0) = out;
+        }
+        return;
+    }
+
+    if (wave == 0 && col_ok) {
+        float* p = partial + (long)blockIdx.y * N + col0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) __hip_atomic_store(p + j, acc[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        s_ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (s_ticket != (unsigned int)(nslices - 1)) return;
+
+    __threadfence();
+    if (wave == 0 && col_ok) {
+        half8_t out;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float v = 0.0f;
+            for (int s = 0; s < nslices; ++s)
+                v += __hip_atomic_load(partial + (long)s * N + col0 + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (bias) v += (float)bias[col0 + j];
+            if (relu) v = fmaxf(v, 0.0f);
+            out[j] = (half_t)v;
+        }
+        *reinterpret_cast<half8_t*>(y + col0) = out;
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// VM order, any N / leading dimension / alignment: one lane per output column, 2-byte loads.
+__global__ __launch_bounds__(256) void gemv_vm_f16_generic_kernel(const half_t* __restrict__ x,
+                                                                  const half_t* __restrict__ A,
+                                                                  const half_t* __restrict__ bias,
+                                                                  half_t* __restrict__ y, int K, int N, long lda,
+                                                                  int relu)
+{
+    const long col = (long)blockIdx.x * 256 + threadIdx.x;
+    if (col >= N) return;
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) acc = fmaf((float)A[(long)k * lda + col], (float)x[k], acc);
+    if (bias) acc += (float)bias[col];
+    if (relu) acc = fmaxf(acc, 0.0f);
+    y[col] = (half_t)acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// VV: y[0] = sum_k a[k] * b[k].  One block of 1024 lanes; any K and alignment.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void dot_f16_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,
+                                                       half_t* __restrict__ y, long K)
+{
+    __shared__ float red[16];
+    float acc = 0.0f;
+    for (long k = threadIdx.x; k < K; k += 1024) acc = fmaf((float)a[k], (float)b[k], acc);
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) v += red[w];
+        y[0] = (half_t)v;
+    }
+}
+
+}  // namespace pimhip

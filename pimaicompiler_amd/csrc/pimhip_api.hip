@@ -1,0 +1,679 @@
+// C ABI of the gfx950 hot path (declared in include/pimhip.h): argument checking, kernel selection and
+// launches.  No torch types, no library GEMM or RNN calls: every kernel launched here is in this directory.
+#include "../../include/pimhip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "gemv_kernels.h"
+#include "lstm_kernels.h"
+#include "shape_logic.h"
+#include "xproj_kernels.h"
+
+using namespace pimhip;
+
+namespace
+{
+thread_local std::string g_last_error;
+
+int fail(int status, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return status;
+}
+
+#define PIMHIP_HIP_CHECK(expr)                                                                             \
+    do {                                                                                                   \
+        hipError_t e_ = (expr);                                                                            \
+        if (e_ != hipSuccess) return fail(PIMHIP_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- per-device state --------------------------------------------------------------------------
+struct SplitWorkspace {
+    float* partial = nullptr;        // [slices][N] fp32 partial sums of the VM kernel
+    size_t partial_elems = 0;
+    unsigned int* tickets = nullptr; // one arrival counter per 512-column block, zero between launches
+    size_t ticket_count = 0;
+};
+
+struct DeviceState {
+    bool initialized = false;
+    int num_cus = 0;
+    std::map<hipStream_t, SplitWorkspace> workspaces;  // one per stream: sibling GEMVs on different streams must not share
+};
+
+std::mutex g_mutex;
+std::map<int, DeviceState> g_devices;
+
+int current_device_state(DeviceState** out)
+{
+    int dev = -1;
+    PIMHIP_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_mutex);
+    auto it = g_devices.find(dev);
+    if (it == g_devices.end() || !it->second.initialized)
+        return fail(PIMHIP_ERR_NOT_INITIALIZED, "device %d: pimhip_initialize has not been called", dev);
+    *out = &it->second;
+    return PIMHIP_OK;
+}
+
+int get_split_workspace(DeviceState* st, hipStream_t stream, size_t partial_elems, size_t ticket_count,
+                        SplitWorkspace** out)
+{
+    std::lock_guard<std::mutex> lock(g_mutex);
+    SplitWorkspace& ws = st->workspaces[stream];
+    if (ws.partial_elems < partial_elems) {
+        // Work already queued on this stream may still use the old buffer.
+        PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
+        if (ws.partial) PIMHIP_HIP_CHECK(hipFree(ws.partial));
+        ws.partial = nullptr;
+        ws.partial_elems = 0;
+        PIMHIP_HIP_CHECK(hipMalloc(&ws.partial, partial_elems * sizeof(float)));
+        ws.partial_elems = partial_elems;
+    }
+    if (ws.ticket_count < ticket_count) {
+        PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
+        if (ws.tickets) PIMHIP_HIP_CHECK(hipFree(ws.tickets));
+        ws.tickets = nullptr;
+        ws.ticket_count = 0;
+        PIMHIP_HIP_CHECK(hipMalloc(&ws.tickets, ticket_count * sizeof(unsigned int)));
+        PIMHIP_HIP_CHECK(hipMemsetAsync(ws.tickets, 0, ticket_count * sizeof(unsigned int), stream));
+        ws.ticket_count = ticket_count;
+    }
+    *out = &ws;
+    return PIMHIP_OK;
+}
+
+// ---- GEMV launch selection ---------------------------------------------------------------------
+template <int R, int U, int WAVES, int KS>
+void launch_mv(const half_t* W, const half_t* x, const half_t* b, half_t* y, int N, int K, long ldw, int relu,
+               hipStream_t s)
+{
+    constexpr int rows_per_block = (WAVES / KS) * R;
+    const int grid = (N + rows_per_block - 1) / rows_per_block;
+    gemv_mv_f16_kernel<R, U, WAVES, KS><<<grid, WAVES * 64, 0, s>>>(W, x, b, y, N, K, ldw, relu);
+}
+
+int gemv_mv(const half_t* W, const half_t* x, const half_t* bias, half_t* y, int64_t N, int64_t K, int64_t ldw,
+            int relu, hipStream_t s)
+{
+    const bool vec_ok = (K % 8 == 0) && (ldw % 8 == 0) && aligned16(W) && aligned16(x);
+    if (!vec_ok) {
+        const int grid = (int)((N + 3) / 4);
+        gemv_mv_f16_generic_kernel<4><<<grid, 256, 0, s>>>(W, x, bias, y, (int)N, (int)K, (long)ldw, relu);
+        return PIMHIP_OK;
+    }
+    // Measured on MI355X over the (out, in) shapes of the GEMV sweep: long rows want the reduction split
+    // over the four wavefronts of a block (more rows of the matrix open at once per CU would thrash DRAM
+    // pages), short rows want two rows per wavefront.  Few rows: one row per block so that enough blocks exist.
+    if (N < 1024) {
+        if (K >= 2048)
+            launch_mv<1, 4, 4, 4>(W, x, bias, y, (int)N, (int)K, (long)ldw, relu, s);
+        else
+            launch_mv<1, 2, 4, 4>(W, x, bias, y, (int)N, (int)K, (long)ldw, relu, s);
+    } else if (K >= 4096) {
+        launch_mv<2, 4, 4, 4>(W, x, bias, y, (int)N, (int)K, (long)ldw, relu, s);
+    } else {
+        launch_mv<2, 2, 4, 2>(W, x, bias, y, (int)N, (int)K, (long)ldw, relu, s);
+    }
+    return PIMHIP_OK;
+}
+
+int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bias, half_t* y, int64_t K, int64_t N,
+            int64_t lda, int relu, hipStream_t s)
+{
+    const bool vec_ok = (N % 8 == 0) && (lda % 8 == 0) && aligned16(A) && aligned16(y);
+    if (!vec_ok) {
+        const int grid = (int)((N + 255) / 256);
+        gemv_vm_f16_generic_kernel<<<grid, 256, 0, s>>>(x, A, bias, y, (int)K, (int)N, (long)lda, relu);
+        return PIMHIP_OK;
+    }
+    constexpr int WAVES = 4;
+    const int col_blocks = (int)((N + 511) / 512);
+    // Enough slices of K that about 4 blocks per CU exist, each slice at least 32 rows deep.
+    int slices = (4 * st->num_cus + col_blocks - 1) / col_blocks;
+    const int max_slices = (int)((K + 31) / 32);
+    if (slices > max_slices) slices = max_slices;
+    if (slices < 1) slices = 1;
+    int k_per_slice = (int)((K + slices - 1) / slices);
+    k_per_slice = (k_per_slice + WAVES - 1) / WAVES * WAVES;
+    slices = (int)((K + k_per_slice - 1) / k_per_slice);
+    SplitWorkspace* ws = nullptr;
+    float* partial = nullptr;
+    unsigned int* tickets = nullptr;
+    if (slices > 1) {
+        int rc = get_split_workspace(st, s, (size_t)slices * (size_t)N, (size_t)col_blocks, &ws);
+        if (rc != PIMHIP_OK) return rc;
+        partial = ws->partial;
+        tickets = ws->tickets;
+    }
+    dim3 grid(col_blocks, slices);
+    gemv_vm_f16_kernel<WAVES, 4><<<grid, WAVES * 64, 0, s>>>(x, A, bias, y, (int)K, (int)N, (long)lda, relu,
+                                                             k_per_slice, partial, tickets);
+    return PIMHIP_OK;
+}
+
+}  // namespace
+
+// ================================================================================================
+// init / teardown
+// ================================================================================================
+struct PimHipLstmPlan;
+namespace
+{
+std::vector<PimHipLstmPlan*> g_plans;
+int destroy_plan_locked(PimHipLstmPlan* plan);
+}  // namespace
+
+extern "C" int pimhip_initialize(int device)
+{
+    int count = 0;
+    PIMHIP_HIP_CHECK(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "device %d out of range [0, %d)", device, count);
+    hipDeviceProp_t prop;
+    PIMHIP_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+    PIMHIP_HIP_CHECK(hipSetDevice(device));
+    std::lock_guard<std::mutex> lock(g_mutex);
+    DeviceState& st = g_devices[device];
+    st.initialized = true;
+    st.num_cus = prop.multiProcessorCount;
+    return PIMHIP_OK;
+}
+
+extern "C" const char* pimhip_last_error(void) { return g_last_error.c_str(); }
+
+// ================================================================================================
+// shape logic
+// ================================================================================================
+extern "C" int pimhip_gemm_broadcast(int64_t* shape1, int* rank1, int64_t* shape2, int* rank2)
+{
+    if (!shape1 || !shape2 || !rank1 || !rank2) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "null argument");
+    if (*rank1 < 1 || *rank1 > 4 || *rank2 < 1 || *rank2 > 4)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "ranks must be in [1, 4], got %d and %d", *rank1, *rank2);
+    std::vector<int64_t> s1(shape1, shape1 + *rank1), s2(shape2, shape2 + *rank2);
+    if (!gemm_broadcast(s1, s2)) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "rank difference above 3");
+    if (s1.size() > 4 || s2.size() > 4) return fail(PIMHIP_ERR_UNSUPPORTED, "broadcast produced a rank above 4");
+    *rank1 = (int)s1.size();
+    *rank2 = (int)s2.size();
+    for (size_t i = 0; i < s1.size(); ++i) shape1[i] = s1[i];
+    for (size_t i = 0; i < s2.size(); ++i) shape2[i] = s2[i];
+    if (s1.size() != 4 || s2.size() != 4)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "shapes stay at ranks %zu and %zu, not 4", s1.size(), s2.size());
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* other_shape4, int* gemm_type)
+{
+    if (!self_shape4 || !other_shape4 || !gemm_type) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "null argument");
+    *gemm_type = get_gemm_type(self_shape4, other_shape4);
+    return PIMHIP_OK;
+}
+
+// ================================================================================================
+// GEMV family
+// ================================================================================================
+extern "C" int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
+                                   int64_t out_w, int64_t ld_weight, int act, int order, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!out || !in || !weight) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "out, in and weight must be non-null");
+    if (in_w < 0 || out_w < 0 || in_w > INT32_MAX || out_w > INT32_MAX)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "in_w=%lld out_w=%lld out of range", (long long)in_w, (long long)out_w);
+    if (act != PIMHIP_ACT_NONE && act != PIMHIP_ACT_RELU) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "unknown activation %d", act);
+    if (order != PIMHIP_I_X_W && order != PIMHIP_W_X_I) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "unknown operand order %d", order);
+    if (out_w == 0) return PIMHIP_OK;
+    const int64_t dense = (order == PIMHIP_W_X_I) ? in_w : out_w;
+    if (ld_weight == 0) ld_weight = dense;
+    if (ld_weight < dense)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "ld_weight=%lld is below the row length %lld", (long long)ld_weight, (long long)dense);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int relu = act == PIMHIP_ACT_RELU;
+    if (order == PIMHIP_W_X_I)
+        rc = gemv_mv((const half_t*)weight, (const half_t*)in, (const half_t*)bias, (half_t*)out, out_w, in_w, ld_weight, relu, s);
+    else
+        rc = gemv_vm(st, (const half_t*)in, (const half_t*)weight, (const half_t*)bias, (half_t*)out, in_w, out_w, ld_weight, relu, s);
+    if (rc != PIMHIP_OK) return rc;
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_execute_dot(void* out, const void* a, const void* b, int64_t in_w, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!out || !a || !b) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "out, a and b must be non-null");
+    if (in_w < 0) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "in_w=%lld is negative", (long long)in_w);
+    dot_f16_kernel<<<1, 1024, 0, static_cast<hipStream_t>(stream)>>>((const half_t*)a, (const half_t*)b, (half_t*)out, (long)in_w);
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const void* const* ins,
+                                         const void* const* weights, const void* const* biases,
+                                         const int64_t* in_ws, const int64_t* out_ws, const int* acts, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (count < 0 || count > 64) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "count=%d not in [0, 64]", count);
+    if (count == 0) return PIMHIP_OK;
+    if (!outs || !ins || !weights || !in_ws || !out_ws) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "null array argument");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    constexpr int R = 2, U = 2, WAVES = 4, KS = 2;
+    constexpr int rows_per_block = (WAVES / KS) * R;
+    int done = 0;
+    while (done < count) {
+        GemvGroupArgs g;
+        memset(&g, 0, sizeof(g));
+        int n = 0, blocks = 0;
+        for (; done + n < count && n < kGemvGroupMax; ++n) {
+            const int i = done + n;
+            if (!outs[i] || !ins[i] || !weights[i]) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "entry %d has a null pointer", i);
+            if (in_ws[i] < 0 || out_ws[i] < 1 || in_ws[i] > INT32_MAX || out_ws[i] > INT32_MAX)
+                return fail(PIMHIP_ERR_INVALID_ARGUMENT, "entry %d: in_w=%lld out_w=%lld out of range", i, (long long)in_ws[i], (long long)out_ws[i]);
+            if (in_ws[i] % 8 != 0 || !aligned16(weights[i]) || !aligned16(ins[i]))
+                return fail(PIMHIP_ERR_UNSUPPORTED, "entry %d: grouped launch needs in_w %% 8 == 0 and 16-byte aligned in/weight", i);
+            const int a = acts ? acts[i] : PIMHIP_ACT_NONE;
+            if (a != PIMHIP_ACT_NONE && a != PIMHIP_ACT_RELU) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "entry %d: unknown activation %d", i, a);
+            g.W[n] = (const half_t*)weights[i];
+            g.x[n] = (const half_t*)ins[i];
+            g.bias[n] = biases ? (const half_t*)biases[i] : nullptr;
+            g.y[n] = (half_t*)outs[i];
+            g.N[n] = (int)out_ws[i];
+            g.K[n] = (int)in_ws[i];
+            g.relu[n] = a == PIMHIP_ACT_RELU;
+            g.block_begin[n] = blocks;
+            blocks += ((int)out_ws[i] + rows_per_block - 1) / rows_per_block;
+        }
+        g.block_begin[n] = blocks;
+        g.count = n;
+        gemv_mv_f16_group_kernel<R, U, WAVES, KS><<<blocks, WAVES * 64, 0, s>>>(g);
+        PIMHIP_HIP_CHECK(hipGetLastError());
+        done += n;
+    }
+    return PIMHIP_OK;
+}
+
+// ================================================================================================
+// input projection
+// ================================================================================================
+namespace
+{
+int launch_input_projection(float* out, const half_t* x, const half_t* w, const float* bias, int64_t T, int64_t K,
+                            int64_t N, hipStream_t s)
+{
+    if (T <= 0 || N <= 0) return PIMHIP_OK;
+    if (K % 8 != 0 || !aligned16(x) || !aligned16(w))
+        return fail(PIMHIP_ERR_UNSUPPORTED, "input projection needs in_w %% 8 == 0 (got %lld) and 16-byte aligned x and w", (long long)K);
+    if (T > INT32_MAX || K > INT32_MAX || N > INT32_MAX) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "dimension above 2^31-1");
+    // One block per 16 output columns; up to 64 * MT time steps per grid row.
+    if (T <= 64) {
+        dim3 grid((unsigned)((N + 15) / 16), 1);
+        input_projection_f16_kernel<1, 1><<<grid, 256, 0, s>>>(x, w, bias, out, (int)T, (int)K, (int)N);
+    } else if (T <= 128) {
+        dim3 grid((unsigned)((N + 15) / 16), 1);
+        input_projection_f16_kernel<2, 1><<<grid, 256, 0, s>>>(x, w, bias, out, (int)T, (int)K, (int)N);
+    } else {
+        dim3 grid((unsigned)((N + 15) / 16), (unsigned)((T + 255) / 256));
+        input_projection_f16_kernel<4, 1><<<grid, 256, 0, s>>>(x, w, bias, out, (int)T, (int)K, (int)N);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(PIMHIP_ERR_HIP, "input projection launch failed: %s", hipGetErrorString(e));
+    return PIMHIP_OK;
+}
+}  // namespace
+
+extern "C" int pimhip_input_projection(void* out, const void* x, const void* w, const void* bias, int64_t seq_len,
+                                       int64_t in_w, int64_t n_out, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!out || !x || !w) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "out, x and w must be non-null");
+    if (seq_len < 0 || in_w < 0 || n_out < 0) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "negative dimension");
+    return launch_input_projection((float*)out, (const half_t*)x, (const half_t*)w, (const float*)bias, seq_len, in_w,
+                                   n_out, static_cast<hipStream_t>(stream));
+}
+
+// ================================================================================================
+// LSTM
+// ================================================================================================
+struct PimHipLstmPlan {
+    int device = -1;
+    int num_cus = 0;
+    int has_biases = 0;
+    int num_layers = 0;
+    int num_dirs = 1;
+    int64_t input_size = 0;
+    int64_t hidden = 0;
+    int64_t max_seq_len = 0;
+    int mode = 0;
+    bool seq_kernel_ok = false;      // shape fits the persistent sequence kernel
+    unsigned int spin_limit = 1u << 22;
+    unsigned int tag_base = 0;
+
+    struct Cell {
+        const half_t* w_ih = nullptr;
+        const half_t* w_hh = nullptr;
+        const half_t* b_ih = nullptr;
+        const half_t* b_hh = nullptr;
+        float* bsum = nullptr;  // [4H] fp32, b_ih + b_hh (zeros when has_biases == 0)
+        int64_t in_w = 0;
+    };
+    std::vector<Cell> cells;          // index = layer * num_dirs + dir
+
+    float* bsum_all = nullptr;        // backing store of every Cell::bsum
+    float* xproj = nullptr;           // [num_dirs][max_seq_len][4H] fp32
+    half_t* ybuf[2] = {nullptr, nullptr};  // inter-layer sequences [max_seq_len][num_dirs * H]
+    float* c_state = nullptr;         // [num_dirs][H] fp32, per-step kernel's cell state
+    unsigned long long* hx = nullptr; // [num_dirs][2][NB][2] exchange words of the sequence kernel
+    unsigned int* abort_flag = nullptr;
+    unsigned int* abort_host = nullptr;  // pinned copy read by pimhip_lstm_plan_status
+    size_t seq_lds_bytes = 0;
+    int seq_blocks = 0;
+};
+
+namespace
+{
+int destroy_plan_locked(PimHipLstmPlan* plan)
+{
+    if (!plan) return PIMHIP_OK;
+    int prev = -1;
+    hipGetDevice(&prev);
+    hipSetDevice(plan->device);
+    hipDeviceSynchronize();
+    if (plan->bsum_all) hipFree(plan->bsum_all);
+    if (plan->xproj) hipFree(plan->xproj);
+    if (plan->ybuf[0]) hipFree(plan->ybuf[0]);
+    if (plan->ybuf[1]) hipFree(plan->ybuf[1]);
+    if (plan->c_state) hipFree(plan->c_state);
+    if (plan->hx) hipFree(plan->hx);
+    if (plan->abort_flag) hipFree(plan->abort_flag);
+    if (plan->abort_host) hipHostFree(plan->abort_host);
+    if (prev >= 0) hipSetDevice(prev);
+    for (size_t i = 0; i < g_plans.size(); ++i) {
+        if (g_plans[i] == plan) {
+            g_plans.erase(g_plans.begin() + i);
+            break;
+        }
+    }
+    delete plan;
+    return PIMHIP_OK;
+}
+}  // namespace
+
+extern "C" int pimhip_deinitialize(void)
+{
+    std::lock_guard<std::mutex> lock(g_mutex);
+    while (!g_plans.empty()) destroy_plan_locked(g_plans.back());
+    int prev = -1;
+    hipGetDevice(&prev);
+    for (auto& kv : g_devices) {
+        if (!kv.second.initialized) continue;
+        hipSetDevice(kv.first);
+        hipDeviceSynchronize();
+        for (auto& w : kv.second.workspaces) {
+            if (w.second.partial) hipFree(w.second.partial);
+            if (w.second.tickets) hipFree(w.second.tickets);
+        }
+        kv.second.workspaces.clear();
+        kv.second.initialized = false;
+    }
+    g_devices.clear();
+    if (prev >= 0) hipSetDevice(prev);
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* const* params, int n_params,
+                                       int has_biases, int num_layers, int bidirectional, int64_t input_size,
+                                       int64_t hidden_size, int64_t max_seq_len, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!plan_out || !params) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan and params must be non-null");
+    *plan_out = nullptr;
+    if (num_layers < 1 || input_size < 1 || hidden_size < 1 || max_seq_len < 1)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "num_layers, input_size, hidden_size and max_seq_len must be positive");
+    const int D = bidirectional ? 2 : 1;
+    const int per_cell = has_biases ? 4 : 2;
+    if (n_params != num_layers * D * per_cell)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "expected %d parameter tensors (layers=%d dirs=%d biases=%d), got %d",
+                    num_layers * D * per_cell, num_layers, D, has_biases ? 1 : 0, n_params);
+    for (int i = 0; i < n_params; ++i)
+        if (!params[i]) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "params[%d] is null", i);
+    const int64_t H = hidden_size;
+    if (H % 8 != 0 || input_size % 8 != 0)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "hidden_size (%lld) and input_size (%lld) must be multiples of 8", (long long)H, (long long)input_size);
+    if (4 * H > INT32_MAX || input_size > INT32_MAX || max_seq_len > INT32_MAX || D * H > INT32_MAX)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "dimension above 2^31-1");
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    PimHipLstmPlan* plan = new PimHipLstmPlan();
+    PIMHIP_HIP_CHECK(hipGetDevice(&plan->device));
+    plan->num_cus = st->num_cus;
+    plan->has_biases = has_biases ? 1 : 0;
+    plan->num_layers = num_layers;
+    plan->num_dirs = D;
+    plan->input_size = input_size;
+    plan->hidden = H;
+    plan->max_seq_len = max_seq_len;
+    plan->cells.resize((size_t)num_layers * D);
+
+    auto cleanup_fail = [&](int status) {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        destroy_plan_locked(plan);
+        return status;
+    };
+#define PLAN_HIP_CHECK(expr)                                                                                    \
+    do {                                                                                                        \
+        hipError_t e_ = (expr);                                                                                 \
+        if (e_ != hipSuccess) return cleanup_fail(fail(PIMHIP_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_))); \
+    } while (0)
+
+    PLAN_HIP_CHECK(hipMalloc(&plan->bsum_all, sizeof(float) * 4 * H * plan->cells.size()));
+    for (int l = 0; l < num_layers; ++l) {
+        for (int d = 0; d < D; ++d) {
+            const int ci = l * D + d;
+            PimHipLstmPlan::Cell& c = plan->cells[ci];
+            const void* const* p = params + (size_t)ci * per_cell;
+            c.w_ih = (const half_t*)p[0];
+            c.w_hh = (const half_t*)p[1];
+            c.b_ih = has_biases ? (const half_t*)p[2] : nullptr;
+            c.b_hh = has_biases ? (const half_t*)p[3] : nullptr;
+            c.in_w = (l == 0) ? input_size : D * H;
+            c.bsum = plan->bsum_all + (size_t)ci * 4 * H;
+            if (!aligned16(c.w_ih) || !aligned16(c.w_hh))
+                return cleanup_fail(fail(PIMHIP_ERR_UNSUPPORTED, "weights of layer %d direction %d are not 16-byte aligned", l, d));
+            lstm_bias_sum_kernel<<<(unsigned)((4 * H + 255) / 256), 256, 0, s>>>(c.b_ih, c.b_hh, c.bsum, (int)(4 * H));
+        }
+    }
+    PLAN_HIP_CHECK(hipGetLastError());
+    PLAN_HIP_CHECK(hipMalloc(&plan->xproj, sizeof(float) * (size_t)D * max_seq_len * 4 * H));
+    if (num_layers > 1) {
+        PLAN_HIP_CHECK(hipMalloc(&plan->ybuf[0], sizeof(half_t) * (size_t)max_seq_len * D * H));
+        if (num_layers > 2) PLAN_HIP_CHECK(hipMalloc(&plan->ybuf[1], sizeof(half_t) * (size_t)max_seq_len * D * H));
+    }
+    PLAN_HIP_CHECK(hipMalloc(&plan->c_state, sizeof(float) * (size_t)D * H));
+    PLAN_HIP_CHECK(hipMalloc(&plan->abort_flag, sizeof(unsigned int)));
+    PLAN_HIP_CHECK(hipMemsetAsync(plan->abort_flag, 0, sizeof(unsigned int), s));
+    PLAN_HIP_CHECK(hipHostMalloc(&plan->abort_host, sizeof(unsigned int), hipHostMallocDefault));
+    *plan->abort_host = 0;
+
+    // Persistent sequence kernel: 16 rows of W_hh per block in LDS, one block per 4 hidden units, all blocks
+    // resident at once.
+    plan->seq_blocks = (int)((H + kSeqUnits - 1) / kSeqUnits);
+    plan->seq_lds_bytes = (size_t)kSeqRows * H * sizeof(half_t) + 2 * 256 * sizeof(float);
+    plan->seq_kernel_ok = false;
+    if (H <= kSeqMaxH && plan->seq_lds_bytes <= 64 * 1024) {
+        int per_cu = 0;
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_seq_f16_kernel, 256, plan->seq_lds_bytes));
+        plan->seq_kernel_ok = (int64_t)per_cu * plan->num_cus >= plan->seq_blocks;
+    }
+    if (plan->seq_kernel_ok) {
+        const size_t words = (size_t)D * 2 * plan->seq_blocks * 2;
+        PLAN_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned long long)));
+        PLAN_HIP_CHECK(hipMemsetAsync(plan->hx, 0, words * sizeof(unsigned long long), s));
+    }
+    PLAN_HIP_CHECK(hipStreamSynchronize(s));
+#undef PLAN_HIP_CHECK
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        g_plans.push_back(plan);
+    }
+    *plan_out = plan;
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan)
+{
+    if (!plan) return PIMHIP_OK;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    bool known = false;
+    for (PimHipLstmPlan* p : g_plans) known = known || (p == plan);
+    if (!known) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "unknown or already destroyed plan");
+    return destroy_plan_locked(plan);
+}
+
+extern "C" int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode)
+{
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    if (mode < 0 || mode > 2) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "mode %d not in {0, 1, 2}", mode);
+    if (mode == 2 && !plan->seq_kernel_ok)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "hidden_size %lld does not fit the persistent sequence kernel", (long long)plan->hidden);
+    plan->mode = mode;
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limit)
+{
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    plan->spin_limit = spin_limit;
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_lstm_plan_status(PimHipLstmPlan* plan)
+{
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    if (*plan->abort_host != 0u) return fail(PIMHIP_ERR_TIMEOUT, "a bounded wait of the persistent LSTM kernel gave up");
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y,
+                                   void* hn, void* cn, int64_t seq_len, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    int dev = -1;
+    PIMHIP_HIP_CHECK(hipGetDevice(&dev));
+    if (dev != plan->device) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan belongs to device %d, current device is %d", plan->device, dev);
+    if (!x || !h0 || !c0 || !y || !hn || !cn) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "x, h0, c0, y, hn and cn must be non-null");
+    if (seq_len < 0 || seq_len > plan->max_seq_len)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "seq_len=%lld not in [0, max_seq_len=%lld]", (long long)seq_len, (long long)plan->max_seq_len);
+    if (!aligned16(x) || !aligned16(h0) || !aligned16(y))
+        return fail(PIMHIP_ERR_UNSUPPORTED, "x, h0 and y must be 16-byte aligned");
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t H = plan->hidden;
+    const int D = plan->num_dirs;
+    const int L = plan->num_layers;
+    const int64_t T = seq_len;
+    const half_t* h0p = (const half_t*)h0;
+    const half_t* c0p = (const half_t*)c0;
+    half_t* hnp = (half_t*)hn;
+    half_t* cnp = (half_t*)cn;
+
+    if (T == 0) {
+        // No step: the state passes through unchanged.
+        PIMHIP_HIP_CHECK(hipMemcpyAsync(hn, h0, sizeof(half_t) * (size_t)L * D * H, hipMemcpyDeviceToDevice, s));
+        PIMHIP_HIP_CHECK(hipMemcpyAsync(cn, c0, sizeof(half_t) * (size_t)L * D * H, hipMemcpyDeviceToDevice, s));
+        return PIMHIP_OK;
+    }
+
+    const bool use_seq = (plan->mode == 2) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2);
+    if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
+    // seq_len == 1: fuse the input projection into the step (one launch per layer and direction).
+    const bool fuse_xproj = !use_seq && T == 1;
+
+    const half_t* layer_in = (const half_t*)x;
+    for (int l = 0; l < L; ++l) {
+        half_t* layer_out = (l == L - 1) ? (half_t*)y : plan->ybuf[l & 1];
+        const int64_t in_w = plan->cells[(size_t)l * D].in_w;
+        for (int d = 0; d < D; ++d) {
+            const int ci = l * D + d;
+            const PimHipLstmPlan::Cell& c = plan->cells[ci];
+            float* xp = plan->xproj + (size_t)d * plan->max_seq_len * 4 * H;
+            half_t* yd = layer_out + (size_t)d * H;
+            const long y_stride = (long)D * H;
+            const half_t* h0c = h0p + (size_t)ci * H;
+            const half_t* c0c = c0p + (size_t)ci * H;
+            half_t* hnc = hnp + (size_t)ci * H;
+            half_t* cnc = cnp + (size_t)ci * H;
+
+            if (!fuse_xproj) {
+                rc = launch_input_projection(xp, layer_in, c.w_ih, c.bsum, T, in_w, 4 * H, s);
+                if (rc != PIMHIP_OK) return rc;
+            }
+            if (use_seq) {
+                LstmSeqArgs a;
+                a.w_hh = c.w_hh;
+                a.xproj = xp;
+                a.h0 = h0c;
+                a.c0 = c0c;
+                a.y = yd;
+                a.hn = hnc;
+                a.cn = cnc;
+                a.hx = plan->hx + (size_t)d * 2 * plan->seq_blocks * 2;
+                a.abort_flag = plan->abort_flag;
+                a.y_stride = y_stride;
+                a.H = (int)H;
+                a.T = (int)T;
+                a.reverse = d;
+                a.tag_base = plan->tag_base;
+                a.spin_limit = plan->spin_limit;
+                plan->tag_base += (unsigned int)T;
+                lstm_seq_f16_kernel<<<plan->seq_blocks, 256, plan->seq_lds_bytes, s>>>(a);
+            } else {
+                float* cst = plan->c_state + (size_t)d * H;
+                const unsigned grid = (unsigned)((H + 3) / 4);
+                for (int64_t step = 0; step < T; ++step) {
+                    const int64_t t = d ? (T - 1 - step) : step;
+                    const int64_t tp = d ? (t + 1) : (t - 1);
+                    const half_t* h_prev = (step == 0) ? h0c : (yd + tp * y_stride);
+                    const bool last = step == T - 1;
+                    lstm_step_f16_kernel<4><<<grid, 256, 0, s>>>(
+                        c.w_ih, c.w_hh, c.bsum, fuse_xproj ? nullptr : (xp + t * 4 * H), layer_in + t * in_w, h_prev,
+                        (step == 0) ? c0c : nullptr, cst, yd + t * y_stride, last ? hnc : nullptr, last ? cnc : nullptr,
+                        (int)in_w, (int)H);
+                }
+            }
+            PIMHIP_HIP_CHECK(hipGetLastError());
+        }
+        layer_in = layer_out;
+    }
+    if (use_seq)
+        PIMHIP_HIP_CHECK(hipMemcpyAsync(plan->abort_host, plan->abort_flag, sizeof(unsigned int), hipMemcpyDeviceToHost, s));
+    return PIMHIP_OK;
+}

@@ -1,0 +1,467 @@
+"""Host-side mirror of the reference runtime's operator interface for the GEMV / LSTM hot path.
+
+Function names, argument meaning and dispatch rules follow the reference's C++ operators
+(paths relative to the reference tree):
+
+    custom_aten_addmm   customAtenAddmm   runtime/source/executor/op_executor/aten_ops.cpp:609-758
+    custom_aten_matmul  customAtenMatmul  runtime/source/executor/op_executor/aten_ops.cpp:760-932
+    aten_linear         atenLinear        runtime/source/executor/op_executor/aten_ops.cpp:304-307
+    aten_lstm1 / 2      atenLstm1 / 2     runtime/source/executor/op_executor/aten_ops.cpp:328-344
+    gemm_broadcast      gemmBroadcast     runtime/source/executor/utils/utils.cpp:293-371
+    get_gemm_type       getGemmType       runtime/source/executor/utils/utils.cpp:373-396
+
+torch tensors carry device memory and the stream; every product that is a batch-1 GEMV, a dot product or an
+LSTM runs in libpimhip.so.  True matrix-matrix products take the same LibTorch passthrough the reference takes
+(atenAddmm / atenMatmul, aten_ops.cpp:47-51,362).  Errors are raised as NNRuntimeException
+(runtime/include/executor/utils/utils.h:166-176) instead of being ignored.
+"""
+import ctypes
+import enum
+import weakref
+
+import torch
+
+from . import _lib as L
+
+
+class NNRuntimeException(RuntimeError):
+    """Counterpart of nn_compiler::runtime::utils::NNRuntimeException."""
+
+
+class GemmType(enum.IntEnum):
+    """GEMM_TYPE of runtime/include/executor/utils/utils.h:30-36."""
+    UNKNOW = L.GEMM_UNKNOWN
+    VV = L.GEMM_VV
+    VM = L.GEMM_VM
+    MV = L.GEMM_MV
+    MM = L.GEMM_MM
+
+
+def _check(rc):
+    if rc != L.PIMHIP_OK:
+        msg = L.load().pimhip_last_error().decode("utf-8", "replace")
+        raise NNRuntimeException(f"pimhip error {rc}: {msg}")
+
+
+_initialized_devices = set()
+
+
+def initialize(device=None):
+    """PimInitialize counterpart (runtime/source/nn_runtime.cpp:32).  Needs a gfx950 GPU."""
+    lib = L.load()
+    if not torch.cuda.is_available():
+        raise NNRuntimeException("no HIP device is visible; this path has no CPU fallback")
+    if device is None:
+        device = torch.cuda.current_device()
+    device = torch.device("cuda", device).index if not isinstance(device, int) else device
+    with torch.cuda.device(device):
+        _check(lib.pimhip_initialize(device))
+    _initialized_devices.add(device)
+
+
+def deinitialize():
+    """PimDeinitialize counterpart (runtime/source/nn_runtime.cpp:85)."""
+    _plan_cache.clear()
+    _check(L.load().pimhip_deinitialize())
+    _initialized_devices.clear()
+
+
+def _ensure_init(t):
+    dev = t.device.index if t.device.index is not None else torch.cuda.current_device()
+    if dev not in _initialized_devices:
+        initialize(dev)
+    return dev
+
+
+def _stream_handle(stream):
+    """hipStream_t as an integer; None means torch's current stream (the null stream unless changed)."""
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, torch.cuda.Stream):
+        return stream.cuda_stream
+    return int(stream)
+
+
+def _require_half_cuda(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise NNRuntimeException("tensors of this path must live on the GPU (there is no CPU fallback)")
+        if t.dtype != torch.float16:
+            raise NNRuntimeException(f"fp16 tensors required, got {t.dtype}")
+
+
+# ---------------------------------------------------------------------------------------------------
+# shape logic
+# ---------------------------------------------------------------------------------------------------
+def gemm_broadcast(shape1, shape2):
+    """Returns the two shapes padded as gemmBroadcast pads them.  Raises if they do not end at rank 4."""
+    lib = L.load()
+    a = (ctypes.c_int64 * 4)(*list(shape1) + [0] * (4 - len(shape1)))
+    b = (ctypes.c_int64 * 4)(*list(shape2) + [0] * (4 - len(shape2)))
+    ra, rb = ctypes.c_int(len(shape1)), ctypes.c_int(len(shape2))
+    _check(lib.pimhip_gemm_broadcast(a, ctypes.byref(ra), b, ctypes.byref(rb)))
+    return list(a[:ra.value]), list(b[:rb.value])
+
+
+def get_gemm_type(self_shape, other_shape):
+    lib = L.load()
+    if len(self_shape) != 4 or len(other_shape) != 4:
+        raise NNRuntimeException("get_gemm_type takes two rank-4 shapes")
+    a = (ctypes.c_int64 * 4)(*self_shape)
+    b = (ctypes.c_int64 * 4)(*other_shape)
+    out = ctypes.c_int(0)
+    _check(lib.pimhip_get_gemm_type(a, b, ctypes.byref(out)))
+    return GemmType(out.value)
+
+
+# ---------------------------------------------------------------------------------------------------
+# GEMV family
+# ---------------------------------------------------------------------------------------------------
+def _weight_view(w2d):
+    """(tensor, order_is_transposed): a 2-D weight usable without a copy, or a contiguous copy.
+
+    A [rows, cols] view whose memory is column-major with a dense pitch (a `.t()` of a row-major matrix, which
+    is what SwapAddmmInputs / SwapMatmulInputs leave behind, compiler/source/frontend/optimizer/
+    swap_addmm_inputs.cpp:45-97) is the other operand order on the same bytes, so the reference's
+    `.contiguous()` copy (aten_ops.cpp:630-632) is not needed.
+    """
+    if w2d.is_contiguous():
+        return w2d, False
+    if w2d.dim() == 2 and w2d.stride(0) == 1 and w2d.stride(1) >= w2d.size(0):
+        return w2d.t(), True
+    return w2d.contiguous(), False
+
+
+def _gemv(x, weight2d, bias, in_w, out_w, order, act, stream):
+    """Launches one GEMV.  weight2d is [in_w, out_w] for I_X_W and [out_w, in_w] for W_X_I."""
+    lib = L.load()
+    _ensure_init(weight2d)
+    w, flipped = _weight_view(weight2d)
+    if flipped:
+        order = L.PIMHIP_W_X_I if order == L.PIMHIP_I_X_W else L.PIMHIP_I_X_W
+    ld = w.stride(0) if w.size(0) > 1 else w.size(1)
+    x = x.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()
+        if bias.numel() != out_w:
+            raise NNRuntimeException(f"bias has {bias.numel()} elements, the GEMV produces {out_w}")
+    out = torch.empty(out_w, dtype=torch.float16, device=weight2d.device)
+    _check(lib.pimhip_execute_gemv(out.data_ptr(), x.data_ptr(), w.data_ptr(),
+                                   bias.data_ptr() if bias is not None else None, in_w, out_w, ld, act, order,
+                                   _stream_handle(stream)))
+    return out
+
+
+def _act_code(act_type):
+    # Only "aten::relu" selects an activation (aten_ops.cpp:622-624); "none" and "aten::max" do not.
+    return L.PIMHIP_ACT_RELU if act_type == "aten::relu" else L.PIMHIP_ACT_NONE
+
+
+def custom_aten_addmm(act_type, self_tensor, mat1_tensor, mat2_tensor, beta=1, alpha=1, stream=None):
+    """customAtenAddmm: act(mat1 . mat2 + self) with the reference's shape dispatch.
+
+    VM and MV products ignore beta and alpha exactly as the reference does (aten_ops.cpp:627-628).
+    """
+    _require_half_cuda(self_tensor, mat1_tensor, mat2_tensor)
+    dim_i0, dim_i1, dim_self = mat1_tensor.dim(), mat2_tensor.dim(), self_tensor.dim()
+    s1, s2 = gemm_broadcast(list(mat1_tensor.shape), list(mat2_tensor.shape))
+    gemm_type = get_gemm_type(s1, s2)
+    act = _act_code(act_type)
+
+    if gemm_type == GemmType.VM and dim_i0 > 1:
+        out_w, in_w = mat2_tensor.size(dim_i1 - 1), mat2_tensor.size(dim_i1 - 2)
+        y = _gemv(mat1_tensor.reshape(-1), mat2_tensor.reshape(in_w, out_w), self_tensor.reshape(-1), in_w, out_w,
+                  L.PIMHIP_I_X_W, act, stream)
+        shape = list(mat1_tensor.shape)
+        shape[dim_i0 - 1], shape[dim_i0 - 2] = out_w, 1
+        return y.view(shape)
+    if gemm_type == GemmType.MV and dim_i1 > 1:
+        out_w, in_w = mat1_tensor.size(dim_i0 - 2), mat1_tensor.size(dim_i0 - 1)
+        y = _gemv(mat2_tensor.reshape(-1), mat1_tensor.reshape(out_w, in_w), self_tensor.reshape(-1), in_w, out_w,
+                  L.PIMHIP_W_X_I, act, stream)
+        shape = list(mat2_tensor.shape)
+        shape[dim_i1 - 1], shape[dim_i1 - 2] = 1, out_w
+        return y.view(shape)
+    if dim_self == 1:
+        # True GEMM with a 1-D bias (aten_ops.cpp:695-711): LibTorch passthrough.
+        bias = self_tensor.unsqueeze(1).repeat(1, mat2_tensor.size(dim_i1 - 1))
+        m2 = mat2_tensor.squeeze(0) if dim_i1 != 2 else mat2_tensor
+        out = torch.addmm(bias, mat1_tensor, m2, beta=beta, alpha=alpha)
+        if act == L.PIMHIP_ACT_RELU:
+            out = torch.relu(out)
+        for _ in range(dim_i1 - 2):
+            out = out.unsqueeze(0)
+        return out
+    # Batched case (aten_ops.cpp:712-757).  The reference's ENABLE_PIM branch never stores its result; the
+    # LibTorch branch is the defined behaviour and is the one taken here.
+    out = torch.addmm(self_tensor, mat1_tensor, mat2_tensor, beta=beta, alpha=alpha)
+    if act == L.PIMHIP_ACT_RELU:
+        out = torch.relu(out)
+    return out
+
+
+def custom_aten_matmul(self_tensor, other_tensor, stream=None):
+    """customAtenMatmul: self . other with the reference's shape dispatch, no bias and no activation."""
+    _require_half_cuda(self_tensor, other_tensor)
+    dim_i0, dim_i1 = self_tensor.dim(), other_tensor.dim()
+    s1, s2 = gemm_broadcast(list(self_tensor.shape), list(other_tensor.shape))
+    gemm_type = get_gemm_type(s1, s2)
+
+    if gemm_type == GemmType.VM:
+        out_w, in_w = other_tensor.size(dim_i1 - 1), other_tensor.size(dim_i1 - 2)
+        y = _gemv(self_tensor.reshape(-1), other_tensor.reshape(in_w, out_w), None, in_w, out_w, L.PIMHIP_I_X_W,
+                  L.PIMHIP_ACT_NONE, stream)
+        if dim_i1 > dim_i0:
+            shape = list(other_tensor.shape)
+            shape[dim_i1 - 1], shape[dim_i1 - 2] = out_w, 1
+        else:
+            shape = list(self_tensor.shape)
+            shape[dim_i0 - 1], shape[dim_i0 - 2] = out_w, 1
+        return y.view(shape)
+    if gemm_type == GemmType.MV:
+        out_w, in_w = self_tensor.size(dim_i0 - 2), self_tensor.size(dim_i0 - 1)
+        y = _gemv(other_tensor.reshape(-1), self_tensor.reshape(out_w, in_w), None, in_w, out_w, L.PIMHIP_W_X_I,
+                  L.PIMHIP_ACT_NONE, stream)
+        if dim_i0 > dim_i1:
+            shape = list(self_tensor.shape)
+            shape[dim_i0 - 2] = out_w
+            shape.pop()
+        else:
+            shape = list(other_tensor.shape)
+            shape[dim_i1 - 1], shape[dim_i1 - 2] = 1, out_w
+        return y.view(shape)
+    if gemm_type == GemmType.VV:
+        lib = L.load()
+        _ensure_init(self_tensor)
+        a, b = self_tensor.contiguous(), other_tensor.contiguous()
+        in_w = 0
+        for i in range(dim_i0):
+            if a.size(i) != 1:
+                in_w = a.size(i)
+                break
+        if b.numel() < in_w or a.numel() < in_w:
+            raise NNRuntimeException("VV operands are shorter than the detected vector length")
+        if dim_i0 > dim_i1:
+            shape = list(self_tensor.shape)
+            shape[dim_i0 - 1], shape[dim_i0 - 2] = 1, 1
+        else:
+            shape = list(other_tensor.shape)
+            shape[dim_i1 - 1], shape[dim_i1 - 2] = 1, 1
+        numel = 1
+        for d in shape:
+            numel *= d
+        if numel != 1:
+            raise NNRuntimeException(f"VV output shape {shape} is not a single element")
+        out = torch.empty(shape, dtype=torch.float16, device=a.device)
+        _check(lib.pimhip_execute_dot(out.data_ptr(), a.data_ptr(), b.data_ptr(), in_w, _stream_handle(stream)))
+        return out
+    # MM (aten_ops.cpp:883-931): LibTorch passthrough.
+    return torch.matmul(self_tensor, other_tensor)
+
+
+def aten_linear(input_tensor, weight, bias=None, act_type="none", stream=None):
+    """atenLinear for a batch-1 input: y = act(W[out,in] . x + b), the MV order on W's own row-major bytes.
+
+    This is the product that ConvertLinearToAddmm + SwapAddmmInputs (+ FuseActivation) reduce aten::linear to
+    (compiler/source/frontend/optimizer/convert_linear_to_addmm.cpp:50-51, swap_addmm_inputs.cpp:45-97),
+    without the two transposes those passes insert.  Inputs with more than one row take the LibTorch passthrough.
+    """
+    _require_half_cuda(input_tensor, weight, bias)
+    out_w, in_w = weight.shape
+    if input_tensor.numel() != in_w:
+        out = torch.nn.functional.linear(input_tensor, weight, bias)
+        return torch.relu(out) if act_type == "aten::relu" else out
+    y = _gemv(input_tensor.reshape(-1), weight, bias, in_w, out_w, L.PIMHIP_W_X_I, _act_code(act_type), stream)
+    return y.view(list(input_tensor.shape[:-1]) + [out_w])
+
+
+def execute_gemv_group(inputs, weights, biases=None, act_types=None, stream=None):
+    """N sibling MV GEMVs (y_i = act_i(W_i . x_i + b_i)) in one launch.
+
+    Replaces executeMultiStream's one-stream-per-GEMV issue
+    (runtime/source/executor/op_executor/stream_ops_executor.cpp:27-50).  Returns the list of outputs.
+    """
+    lib = L.load()
+    n = len(weights)
+    if len(inputs) != n:
+        raise NNRuntimeException("inputs and weights differ in length")
+    biases = biases if biases is not None else [None] * n
+    act_types = act_types if act_types is not None else ["none"] * n
+    _require_half_cuda(*inputs, *weights, *biases)
+    if n == 0:
+        return []
+    _ensure_init(weights[0])
+    xs = [x.contiguous().reshape(-1) for x in inputs]
+    ws = [w.contiguous() for w in weights]
+    bs = [b.contiguous() if b is not None else None for b in biases]
+    outs = [torch.empty(w.size(0), dtype=torch.float16, device=w.device) for w in ws]
+    for x, w in zip(xs, ws):
+        if w.dim() != 2 or x.numel() != w.size(1):
+            raise NNRuntimeException("each weight must be [out, in] and each input must have `in` elements")
+    vp = ctypes.c_void_p * n
+    rc = lib.pimhip_execute_gemv_group(
+        n, vp(*[o.data_ptr() for o in outs]), vp(*[x.data_ptr() for x in xs]), vp(*[w.data_ptr() for w in ws]),
+        vp(*[b.data_ptr() if b is not None else None for b in bs]),
+        (ctypes.c_int64 * n)(*[w.size(1) for w in ws]), (ctypes.c_int64 * n)(*[w.size(0) for w in ws]),
+        (ctypes.c_int * n)(*[_act_code(a) for a in act_types]), _stream_handle(stream))
+    _check(rc)
+    return outs
+
+
+def input_projection(x, w, bias=None, stream=None):
+    """out[T, N] fp32 = x[T, K] . w[N, K]^T + bias[N] (fp32) on the matrix cores."""
+    lib = L.load()
+    _require_half_cuda(x, w)
+    _ensure_init(w)
+    x, w = x.contiguous(), w.contiguous()
+    T, K = x.shape
+    N = w.size(0)
+    if w.size(1) != K:
+        raise NNRuntimeException("x and w disagree on the reduction width")
+    if bias is not None:
+        if bias.dtype != torch.float32 or not bias.is_cuda or bias.numel() != N:
+            raise NNRuntimeException("bias must be an fp32 GPU tensor of N elements")
+        bias = bias.contiguous()
+    out = torch.empty((T, N), dtype=torch.float32, device=x.device)
+    _check(lib.pimhip_input_projection(out.data_ptr(), x.data_ptr(), w.data_ptr(),
+                                       bias.data_ptr() if bias is not None else None, T, K, N,
+                                       _stream_handle(stream)))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------
+# LSTM
+# ---------------------------------------------------------------------------------------------------
+class LstmPlan:
+    """Owns a PimHipLstmPlan: the one-time weight preparation of an aten::lstm layer stack.
+
+    Counterpart of ModelBuilder::buildLstmParameterVector / reArangeLstmWeights
+    (runtime/source/builder/model_builder.cpp:158-319): `params` is the LibTorch-ordered list
+    (w_ih, w_hh[, b_ih, b_hh]) per layer and direction.
+    """
+
+    MODE_AUTO, MODE_STEP, MODE_SEQUENCE = 0, 1, 2
+
+    def __init__(self, params, has_biases, num_layers, bidirectional, max_seq_len, stream=None):
+        lib = L.load()
+        _require_half_cuda(*params)
+        _ensure_init(params[0])
+        self.params = [p.contiguous() for p in params]  # keeps the weights alive for the plan's lifetime
+        self.has_biases = bool(has_biases)
+        self.num_layers = int(num_layers)
+        self.num_dirs = 2 if bidirectional else 1
+        self.hidden = self.params[1].size(1)
+        self.input_size = self.params[0].size(1)
+        per_cell = 4 if has_biases else 2
+        if len(self.params) != self.num_layers * self.num_dirs * per_cell:
+            raise NNRuntimeException(
+                f"expected {self.num_layers * self.num_dirs * per_cell} parameter tensors, got {len(self.params)}")
+        for ci in range(self.num_layers * self.num_dirs):
+            in_w = self.input_size if ci < self.num_dirs else self.num_dirs * self.hidden
+            w_ih, w_hh = self.params[ci * per_cell], self.params[ci * per_cell + 1]
+            if tuple(w_ih.shape) != (4 * self.hidden, in_w) or tuple(w_hh.shape) != (4 * self.hidden, self.hidden):
+                raise NNRuntimeException(f"parameter shapes of cell {ci} do not match an LSTM with H={self.hidden}")
+            if has_biases:
+                for b in self.params[ci * per_cell + 2:ci * per_cell + 4]:
+                    if b.numel() != 4 * self.hidden:
+                        raise NNRuntimeException(f"bias of cell {ci} does not have 4H elements")
+        self.max_seq_len = int(max_seq_len)
+        self.device = self.params[0].device
+        n = len(self.params)
+        arr = (ctypes.c_void_p * n)(*[p.data_ptr() for p in self.params])
+        handle = ctypes.c_void_p()
+        _check(lib.pimhip_lstm_plan_create(ctypes.byref(handle), arr, n, int(self.has_biases), self.num_layers,
+                                           int(self.num_dirs == 2), self.input_size, self.hidden, self.max_seq_len,
+                                           _stream_handle(stream)))
+        self._handle = handle
+        self._finalizer = weakref.finalize(self, LstmPlan._destroy, handle.value)
+
+    @staticmethod
+    def _destroy(handle_value):
+        try:
+            L.load().pimhip_lstm_plan_destroy(ctypes.c_void_p(handle_value))
+        except Exception:  # interpreter shutdown
+            pass
+
+    def set_mode(self, mode):
+        _check(L.load().pimhip_lstm_plan_set_mode(self._handle, mode))
+
+    def set_spin_limit(self, limit):
+        _check(L.load().pimhip_lstm_plan_set_spin_limit(self._handle, limit))
+
+    def status(self):
+        """Raises NNRuntimeException if the last forward's persistent kernel gave up a wait.  Synchronises."""
+        torch.cuda.synchronize(self.device)
+        _check(L.load().pimhip_lstm_plan_status(self._handle))
+
+    def forward(self, x2d, h0, c0, stream=None):
+        """x2d [T, I]; h0, c0 [L*D, H] (any shape with those elements).  Returns y [T, D*H], hn, cn [L*D, H]."""
+        lib = L.load()
+        _require_half_cuda(x2d, h0, c0)
+        T = x2d.size(0)
+        if x2d.dim() != 2 or x2d.size(1) != self.input_size:
+            raise NNRuntimeException(f"input must be [T, {self.input_size}], got {list(x2d.shape)}")
+        n_state = self.num_layers * self.num_dirs * self.hidden
+        if h0.numel() != n_state or c0.numel() != n_state:
+            raise NNRuntimeException(f"h0 / c0 must have {n_state} elements")
+        x2d, h0, c0 = x2d.contiguous(), h0.contiguous(), c0.contiguous()
+        y = torch.empty((T, self.num_dirs * self.hidden), dtype=torch.float16, device=self.device)
+        hn = torch.empty((self.num_layers * self.num_dirs, self.hidden), dtype=torch.float16, device=self.device)
+        cn = torch.empty_like(hn)
+        _check(lib.pimhip_lstm_forward(self._handle, x2d.data_ptr(), h0.data_ptr(), c0.data_ptr(), y.data_ptr(),
+                                       hn.data_ptr(), cn.data_ptr(), T, _stream_handle(stream)))
+        return y, hn, cn
+
+
+_plan_cache = {}
+
+
+def _plan_for(params, has_biases, num_layers, bidirectional, seq_len):
+    key = (tuple(p.data_ptr() for p in params), bool(has_biases), int(num_layers), bool(bidirectional))
+    plan = _plan_cache.get(key)
+    if plan is None or plan.max_seq_len < seq_len:
+        cap = max(int(seq_len), 2 * plan.max_seq_len if plan is not None else 0, 16)
+        plan = LstmPlan(params, has_biases, num_layers, bidirectional, cap)
+        _plan_cache[key] = plan
+    return plan
+
+
+def aten_lstm1(input, hx, params, has_biases, num_layers, dropout, train, bidirectional, batch_first, stream=None):
+    """atenLstm1: padded-sequence aten::lstm, batch 1 (the reference's GPU LSTM hard-codes batch 1,
+    miopen_ops_executor.cpp:117).  dropout is ignored as in the reference (aten_ops.cpp:333); train must be false.
+    Returns (output, hy, cy) shaped like at::lstm's results."""
+    del dropout
+    if train:
+        raise NNRuntimeException("training mode is not part of this inference path")
+    if input.dim() != 3:
+        raise NNRuntimeException("input must be [T, 1, I] or, with batch_first, [1, T, I]")
+    batch = input.size(0) if batch_first else input.size(1)
+    if batch != 1:
+        raise NNRuntimeException(f"batch size {batch} is not supported (batch 1 only)")
+    T = input.size(1) if batch_first else input.size(0)
+    h0, c0 = hx[0], hx[1]
+    plan = _plan_for(list(params), has_biases, num_layers, bidirectional, T)
+    y, hn, cn = plan.forward(input.reshape(T, input.size(2)), h0, c0, stream)
+    D, H = plan.num_dirs, plan.hidden
+    out = y.view(1, T, D * H) if batch_first else y.view(T, 1, D * H)
+    return out, hn.view(num_layers * D, 1, H), cn.view(num_layers * D, 1, H)
+
+
+def aten_lstm2(data, batch_sizes, hx, params, has_biases, num_layers, dropout, train, bidirectional, stream=None):
+    """atenLstm2: packed-sequence aten::lstm.  With batch 1 the packed data [T, I] is the padded sequence and
+    batch_sizes must be all ones."""
+    del dropout
+    if train:
+        raise NNRuntimeException("training mode is not part of this inference path")
+    if data.dim() != 2:
+        raise NNRuntimeException("packed data must be [sum(batch_sizes), I]")
+    bs = batch_sizes.cpu() if isinstance(batch_sizes, torch.Tensor) else torch.as_tensor(batch_sizes)
+    if bs.numel() != data.size(0) or not bool((bs == 1).all()):
+        raise NNRuntimeException("only batch 1 packed sequences (batch_sizes all ones) are supported")
+    T = data.size(0)
+    plan = _plan_for(list(params), has_biases, num_layers, bidirectional, T)
+    y, hn, cn = plan.forward(data, hx[0], hx[1], stream)
+    D, H = plan.num_dirs, plan.hidden
+    return y, hn.view(num_layers * D, 1, H), cn.view(num_layers * D, 1, H)
