@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the fp16 GEMV + LSTM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  A step is one pass of the batch-1 fp16 GEMV sweep
+(out,in) in {(4096,4096), (16384,4096), (4096,16384), (32000,1024)}, y = W.x + b, with every operand already
+resident in HBM and the weights COLD: each shape rotates over enough distinct weight copies (>= 500 MB per shape,
+about 2 GB per round) that the 256 MB Infinity Cache cannot hold what the next launch reads.  `value` is the
+algorithmic bytes of a step (2NK + 2K + 2N + 2N per GEMV) divided by the measured time of a step, in GB/s.
+The same line carries the LSTM figure of the metric (microseconds per layer-step of the 2-layer H=1024, T=200
+sequence, persistent kernel), the MFMA utilisation of the input projection, a roofline object for the dominant
+kernel and the CPU baseline (LibTorch CPU at::addmm, the op the reference's atenAddmm passes through to, on the
+host cores of this box).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix rate
+SWEEP = [(4096, 4096), (16384, 4096), (4096, 16384), (32000, 1024)]
+POOL_BYTES_PER_SHAPE = 512 << 20
+
+
+def gemv_bytes(n, k, bias=True):
+    return 2 * n * k + 2 * k + (2 * n if bias else 0) + 2 * n
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the LibTorch CPU timing")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+    import pimaicompiler_amd as P
+    from pimaicompiler_amd import _lib as L
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a gfx950 GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    P.initialize(0)
+    lib = L.load()
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+
+    # ---- operands, resident in HBM ---------------------------------------------------------------------------
+    g = torch.Generator(device=dev).manual_seed(2001)
+    shapes = []
+    for n, k in SWEEP:
+        copies = max(2, math.ceil(POOL_BYTES_PER_SHAPE / (2 * n * k)))
+        pool = torch.empty((copies, n, k), dtype=torch.float16, device=dev)
+        for c in range(copies):
+            pool[c] = (0.02 * torch.randn(n, k, generator=g, device=dev)).half()
+        x = (2 * torch.rand(k, generator=g, device=dev) - 1).half()
+        b = (0.01 * torch.randn(n, generator=g, device=dev)).half()
+        y = torch.empty(n, dtype=torch.float16, device=dev)
+        shapes.append(dict(n=n, k=k, copies=copies, pool=pool, x=x, b=b, y=y, it=0))
+    torch.cuda.synchronize()
+
+    def launch(s):
+        w = s["pool"][s["it"] % s["copies"]]
+        s["it"] += 1
+        rc = lib.pimhip_execute_gemv(s["y"].data_ptr(), s["x"].data_ptr(), w.data_ptr(), s["b"].data_ptr(), s["k"], s["n"],
+                                     0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+        if rc != 0:
+            raise RuntimeError(lib.pimhip_last_error().decode())
+
+    def step():
+        for s in shapes:
+            launch(s)
+
+    # ---- sanity: a few rows of every shape against float64 on the host (outside any timed region) ---------------
+    for s in shapes:
+        launch(s)
+        torch.cuda.synchronize()
+        w = s["pool"][(s["it"] - 1) % s["copies"]]
+        rows = torch.arange(0, s["n"], max(1, s["n"] // 32), device=dev)[:32]
+        want = w[rows].double().cpu() @ s["x"].double().cpu() + s["b"][rows].double().cpu()
+        err = float((s["y"][rows].double().cpu() - want).abs().max())
+        if not err <= 2e-3:
+            raise RuntimeError(f"GEMV {s['n']}x{s['k']} differs from the float64 product by {err}")
+
+    # ---- the timed region: exactly K steps -----------------------------------------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    step_bytes = sum(gemv_bytes(n, k) for n, k in SWEEP)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-shape launch durations (HIP events on the launch stream, cold rotation, back to back) ---------------
+    per_shape = []
+    for s in shapes:
+        reps = max(50, args.steps)
+        for _ in range(5):
+            launch(s)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(reps):
+            launch(s)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        bts = gemv_bytes(s["n"], s["k"])
+        per_shape.append(dict(out=s["n"], **{"in": s["k"]}, us=round(us, 3), gbs=round(bts / us / 1e3, 1),
+                              frac_of_peak=round(bts / us / 1e3 / HBM_PEAK_GBS, 4)))
+    # Dominant kernel: gemv_mv_f16_kernel<2,4,4,4>, which runs the three in >= 4096 shapes (90 % of a step's bytes).
+    dom = [(p, gemv_bytes(p["out"], p["in"])) for p in per_shape if p["in"] >= 4096]
+    dom_bytes = sum(b for _, b in dom) / len(dom)
+    dom_us = sum(p["us"] for p, _ in dom) / len(dom)
+    achieved = dom_bytes / dom_us / 1e3
+    roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
+                    kernel="gemv_mv_f16_kernel<2,4,4,4>", bytes_per_launch=int(dom_bytes), us_per_launch=round(dom_us, 3))
+
+    # ---- LSTM: RNNT-style 2 layers, I=240, H=1024, T=200 (400 layer-steps per call) ------------------------------
+    from oracle import oracle  # seeded inputs only; the oracle's arithmetic is not called here
+    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    lstm = {}
+    for mode, name in ((2, "persistent"), (1, "per_step_launches")):
+        plan = P.LstmPlan([p.to(dev) for p in params], True, 2, False, 200)
+        plan.set_mode(mode)
+        xd, hd, cd = x.reshape(200, 240).to(dev), h0.to(dev), c0.to(dev)
+        for _ in range(5):
+            plan.forward(xd, hd, cd)
+        plan.status()
+        reps = 30
+        e0.record(stream)
+        for _ in range(reps):
+            plan.forward(xd, hd, cd)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        plan.status()
+        lstm[name] = e0.elapsed_time(e1) * 1e3 / reps / 400
+    # input projection of layer 1 (T=200, I=1024, 4H=4096): the MFMA kernel
+    xp_x = torch.randn(200, 1024, device=dev).half()
+    xp_w = (0.03 * torch.randn(4096, 1024, device=dev)).half()
+    for _ in range(5):
+        P.input_projection(xp_x, xp_w)
+    torch.cuda.synchronize()
+    e0.record(stream)
+    for _ in range(50):
+        P.input_projection(xp_x, xp_w)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    xp_us = e0.elapsed_time(e1) * 1e3 / 50
+    xp_tflops = 2 * 200 * 1024 * 4096 / xp_us / 1e6
+
+    # ---- CPU baseline: LibTorch CPU at::addmm in fp16 on the same sweep, bounded sample ---------------------------
+    cpu = None
+    if not args.no_cpu_baseline:
+        threads = torch.get_num_threads()
+        t_total, b_total, detail = 0.0, 0, []
+        for s in shapes:
+            W = s["pool"][0].cpu()
+            xc, bc = s["x"].cpu().reshape(1, -1), s["b"].cpu()
+            Wt = W.t()
+            for _ in range(2):
+                torch.addmm(bc, xc, Wt)
+            times = []
+            t_start = time.perf_counter()
+            while len(times) < 20 and (time.perf_counter() - t_start) < 4.0:
+                t = time.perf_counter()
+                torch.addmm(bc, xc, Wt)
+                times.append(time.perf_counter() - t)
+            med = sorted(times)[len(times) // 2]
+            t_total += med
+            b_total += gemv_bytes(s["n"], s["k"])
+            detail.append(f"{s['n']}x{s['k']}: {med * 1e3:.2f} ms")
+        cpu = dict(value=round(b_total / t_total / 1e9, 2), unit="GB/s", cores=threads, kind="reference",
+                   sample="LibTorch CPU at::addmm(b, x, W^T) in fp16, the op atenAddmm passes through to: median of <= 20 "
+                          "runs (<= 4 s) per sweep shape after 2 warm-ups, one pass of the same 4-GEMV sweep; " + "; ".join(detail))
+
+    out = {
+        "metric": "fp16 GEMV HBM GB/s (% of peak) at 1 GPU; LSTM us/layer-step at H=1024",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 storage, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "GEMV sweep, batch 1, fp16: (out,in) in {(4096,4096),(16384,4096),(4096,16384),(32000,1024)}, "
+                               "y = W.x + b, cold weights (rotating copies, >= 500 MB per shape)",
+                   "bytes_per_step": step_bytes},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "gemv_per_shape": per_shape,
+        "lstm_us_per_layer_step": round(lstm["persistent"], 3),
+        "lstm_us_per_layer_step_per_step_launches": round(lstm["per_step_launches"], 3),
+        "lstm_config": "2 layers unidirectional, I=240, H=1024, T=200, batch 1 (400 layer-steps per call, input projection included)",
+        "input_projection": {"shape": "T=200, I=1024, 4H=4096", "us": round(xp_us, 2), "tflops": round(xp_tflops, 2),
+                             "mfma_utilisation": round(xp_tflops / MFMA_FP16_PEAK_TFLOPS, 5)},
+        "wall_ms_timed_region": round(wall_ms, 2),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

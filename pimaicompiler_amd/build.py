@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libpimhip.so")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-result",
+    "-Wno-unused-result", "-Wno-unused-value",
 ]
 
 

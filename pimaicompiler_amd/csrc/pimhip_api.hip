@@ -152,7 +152,9 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     if (slices < 1) slices = 1;
     int k_per_slice = (int)((K + slices - 1) / slices);
     k_per_slice = (k_per_slice + WAVES - 1) / WAVES * WAVES;
+    if (k_per_slice < WAVES) k_per_slice = WAVES;  // K == 0: one empty slice, y = act(bias)
     slices = (int)((K + k_per_slice - 1) / k_per_slice);
+    if (slices < 1) slices = 1;
     SplitWorkspace* ws = nullptr;
     float* partial = nullptr;
     unsigned int* tickets = nullptr;
@@ -319,6 +321,8 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
 // ================================================================================================
 namespace
 {
+__global__ void fill_u32_kernel(unsigned int* p, unsigned int v) { *p = v; }
+
 int launch_input_projection(float* out, const half_t* x, const half_t* w, const float* bias, int64_t T, int64_t K,
                             int64_t N, hipStream_t s)
 {
@@ -589,7 +593,8 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     int dev = -1;
     PIMHIP_HIP_CHECK(hipGetDevice(&dev));
     if (dev != plan->device) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan belongs to device %d, current device is %d", plan->device, dev);
-    if (!x || !h0 || !c0 || !y || !hn || !cn) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "x, h0, c0, y, hn and cn must be non-null");
+    if (!h0 || !c0 || !hn || !cn) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "h0, c0, hn and cn must be non-null");
+    if (seq_len > 0 && (!x || !y)) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "x and y must be non-null when seq_len > 0");
     if (seq_len < 0 || seq_len > plan->max_seq_len)
         return fail(PIMHIP_ERR_INVALID_ARGUMENT, "seq_len=%lld not in [0, max_seq_len=%lld]", (long long)seq_len, (long long)plan->max_seq_len);
     if (!aligned16(x) || !aligned16(h0) || !aligned16(y))
@@ -612,6 +617,12 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         return PIMHIP_OK;
     }
 
+    if (*plan->abort_host != 0u) {
+        // The previous forward of this plan timed out: re-arm the flag (a fill kernel, not a memset node, so
+        // that callers may capture this call).
+        fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 0u);
+        *plan->abort_host = 0u;
+    }
     const bool use_seq = (plan->mode == 2) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2);
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
     // seq_len == 1: fuse the input projection into the step (one launch per layer and direction).

@@ -1,0 +1,250 @@
+"""GPU parity of the LSTM path (fused step kernel, persistent sequence kernel, MFMA input projection), called
+through the C ABI.  Checkers: LibTorch CPU at::lstm live on the same seeded inputs (fp16, the arbiter, and fp32 on
+the same fp16-valued weights), the committed LibTorch golden vectors, the CPU oracle, and structural properties.
+Tolerance: max abs error <= 5e-3 on y / h / c after the full sequence."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+LSTM_TOL = 5e-3
+DEV = "cuda:0"
+MODES = [1, 2]  # 1: one fused launch per step, 2: persistent sequence kernel
+
+
+def maxabs(a, b):
+    b = b if isinstance(b, torch.Tensor) else torch.as_tensor(np.asarray(b, dtype=np.float32))
+    return float((a.detach().float().cpu().reshape(-1) - b.float().reshape(-1)).abs().max())
+
+
+def run_plan(ops, params, x, h0, c0, has_b, L, bidir, mode, T=None):
+    T = x.shape[0] if T is None else T
+    plan = ops.LstmPlan([p.to(DEV) for p in params], has_b, L, bidir, max(T, 1))
+    if mode:
+        plan.set_mode(mode)
+    y, hn, cn = plan.forward(x.reshape(x.shape[0], -1).to(DEV), h0.to(DEV), c0.to(DEV))
+    plan.status()
+    return y, hn, cn
+
+
+# ---- tiny golden cases (LibTorch CPU, committed) --------------------------------------------------------------
+TINY = [f"L{L}_D{D}_b{b}" for L in (1, 2) for D in (1, 2) for b in (1, 0)]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("key", TINY)
+def test_lstm_tiny_golden(ops, golden, key, mode):
+    g = golden["lstm_tiny"]
+    L, D, has_b = int(key[1]), int(key[4]), int(key[7])
+    n = L * D * (4 if has_b else 2)
+    params = [torch.as_tensor(g[f"{key}_p{i}"]) for i in range(n)]
+    x, h0, c0 = (torch.as_tensor(g[key + s]) for s in ("_x", "_h0", "_c0"))
+    y, hn, cn = run_plan(ops, params, x, h0, c0, has_b, L, D == 2, mode)
+    assert maxabs(y, g[key + "_y"]) <= 2e-3
+    assert maxabs(hn, g[key + "_hn"]) <= 2e-3
+    assert maxabs(cn, g[key + "_cn"]) <= 2e-3
+
+
+# ---- against the CPU oracle over ragged shapes ---------------------------------------------------------------
+CASES = [  # I, H, L, bidirectional, T, biases
+    (8, 8, 1, False, 1, True), (8, 8, 1, False, 2, True), (24, 40, 1, False, 9, True), (64, 320, 1, False, 13, True),
+    (16, 72, 2, True, 6, True), (32, 128, 3, False, 5, False), (32, 128, 3, True, 4, True), (240, 512, 2, False, 17, True),
+    (8, 1024, 1, False, 3, True), (40, 1032, 1, False, 3, True), (16, 2048, 1, True, 2, False),
+]
+
+
+@pytest.mark.parametrize("mode", [0] + MODES)
+@pytest.mark.parametrize("I,H,L,bidir,T,has_b", CASES)
+def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
+    if mode == 2 and H > 1024:
+        pytest.skip("the persistent kernel takes hidden sizes up to 1024; larger ones run step by step")
+    params, x, h0, c0 = oracle.lstm_inputs(900 + I + H + T, I, H, L, bidir, T, has_b)
+    g = torch.Generator().manual_seed(T)
+    h0 = (0.3 * torch.randn(h0.shape, generator=g)).half()
+    c0 = (0.3 * torch.randn(c0.shape, generator=g)).half()
+    D = 2 if bidir else 1
+    wy, whn, wcn = oracle.lstm(x.numpy().reshape(T, I), h0.numpy().reshape(L * D, H), c0.numpy().reshape(L * D, H),
+                               [p.numpy() for p in params], has_b, L, bidir)
+    y, hn, cn = run_plan(ops, params, x, h0, c0, has_b, L, bidir, mode)
+    assert maxabs(y, wy) <= 2e-3 and maxabs(hn, whn) <= 2e-3 and maxabs(cn, wcn) <= 2e-3
+
+
+def test_persistent_kernel_refuses_what_it_cannot_hold(ops):
+    params, x, h0, c0 = oracle.lstm_inputs(1, 16, 2048, 1, False, 2)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 2)
+    with pytest.raises(ops.NNRuntimeException):
+        plan.set_mode(2)
+
+
+# ---- benchmark configurations -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("mode", MODES)
+def test_lstm_c3_rnnt_matches_libtorch_cpu(ops, golden, mode):
+    """2 layers unidirectional, I=240, H=1024, T=200."""
+    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    wy, whn, wcn = oracle.torch_lstm(x, h0, c0, params, True, 2, False)                      # fp16 CPU (arbiter)
+    fy, fhn, fcn = oracle.torch_lstm(x.float(), h0.float(), c0.float(), [p.float() for p in params], True, 2, False)
+    y, hn, cn = run_plan(ops, params, x, h0, c0, True, 2, False, mode)
+    for got, w16, w32 in ((y, wy, fy), (hn, whn, fhn), (cn, wcn, fcn)):
+        assert maxabs(got, w16) <= LSTM_TOL
+        assert maxabs(got, w32) <= LSTM_TOL
+    g = golden["lstm_large"]
+    assert maxabs(hn, g["c3_hn"]) <= LSTM_TOL and maxabs(cn, g["c3_cn"]) <= LSTM_TOL
+    assert maxabs(y.reshape(200, 1024)[::25, ::16], g["c3_y_samples"]) <= LSTM_TOL
+
+
+def test_lstm_c4_gnmt_stack_matches_libtorch_cpu(ops, golden):
+    """Four at::lstm calls as GNMT composes them (L0 bidirectional I=1024 -> 2048, L1 I=2048, L2, L3 I=1024), T=50,
+    then the 1024 -> 32000 classifier GEMV on the last step's output."""
+    g = golden["lstm_large"]
+    seq_dev, seq_cpu = None, None
+    for li, (in_w, bidir) in enumerate([(1024, True), (2048, False), (1024, False), (1024, False)]):
+        params, x0, h0, c0 = oracle.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
+        if seq_dev is None:
+            seq_dev, seq_cpu = x0.to(DEV), x0
+        wy, whn, wcn = oracle.torch_lstm(seq_cpu, h0, c0, params, True, 1, bidir)
+        y, hn, cn = ops.aten_lstm1(seq_dev, (h0.to(DEV), c0.to(DEV)), [p.to(DEV) for p in params], True, 1, 0.0, False,
+                                   bidir, False)
+        D = 2 if bidir else 1
+        assert list(y.shape) == [50, 1, D * 1024] and list(hn.shape) == [D, 1, 1024] and list(cn.shape) == [D, 1, 1024]
+        assert maxabs(y, wy) <= LSTM_TOL and maxabs(hn, whn) <= LSTM_TOL and maxabs(cn, wcn) <= LSTM_TOL
+        assert maxabs(hn, g[f"c4_l{li}_hn"]) <= LSTM_TOL and maxabs(cn, g[f"c4_l{li}_cn"]) <= LSTM_TOL
+        assert maxabs(y.reshape(50, -1)[::7, ::32], g[f"c4_l{li}_y_samples"]) <= LSTM_TOL
+        seq_dev, seq_cpu = y, wy
+    W, _, b = oracle.gemv_inputs(4010, 32000, 1024)
+    logits = ops.aten_linear(seq_dev[-1].reshape(1, 1024), W.to(DEV), b.to(DEV)).reshape(-1)
+    want = oracle.torch_addmm(b, seq_cpu[-1].reshape(1, 1024), W).reshape(-1)
+    # the GEMV input differs by the LSTM's own error (<= 5e-3 per element) times |W| summed: allow for it
+    assert maxabs(logits, want) <= 2e-3 + LSTM_TOL * 0.02 * math.sqrt(1024) * 0.5
+    assert maxabs(logits[torch.as_tensor(g["c4_logits_idx"])], g["c4_logits_samples"]) <= 2e-3 + LSTM_TOL * 0.02 * math.sqrt(1024) * 0.5
+
+
+# ---- interface forms --------------------------------------------------------------------------------------------
+def test_lstm1_batch_first_and_lstm2_packed_agree(ops):
+    params, x, h0, c0 = oracle.lstm_inputs(55, 32, 64, 2, True, 6)
+    pd = [p.to(DEV) for p in params]
+    hx = (h0.to(DEV), c0.to(DEV))
+    y, hn, cn = ops.aten_lstm1(x.to(DEV), hx, pd, True, 2, 0.5, False, True, False)       # dropout is ignored
+    yb, hnb, cnb = ops.aten_lstm1(x.to(DEV).transpose(0, 1), hx, pd, True, 2, 0.0, False, True, True)
+    assert list(y.shape) == [6, 1, 128] and list(yb.shape) == [1, 6, 128]
+    assert torch.equal(y.reshape(-1), yb.reshape(-1)) and torch.equal(hn, hnb) and torch.equal(cn, cnb)
+    yp, hnp, cnp = ops.aten_lstm2(x.to(DEV).reshape(6, 32), torch.ones(6, dtype=torch.int64), hx, pd, True, 2, 0.0, False, True)
+    assert list(yp.shape) == [6, 128]
+    assert torch.equal(y.reshape(-1), yp.reshape(-1)) and torch.equal(hn, hnp) and torch.equal(cn, cnp)
+    wy, whn, wcn = oracle.torch_lstm(x, h0, c0, params, True, 2, True)
+    assert maxabs(y, wy) <= 2e-3 and maxabs(hn, whn) <= 2e-3 and maxabs(cn, wcn) <= 2e-3
+    with pytest.raises(ops.NNRuntimeException):
+        ops.aten_lstm1(x.to(DEV).repeat(1, 2, 1), hx, pd, True, 2, 0.0, False, True, False)   # batch 2
+    with pytest.raises(ops.NNRuntimeException):
+        ops.aten_lstm2(x.to(DEV).reshape(6, 32), torch.tensor([2, 1, 1, 1, 1, 0]), hx, pd, True, 2, 0.0, False, True)
+
+
+def test_lstm_decode_loop_step_by_step_equals_one_sequence_call(ops):
+    """The decoders call aten::lstm with seq_len == 1 inside prim::Loop, feeding (hy, cy) back: T such calls must
+    reproduce one call over the whole sequence (same rounding points: h fp16 every step; c passes through fp16
+    between calls, so c is compared to tolerance)."""
+    params, x, h0, c0 = oracle.lstm_inputs(66, 64, 256, 2, False, 12)
+    pd = [p.to(DEV) for p in params]
+    y_all, hn_all, cn_all = ops.aten_lstm1(x.to(DEV), (h0.to(DEV), c0.to(DEV)), pd, True, 2, 0.0, False, False, False)
+    h, c = h0.to(DEV), c0.to(DEV)
+    ys = []
+    for t in range(12):
+        y, h, c = ops.aten_lstm1(x[t:t + 1].to(DEV), (h, c), pd, True, 2, 0.0, False, False, False)
+        ys.append(y)
+    assert maxabs(torch.cat(ys), y_all.cpu()) <= 2e-3
+    assert maxabs(h, hn_all.cpu()) <= 2e-3 and maxabs(c, cn_all.cpu()) <= 2e-3
+
+
+def test_lstm_zero_length_sequence_passes_state_through(ops):
+    params, x, h0, c0 = oracle.lstm_inputs(77, 16, 32, 1, False, 4)
+    g = torch.Generator().manual_seed(1)
+    h0 = torch.randn(h0.shape, generator=g).half()
+    c0 = torch.randn(c0.shape, generator=g).half()
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 4)
+    y, hn, cn = plan.forward(x[:0].reshape(0, 16).to(DEV), h0.to(DEV), c0.to(DEV))
+    assert y.shape[0] == 0 and torch.equal(hn.cpu().reshape(-1), h0.reshape(-1)) and torch.equal(cn.cpu().reshape(-1), c0.reshape(-1))
+
+
+def test_lstm_plan_reuse_and_sequence_longer_than_plan(ops):
+    params, x, h0, c0 = oracle.lstm_inputs(88, 16, 64, 1, False, 20)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 10)
+    with pytest.raises(ops.NNRuntimeException):
+        plan.forward(x.reshape(20, 16).to(DEV), h0.to(DEV), c0.to(DEV))
+    want = oracle.torch_lstm(x[:10], h0, c0, params, True, 1, False)
+    for _ in range(3):  # exchange tags keep advancing across launches of one plan
+        y, hn, cn = plan.forward(x[:10].reshape(10, 16).to(DEV), h0.to(DEV), c0.to(DEV))
+        plan.status()
+        assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
+
+
+# ---- structure at full size -------------------------------------------------------------------------------------
+def test_lstm_full_size_zero_weights_closed_form(ops):
+    H, I, T = 1024, 240, 40
+    b_ih = torch.cat([torch.full((H,), 0.5), torch.full((H,), -1.0), torch.full((H,), 2.0), torch.full((H,), 0.25)]).half()
+    b_hh = torch.cat([torch.full((H,), 0.25), torch.full((H,), 0.5), torch.full((H,), -0.5), torch.full((H,), 1.0)]).half()
+    params = [torch.zeros(4 * H, I).half(), torch.zeros(4 * H, H).half(), b_ih, b_hh]
+    x = torch.randn(T, 1, I).half()
+    h0, c0 = torch.zeros(1, 1, H).half(), torch.full((1, 1, H), 0.75).half()
+    sig = lambda v: 1 / (1 + math.exp(-v))
+    i, f, g, o = sig(0.75), sig(-0.5), math.tanh(1.5), sig(1.25)
+    for mode in MODES:
+        y, hn, cn = run_plan(ops, params, x, h0, c0, True, 1, False, mode)
+        c = 0.75
+        for t in range(T):
+            c = f * c + i * g
+            assert float((y[t].float() - o * math.tanh(c)).abs().max()) <= 6e-4
+        assert float((cn.float() - c).abs().max()) <= 1e-3
+
+
+def test_lstm_bidirectional_equals_forward_on_reversed_input(ops):
+    params, x, h0, c0 = oracle.lstm_inputs(99, 128, 1024, 1, True, 24)
+    y, hn, cn = run_plan(ops, params, x, h0, c0, True, 1, True, 2)
+    yf, hf, cf = run_plan(ops, params[:4], x, h0[:1], c0[:1], True, 1, False, 2)
+    yb, hb, cb = run_plan(ops, params[4:], x.flip(0), h0[1:], c0[1:], True, 1, False, 2)
+    assert torch.equal(y[:, :1024], yf) and torch.equal(y[:, 1024:], yb.flip(0))
+    assert torch.equal(hn[0], hf[0]) and torch.equal(hn[1], hb[0]) and torch.equal(cn[1], cb[0])
+    assert torch.equal(hn[1], y[0, 1024:]) and torch.equal(hn[0], y[-1, :1024])
+
+
+def test_step_and_sequence_kernels_agree(ops):
+    params, x, h0, c0 = oracle.lstm_inputs(111, 1024, 1024, 1, False, 50)
+    y1, h1, c1 = run_plan(ops, params, x, h0, c0, True, 1, False, 1)
+    y2, h2, c2 = run_plan(ops, params, x, h0, c0, True, 1, False, 2)
+    assert maxabs(y1, y2.cpu()) <= 1e-3 and maxabs(c1, c2.cpu()) <= 1e-3
+
+
+# ---- the bounded wait ---------------------------------------------------------------------------------------------
+def test_persistent_kernel_wait_gives_up_and_reports(ops):
+    """Forced from the host: with a spin limit of 0 every wait gives up at its first unsuccessful poll, the kernel
+    still runs to its end, and the plan reports the time-out.  A later forward with the default limit works."""
+    params, x, h0, c0 = oracle.lstm_inputs(123, 64, 1024, 1, False, 30)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 30)
+    plan.set_mode(2)
+    plan.set_spin_limit(0)
+    plan.forward(x.reshape(30, 64).to(DEV), h0.to(DEV), c0.to(DEV))
+    with pytest.raises(ops.NNRuntimeException, match="gave up"):
+        plan.status()
+    plan.set_spin_limit(1 << 22)
+    y, hn, cn = plan.forward(x.reshape(30, 64).to(DEV), h0.to(DEV), c0.to(DEV))
+    plan.status()
+    want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
+    assert maxabs(y, want[0]) <= 2e-3
+
+
+# ---- input projection (the MFMA kernel) against fp32 torch on the host ---------------------------------------------
+@pytest.mark.parametrize("T,K,N", [(1, 8, 16), (5, 24, 40), (16, 32, 16), (17, 40, 100), (50, 1024, 4096), (50, 2048, 4096),
+                                   (200, 240, 4096), (200, 1024, 4096), (341, 240, 4096), (700, 64, 256)])
+def test_input_projection_matches_fp32_matmul(ops, T, K, N):
+    g = torch.Generator().manual_seed(T + K + N)
+    x = torch.randn(T, K, generator=g).half()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).half()
+    b = torch.randn(N, generator=g)
+    want = x.float() @ w.float().t() + b
+    out = ops.input_projection(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert out.dtype == torch.float32 and list(out.shape) == [T, N]
+    assert maxabs(out, want) <= 1e-4 * max(1.0, float(want.abs().max()))   # fp32 accumulation of exact fp16 products
+    out = ops.input_projection(x.to(DEV), w.to(DEV))
+    assert maxabs(out, want - b) <= 1e-4 * max(1.0, float(want.abs().max()))
