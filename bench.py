@@ -39,6 +39,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the LibTorch CPU timing")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="first run three out-of-place fp32 adds over 256 MiB (read 256 MiB, write 256 MiB each): "
+                         "a kernel of known traffic that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)", file=sys.stderr)
@@ -57,6 +60,14 @@ def main():
     lib = L.load()
     stream = torch.cuda.current_stream()
     sh = stream.cuda_stream
+
+    if args.calibration_copy:
+        src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- operands, resident in HBM ---------------------------------------------------------------------------
     g = torch.Generator(device=dev).manual_seed(2001)

@@ -61,6 +61,13 @@ __device__ __forceinline__ float wave_sum(float v)
 
 __device__ __forceinline__ float sigmoid_f32(float v) { return 1.0f / (1.0f + __expf(-v)); }
 
+// Sigmoid on the hardware exp2 and reciprocal (about 1 ulp each): exact limits 0 and 1 at -+inf, absolute error
+// below 1e-6, far inside the fp16 rounding of h.  Used where the activation sits on a latency-critical path.
+__device__ __forceinline__ float fast_sigmoid_f32(float v)
+{
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+}
+
 __device__ __forceinline__ float tanh_f32(float v)
 {
     // tanh(v) = 1 - 2 / (exp(2v) + 1); exact limits at +-inf, no cancellation near 0 beyond 1 ulp of 1.

@@ -118,86 +118,60 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 // Whole sequence, one (layer, direction).
 //
 // Grid: NB = ceil(H / 4) blocks of 256 lanes (H <= 1024, H % 8 == 0), all resident at once.  Block b owns
-// hidden units 4b .. 4b+3, i.e. 16 gate rows of W_hh, held in LDS as `slot = 4 * unit + gate` rows of H
-// halves.  Lane t of the block owns columns 4t .. 4t+3 of every row, which are exactly the four h values
-// block t produces.
+// hidden units 4b .. 4b+3, one per wavefront: wavefront w keeps the four gate rows of unit 4b+w in registers
+// for the whole sequence (lane l holds columns 16l .. 16l+15 of each row) and its cell state in a register.
 //
-// Exchange buffer: hx[2][NB][2] 64-bit words, word = (tag << 32) | two fp16 values.  Step s of a launch
-// publishes its h under tag `tag_base + s + 1` into parity s & 1; step s >= 1 waits until both words of
-// its entry in parity (s - 1) & 1 carry tag `tag_base + s`.  Data and flag travel in one word, written
-// and read with device-scope relaxed atomics (which go to memory past the per-XCD L2), so one store/load
-// round trip publishes a step.  A block cannot overwrite parity p before every block has consumed it:
-// writing step s + 2 needs h of step s + 1 from all blocks, which they publish only after reading step s.
-// The host advances tag_base by seq_len per launch, so tags left by earlier launches never match.
+// A step:
+//   1. lane t of the block (t < NB) obtains the four h values of block t from the exchange buffer (below)
+//      and puts them into LDS; one barrier; every wavefront reads the whole h from LDS;
+//   2. 4 rows x 16 columns of dot products per lane, a transpose-sum over the 64 lanes (7 exchanges) that
+//      leaves gate k in lane k, the four activations in parallel in lanes 0..3, the cell update;
+//   3. lane 0 of each wavefront publishes its h value and stores y.
+//
+// Exchange buffer: hx[2][NB][16] 32-bit words; block b uses words 0..3 of its 64-byte entry (one per unit;
+// entries of different blocks do not share a 64-byte segment, which measurably shortens the exchange).
+// word = fp16 bits | tag << 16.  Step s of a launch publishes under tag (tag_base + s + 1) & 0xffff into
+// parity s & 1; step s >= 1 waits until the four words of an entry in parity (s - 1) & 1 carry tag
+// (tag_base + s) & 0xffff.  Data and flag travel in one word, written and read with device-scope relaxed
+// atomics, so one store / load round trip through memory publishes a step.  A block cannot overwrite parity
+// p before every block has consumed it: publishing step s + 2 needs h of step s + 1 from all blocks, which
+// they publish only after reading step s.  The host advances tag_base by seq_len per launch (seq_len <=
+// 65000), so the tags left behind by earlier launches (at most tag_base) never equal an expected one.
 //
 // Every wait is bounded: after `spin_limit` polls a lane raises *abort_flag and stops waiting; lanes poll
 // the flag every 256 spins and stop waiting once it is set.  The kernel then runs to the end with
 // undefined results and the host reports a time-out.
 // ---------------------------------------------------------------------------------------------
-static constexpr int kSeqUnits = 4;   // hidden units per block
-static constexpr int kSeqRows = 16;   // gate rows per block
-static constexpr int kSeqMaxH = 1024; // 256 lanes x 4 columns
+static constexpr int kSeqUnits = 4;        // hidden units per block, one per wavefront
+static constexpr int kSeqMaxH = 1024;      // 64 lanes x 16 columns
+static constexpr int kSeqEntryWords = 16;  // 32-bit words between the entries of consecutive blocks (64 bytes)
+static constexpr int kSeqMaxT = 65000;
 
-// Exchange of a register with the lane whose index differs in bit 2 (xor 4) inside a row of 16 lanes.
-__device__ __forceinline__ float dpp_xor4_f32(float v)
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov_f32(float v)
 {
-    int iv = __builtin_bit_cast(int, v);
-    // row_ror:4 delivers lane i-4 (taken by lanes with bit 2 set: banks 1 and 3),
-    // row_ror:12 delivers lane i+4 (taken by lanes with bit 2 clear: banks 0 and 2).
-    int r = __builtin_amdgcn_update_dpp(0, iv, 0x124, 0xf, 0xA, false);
-    r = __builtin_amdgcn_update_dpp(r, iv, 0x12C, 0xf, 0x5, false);
-    return __builtin_bit_cast(float, r);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
 
-__device__ __forceinline__ float dpp_xor8_f32(float v)
+// Sum over all lanes that share (lane & 3); every lane receives the total of its class.
+__device__ __forceinline__ float wave_sum_mod4(float v)
 {
-    // row_ror:8 is the xor-8 exchange inside a row of 16 lanes.
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
-}
-
-__device__ __forceinline__ float dpp_xor1_f32(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kDppQuadXor1, 0xf, 0xf, false));
-}
-
-__device__ __forceinline__ float dpp_xor2_f32(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kDppQuadXor2, 0xf, 0xf, false));
-}
-
-// Sums 16 per-lane values over each row of 16 lanes so that lane r of the row ends up with the row total of
-// value index  8*bit0(r) + 4*bit1(r) + 2*bit3(r) + bit2(r).  15 exchanges instead of 64.
-__device__ __forceinline__ float row16_transpose_sum(const float (&v)[16], int lane)
-{
-    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4, b3 = lane & 8;
-    float a[8], b[4], c[2];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float keep = b0 ? v[i + 8] : v[i];
-        const float give = b0 ? v[i] : v[i + 8];
-        a[i] = keep + dpp_xor1_f32(give);
+    v += dpp_mov_f32<0x124>(v);  // row_ror:4
+    v += dpp_mov_f32<0x128>(v);  // row_ror:8  -> total over the four quads of a row of 16 lanes
+    // v_permlane16_swap a, b exchanges rows 1 and 3 of a with rows 0 and 2 of b; v_permlane32_swap a, b exchanges the
+    // upper 32 lanes of a with the lower 32 lanes of b.  With a == b == v on entry, a + b is the pairwise sum in
+    // every lane.  (Written as asm: the compiler's builtin returns the first result twice.)
+    {
+        float a = v, b = v;
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        v = a + b;
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float keep = b1 ? a[i + 4] : a[i];
-        const float give = b1 ? a[i] : a[i + 4];
-        b[i] = keep + dpp_xor2_f32(give);
+    {
+        float a = v, b = v;
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        v = a + b;
     }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const float keep = b3 ? b[i + 2] : b[i];
-        const float give = b3 ? b[i] : b[i + 2];
-        c[i] = keep + dpp_xor8_f32(give);
-    }
-    const float keep = b2 ? c[1] : c[0];
-    const float give = b2 ? c[0] : c[1];
-    return keep + dpp_xor4_f32(give);
-}
-
-// Value index held by lane r (0..15) of a row after row16_transpose_sum.
-__host__ __device__ constexpr int row16_value_index(int r)
-{
-    return 8 * (r & 1) + 4 * ((r >> 1) & 1) + 2 * ((r >> 3) & 1) + ((r >> 2) & 1);
+    return v;
 }
 
 struct LstmSeqArgs {
@@ -208,7 +182,7 @@ struct LstmSeqArgs {
     half_t* y;                // row t at y + t * y_stride
     half_t* hn;               // [H]
     half_t* cn;               // [H]
-    unsigned long long* hx;   // [2][NB][2]
+    unsigned int* hx;         // [2][NB][kSeqEntryWords]
     unsigned int* abort_flag; // set to 1 when a wait gives up
     long y_stride;            // elements between consecutive time steps of y
     int H;
@@ -220,72 +194,81 @@ struct LstmSeqArgs {
 
 __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
 {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    half_t* wl = reinterpret_cast<half_t*>(smem_raw);                        // [16][H]
-    float* red_base = reinterpret_cast<float*>(smem_raw + (size_t)kSeqRows * p.H * sizeof(half_t));  // [2][16 partials][16 slots]
+    __shared__ __align__(16) half_t hbuf[2][kSeqMaxH];  // h of the previous step, double buffered by step parity
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int H = p.H;
     const int nb = gridDim.x;
-    const int j0 = blockIdx.x * kSeqUnits;
+    const int j = blockIdx.x * kSeqUnits + wave;  // this wavefront's hidden unit
+    const bool unit_ok = j < H;
 
-    // ---- stage this block's 16 rows of W_hh into LDS (zero rows for units past H) ----
+    // ---- this wavefront's four gate rows, columns 16 * lane .. + 15, into registers ----
+    // Accumulator slot v holds gate {i, g, f, o}[v]: the transpose-sum below then leaves gate k in lane k.
+    half8_t w[4][2];
     {
-        const int chunks_per_row = H >> 3;
-        const int total = kSeqRows * chunks_per_row;
-        for (int i = tid; i < total; i += 256) {
-            const int slot = i / chunks_per_row;
-            const int cc = i - slot * chunks_per_row;
-            const int unit = slot >> 2, gate = slot & 3;
-            half8_t w;
+        const int gate_of_slot[4] = {0, 2, 1, 3};
 #pragma unroll
-            for (int e = 0; e < 8; ++e) w[e] = (half_t)0.0f;
-            if (j0 + unit < H) w = *reinterpret_cast<const half8_t*>(p.w_hh + ((long)gate * H + j0 + unit) * H + cc * 8);
-            *reinterpret_cast<half8_t*>(wl + (long)slot * H + cc * 8) = w;
+        for (int v = 0; v < 4; ++v) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int col = lane * 16 + c * 8;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) w[v][c][e] = (half_t)0.0f;
+                if (unit_ok && col < H)  // H % 8 == 0: an 8-wide chunk is entirely inside or outside the row
+                    w[v][c] = *reinterpret_cast<const half8_t*>(p.w_hh + ((long)gate_of_slot[v] * H + j) * H + col);
+            }
         }
+    }
+    // Columns at and past H stay zero in both h buffers for the whole kernel.
+    for (int i = tid; i < 2 * kSeqMaxH / 8; i += 256) {
+        half8_t z;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) z[e] = (half_t)0.0f;
+        reinterpret_cast<half8_t*>(&hbuf[0][0])[i] = z;
     }
     __syncthreads();
 
-    // Column ownership: lane t owns columns 4t..4t+3 <=> the h values of block t.
-    const bool has_cols = tid < nb;
-    // Final-stage roles (wave 0, lanes 0..15): lane v finishes slot v = 4 * unit + gate.
-    const int my_unit = (lane >> 2) & 3;
-    const int my_gate = lane & 3;
-    const bool unit_ok = (j0 + my_unit) < H;
-    float c_reg = 0.0f;
-    if (wave == 0 && lane < 16 && unit_ok) c_reg = (float)p.c0[j0 + my_unit];
-
+    const bool has_entry = tid < nb;            // lane t fetches the h values of block t
+    const int my_gate = lane & 3;               // role of lanes 0..3 after the transpose-sum
+    const bool gate_lane = lane < 4 && unit_ok;
+    float c_reg = gate_lane ? (float)p.c0[j] : 0.0f;
     bool gave_up = false;
-    const int row_in_wave = lane >> 4;                         // which row of 16 lanes
-    const int my_value = row16_value_index(lane & 15);         // slot this lane holds after the transpose-sum
 
-    for (int s = 0; s < p.T; ++s) {
+    // The input-projection term does not depend on h: it is fetched two steps ahead, into two registers that
+    // alternate between even and odd steps (the step loop is unrolled by two so that no copy of a pending
+    // load, and hence no wait for it, is needed at the loop's back edge).
+    // Every lane loads (lanes 4..63 repeat the addresses of lanes 0..3, units past H are clamped to H - 1 and
+    // steps past the end to the last step): an unconditional load keeps the two registers free of copies.
+    const float* xp_ptr = p.xproj + (long)my_gate * H + (unit_ok ? j : H - 1);
+    const long xp_step = p.reverse ? -(long)4 * H : (long)4 * H;
+    if (p.reverse) xp_ptr += (long)(p.T - 1) * 4 * H;
+    float xp_even = xp_ptr[0];
+    float xp_odd = xp_ptr[p.T > 1 ? xp_step : 0];
+
+    auto step = [&](const int s, float& xp_slot) __attribute__((always_inline)) {
         const int t = p.reverse ? (p.T - 1 - s) : s;
+        half_t* hb = hbuf[s & 1];
 
-        // Prefetch the input-projection term of this step (independent of h).
-        float xp = 0.0f;
-        if (wave == 0 && lane < 16 && unit_ok) xp = p.xproj[(long)t * 4 * H + (long)my_gate * H + j0 + my_unit];
-
-        // ---- obtain h_{s-1}: this lane's four columns ----
-        half4_t hv;
-        hv[0] = hv[1] = hv[2] = hv[3] = (half_t)0.0f;
-        if (has_cols) {
+        // ---- 1. h_{s-1} of block `tid` into LDS ----
+        if (has_entry) {
+            half4_t hv;
             if (s == 0) {
-                // H % 8 == 0, so a block's four units are either all valid or the entry ends at H.
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (tid * 4 + e < H) hv[e] = p.h0[tid * 4 + e];
+                for (int e = 0; e < 4; ++e) hv[e] = (tid * 4 + e < H) ? p.h0[tid * 4 + e] : (half_t)0.0f;
             } else {
-                const unsigned int want = p.tag_base + (unsigned int)s;
-                unsigned long long* src = p.hx + ((long)((s - 1) & 1) * nb + tid) * 2;
+                const unsigned int want = (p.tag_base + (unsigned int)s) & 0xffffu;
+                unsigned long long* src =
+                    reinterpret_cast<unsigned long long*>(p.hx + ((long)((s - 1) & 1) * nb + tid) * kSeqEntryWords);
                 unsigned long long w0 = 0, w1 = 0;
                 unsigned int spins = 0;
                 while (true) {
                     w0 = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     w1 = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (((unsigned int)(w0 >> 32) == want && (unsigned int)(w1 >> 32) == want) || gave_up) break;
+                    const bool ok = ((unsigned int)(w0 >> 16) & 0xffffu) == want && (unsigned int)(w0 >> 48) == want &&
+                                    ((unsigned int)(w1 >> 16) & 0xffffu) == want && (unsigned int)(w1 >> 48) == want;
+                    if (ok || gave_up) break;
                     ++spins;
                     if ((spins & 255u) == 0u) {
                         if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
@@ -295,73 +278,67 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
                         gave_up = true;
                     }
                 }
-                const unsigned int lo0 = (unsigned int)w0, lo1 = (unsigned int)w1;
-                const half2_t p0 = __builtin_bit_cast(half2_t, lo0);
-                const half2_t p1 = __builtin_bit_cast(half2_t, lo1);
-                hv[0] = p0[0];
-                hv[1] = p0[1];
-                hv[2] = p1[0];
-                hv[3] = p1[1];
+                hv[0] = __builtin_bit_cast(half_t, (unsigned short)(w0 & 0xffffu));
+                hv[1] = __builtin_bit_cast(half_t, (unsigned short)((w0 >> 32) & 0xffffu));
+                hv[2] = __builtin_bit_cast(half_t, (unsigned short)(w1 & 0xffffu));
+                hv[3] = __builtin_bit_cast(half_t, (unsigned short)((w1 >> 32) & 0xffffu));
             }
+            *reinterpret_cast<half4_t*>(hb + tid * 4) = hv;
         }
-
-        // ---- 16 partial dot products over this lane's 4 columns ----
-        float part[16];
-        {
-            const half_t* wrow = wl + tid * 4;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                half4_t w = has_cols ? *reinterpret_cast<const half4_t*>(wrow + (long)v * H) : hv;
-                part[v] = dot4(w, hv, 0.0f);
-            }
-        }
-
-        // ---- reduce over the 256 lanes: transpose-sum inside rows of 16, then LDS across the 16 rows ----
-        // `red` is double buffered by step parity: a wavefront that owns no columns does not wait for h and
-        // may already be writing step s + 1 while wave 0 still reads step s; the barrier below keeps it from
-        // getting further ahead than that.
-        float* red = red_base + (s & 1) * 256;
-        const float rowsum = row16_transpose_sum(part, lane);
-        red[(wave * 4 + row_in_wave) * 16 + my_value] = rowsum;
         __syncthreads();
 
-        if (wave == 0) {
-            float a = 0.0f;
-            if (lane < 16) {
-                float q[16];
+        // ---- 2. gates: 4 rows x 16 columns per lane, then over the wavefront ----
+        const half8_t ha = *reinterpret_cast<const half8_t*>(hb + lane * 16);
+        const half8_t hc = *reinterpret_cast<const half8_t*>(hb + lane * 16 + 8);
+        float acc[4];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) q[i] = red[i * 16 + lane];
-                a = (((q[0] + q[1]) + (q[2] + q[3])) + ((q[4] + q[5]) + (q[6] + q[7]))) +
-                    (((q[8] + q[9]) + (q[10] + q[11])) + ((q[12] + q[13]) + (q[14] + q[15])));
-                a += xp;
-            }
-            // Gather the four gates of a unit inside its quad (slot = 4 * unit + gate).
-            const int ai = __builtin_bit_cast(int, a);
-            const float a_i = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, ai, 0x00, 0xf, 0xf, false));
-            const float a_f = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, ai, 0x55, 0xf, 0xf, false));
-            const float a_g = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, ai, 0xAA, 0xf, 0xf, false));
-            const float a_o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, ai, 0xFF, 0xf, 0xf, false));
-            const float c_new = sigmoid_f32(a_f) * c_reg + sigmoid_f32(a_i) * tanh_f32(a_g);
-            const half_t h_new = (half_t)(sigmoid_f32(a_o) * tanh_f32(c_new));
-            c_reg = c_new;
-            // Lanes 4u (gate lane 0 of unit u) now hold h of unit u; fetch the neighbour unit's h for packing.
-            const unsigned int hbits = (unsigned int)__builtin_bit_cast(unsigned short, h_new);
-            const unsigned int hnext = (unsigned int)__builtin_amdgcn_update_dpp(0, (int)hbits, 0x104, 0xf, 0xf, true);  // row_shl:4 -> lane i+4
-            if (lane == 0 || lane == 8) {
-                const unsigned long long word =
-                    ((unsigned long long)(p.tag_base + (unsigned int)s + 1u) << 32) | (unsigned long long)(hbits | (hnext << 16));
-                unsigned long long* dst = p.hx + ((long)(s & 1) * nb + blockIdx.x) * 2 + (lane >> 3);
-                __hip_atomic_store(dst, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (lane < 16 && my_gate == 0 && unit_ok) {
-                p.y[(long)t * p.y_stride + j0 + my_unit] = h_new;
+        for (int v = 0; v < 4; ++v) acc[v] = dot8(w[v][1], hc, dot8(w[v][0], ha, 0.0f));
+
+        // Transpose-sum: after the two halving exchanges lane l holds slot 2 * (l & 1) + ((l >> 1) & 1) summed
+        // over its quad, i.e. gate (l & 3); wave_sum_mod4 then adds the 16 quads.
+        const bool b0 = lane & 1, b1 = lane & 2;
+        const float a0 = (b0 ? acc[2] : acc[0]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[0] : acc[2]);
+        const float a1 = (b0 ? acc[3] : acc[1]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[1] : acc[3]);
+        const float a = wave_sum_mod4((b1 ? a1 : a0) + dpp_mov_f32<kDppQuadXor2>(b1 ? a0 : a1)) + xp_slot;
+        // The term fetched two steps ago has been consumed: refill the same register for two steps ahead.  (Issued
+        // only now so that the old and the new value never live at once, which would cost a copy, and with it a
+        // wait for this load and for the stores below, at the loop's back edge.)
+        xp_slot = xp_ptr[(long)min(s + 2, p.T - 1) * xp_step];
+
+        // Each of lanes 0..3 activates its own gate: sigmoid for i, f, o and tanh(a) = 2 * sigmoid(2a) - 1 for g.
+        const bool is_g = my_gate == 2;
+        const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
+        const float act = is_g ? 2.0f * sg - 1.0f : sg;
+        const float g_i = dpp_mov_f32<0x00>(act);  // quad_perm broadcasts of lanes 0, 1, 2, 3 of the quad
+        const float g_f = dpp_mov_f32<0x55>(act);
+        const float g_g = dpp_mov_f32<0xAA>(act);
+        const float g_o = dpp_mov_f32<0xFF>(act);
+        const float c_new = g_f * c_reg + g_i * g_g;
+        const half_t h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
+        c_reg = c_new;
+
+        // ---- 3. publish ----
+        if (lane == 0) {
+            const unsigned int hbits = unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new) : 0u;
+            const unsigned int word = hbits | (((p.tag_base + (unsigned int)s + 1u) & 0xffffu) << 16);
+            __hip_atomic_store(p.hx + ((long)(s & 1) * nb + blockIdx.x) * kSeqEntryWords + wave, word, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            if (unit_ok) {
+                p.y[(long)t * p.y_stride + j] = h_new;
                 if (s == p.T - 1) {
-                    p.hn[j0 + my_unit] = h_new;
-                    p.cn[j0 + my_unit] = (half_t)c_new;
+                    p.hn[j] = h_new;
+                    p.cn[j] = (half_t)c_new;
                 }
             }
         }
+    };
+
+    int s = 0;
+    for (; s + 1 < p.T; s += 2) {
+        step(s, xp_even);
+        step(s + 1, xp_odd);
     }
+    if (s < p.T) step(s, xp_even);
 }
 
 }  // namespace pimhip

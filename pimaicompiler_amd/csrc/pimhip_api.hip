@@ -390,10 +390,9 @@ struct PimHipLstmPlan {
     float* xproj = nullptr;           // [num_dirs][max_seq_len][4H] fp32
     half_t* ybuf[2] = {nullptr, nullptr};  // inter-layer sequences [max_seq_len][num_dirs * H]
     float* c_state = nullptr;         // [num_dirs][H] fp32, per-step kernel's cell state
-    unsigned long long* hx = nullptr; // [num_dirs][2][NB][2] exchange words of the sequence kernel
+    unsigned int* hx = nullptr;       // [num_dirs][2][NB][kSeqEntryWords] exchange words of the sequence kernel
     unsigned int* abort_flag = nullptr;
     unsigned int* abort_host = nullptr;  // pinned copy read by pimhip_lstm_plan_status
-    size_t seq_lds_bytes = 0;
     int seq_blocks = 0;
 };
 
@@ -524,20 +523,19 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
     PLAN_HIP_CHECK(hipHostMalloc(&plan->abort_host, sizeof(unsigned int), hipHostMallocDefault));
     *plan->abort_host = 0;
 
-    // Persistent sequence kernel: 16 rows of W_hh per block in LDS, one block per 4 hidden units, all blocks
-    // resident at once.
+    // Persistent sequence kernel: one block per 4 hidden units (one unit per wavefront, weights in registers),
+    // all blocks resident at once.
     plan->seq_blocks = (int)((H + kSeqUnits - 1) / kSeqUnits);
-    plan->seq_lds_bytes = (size_t)kSeqRows * H * sizeof(half_t) + 2 * 256 * sizeof(float);
     plan->seq_kernel_ok = false;
-    if (H <= kSeqMaxH && plan->seq_lds_bytes <= 64 * 1024) {
+    if (H <= kSeqMaxH) {
         int per_cu = 0;
-        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_seq_f16_kernel, 256, plan->seq_lds_bytes));
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_seq_f16_kernel, 256, 0));
         plan->seq_kernel_ok = (int64_t)per_cu * plan->num_cus >= plan->seq_blocks;
     }
     if (plan->seq_kernel_ok) {
-        const size_t words = (size_t)D * 2 * plan->seq_blocks * 2;
-        PLAN_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned long long)));
-        PLAN_HIP_CHECK(hipMemsetAsync(plan->hx, 0, words * sizeof(unsigned long long), s));
+        const size_t words = (size_t)D * 2 * plan->seq_blocks * kSeqEntryWords;
+        PLAN_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned int)));
+        PLAN_HIP_CHECK(hipMemsetAsync(plan->hx, 0, words * sizeof(unsigned int), s));
     }
     PLAN_HIP_CHECK(hipStreamSynchronize(s));
 #undef PLAN_HIP_CHECK
@@ -623,7 +621,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 0u);
         *plan->abort_host = 0u;
     }
-    const bool use_seq = (plan->mode == 2) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2);
+    const bool use_seq = (plan->mode == 2 && T <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T <= kSeqMaxT);
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
     // seq_len == 1: fuse the input projection into the step (one launch per layer and direction).
     const bool fuse_xproj = !use_seq && T == 1;
@@ -656,7 +654,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                 a.y = yd;
                 a.hn = hnc;
                 a.cn = cnc;
-                a.hx = plan->hx + (size_t)d * 2 * plan->seq_blocks * 2;
+                a.hx = plan->hx + (size_t)d * 2 * plan->seq_blocks * kSeqEntryWords;
                 a.abort_flag = plan->abort_flag;
                 a.y_stride = y_stride;
                 a.H = (int)H;
@@ -665,7 +663,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                 a.tag_base = plan->tag_base;
                 a.spin_limit = plan->spin_limit;
                 plan->tag_base += (unsigned int)T;
-                lstm_seq_f16_kernel<<<plan->seq_blocks, 256, plan->seq_lds_bytes, s>>>(a);
+                lstm_seq_f16_kernel<<<plan->seq_blocks, 256, 0, s>>>(a);
             } else {
                 float* cst = plan->c_state + (size_t)d * H;
                 const unsigned grid = (unsigned)((H + 3) / 4);
