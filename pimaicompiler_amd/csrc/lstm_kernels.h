@@ -115,28 +115,39 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Whole sequence, one (layer, direction).
+// Whole sequences in one launch: NC recurrences ("chains") advance together, one super-step at a time.
+//
+// Two ways to combine chains (template parameter WAVEFRONT):
+//   WAVEFRONT = true   chain k is layer k of a unidirectional stack; at super-step tau it computes its time
+//                      step tau - k from h of layer k-1 at that time step (its input, multiplied by its W_ih
+//                      inside the kernel) and its own h of the step before.  Both were published at super-step
+//                      tau - 1, so NC layers cost T + NC - 1 exchanges instead of NC * T.  Only chain 0 takes a
+//                      precomputed input projection.
+//   WAVEFRONT = false  the chains are independent (the two directions of a bidirectional layer): every chain
+//                      takes its own precomputed input projection; chain k runs forward or backward in time.
 //
 // Grid: NB = ceil(H / 4) blocks of 256 lanes (H <= 1024, H % 8 == 0), all resident at once.  Block b owns
-// hidden units 4b .. 4b+3, one per wavefront: wavefront w keeps the four gate rows of unit 4b+w in registers
-// for the whole sequence (lane l holds columns 16l .. 16l+15 of each row) and its cell state in a register.
+// hidden units 4b .. 4b+3 of every chain, one unit per wavefront: wavefront w keeps, per chain, the four W_hh
+// gate rows of unit 4b+w (and the four W_ih rows for wavefront chains k > 0) in registers for the whole
+// launch (lane l holds columns 16l .. 16l+15 of each row) and the cell states in registers.
 //
-// A step:
-//   1. lane t of the block (t < NB) obtains the four h values of block t from the exchange buffer (below)
-//      and puts them into LDS; one barrier; every wavefront reads the whole h from LDS;
-//   2. 4 rows x 16 columns of dot products per lane, a transpose-sum over the 64 lanes (7 exchanges) that
-//      leaves gate k in lane k, the four activations in parallel in lanes 0..3, the cell update;
-//   3. lane 0 of each wavefront publishes its h value and stores y.
+// A super-step:
+//   1. lane t of the block (t < NB) obtains the h values block t published at the previous super-step (four
+//      per chain) from the exchange buffer and puts them into LDS; one barrier; every wavefront reads h from LDS;
+//   2. per chain: 4 rows x 16 columns of dot products per lane (twice that with W_ih), a transpose-sum over
+//      the 64 lanes (6 exchanges) that leaves gate k in lane k, the four activations in parallel in lanes 0..3,
+//      the cell update;
+//   3. lane 0 of each wavefront publishes its h values of all chains with one store per 8 bytes, and stores y.
 //
-// Exchange buffer: hx[2][NB][16] 32-bit words; block b uses words 0..3 of its 64-byte entry (one per unit;
-// entries of different blocks do not share a 64-byte segment, which measurably shortens the exchange).
-// word = fp16 bits | tag << 16.  Step s of a launch publishes under tag (tag_base + s + 1) & 0xffff into
-// parity s & 1; step s >= 1 waits until the four words of an entry in parity (s - 1) & 1 carry tag
-// (tag_base + s) & 0xffff.  Data and flag travel in one word, written and read with device-scope relaxed
-// atomics, so one store / load round trip through memory publishes a step.  A block cannot overwrite parity
-// p before every block has consumed it: publishing step s + 2 needs h of step s + 1 from all blocks, which
-// they publish only after reading step s.  The host advances tag_base by seq_len per launch (seq_len <=
-// 65000), so the tags left behind by earlier launches (at most tag_base) never equal an expected one.
+// Exchange buffer: hx[2][NB][16] 32-bit words; block b uses words [w * NC + k] (wavefront w, chain k) of its
+// 64-byte entry (entries of different blocks do not share a 64-byte segment, which measurably shortens the
+// exchange).  word = fp16 bits | tag << 16.  Super-step tau publishes under tag (tag_base + tau + 1) & 0xffff
+// into parity tau & 1; super-step tau >= 1 waits until all 4 * NC words of an entry in parity (tau - 1) & 1
+// carry tag (tag_base + tau) & 0xffff.  Data and flag travel in one word, written and read with device-scope
+// relaxed atomics, so one store / load round trip through memory publishes a super-step.  A block cannot
+// overwrite parity p before every block has consumed it: publishing super-step tau + 2 needs the words of
+// tau + 1 from all blocks, which they publish only after reading tau.  The host advances tag_base by the
+// number of super-steps per launch (at most 65000), so tags left by earlier launches never equal an expected one.
 //
 // Every wait is bounded: after `spin_limit` polls a lane raises *abort_flag and stops waiting; lanes poll
 // the flag every 256 spins and stop waiting once it is set.  The kernel then runs to the end with
@@ -145,7 +156,8 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 static constexpr int kSeqUnits = 4;        // hidden units per block, one per wavefront
 static constexpr int kSeqMaxH = 1024;      // 64 lanes x 16 columns
 static constexpr int kSeqEntryWords = 16;  // 32-bit words between the entries of consecutive blocks (64 bytes)
-static constexpr int kSeqMaxT = 65000;
+static constexpr int kSeqMaxT = 65000;       // super-steps per launch
+static constexpr int kSeqMaxChains = 4;
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_mov_f32(float v)
@@ -174,100 +186,127 @@ __device__ __forceinline__ float wave_sum_mod4(float v)
     return v;
 }
 
+struct LstmSeqChain {
+    const half_t* w_hh;   // [4H, H]
+    const half_t* w_ih;   // [4H, H]: wavefront chains k > 0 only
+    const float* xproj;   // [T, 4H] fp32 with biases: chain 0, and every chain when not in wavefront mode
+    const float* bsum;    // [4H] fp32 b_ih + b_hh: wavefront chains k > 0 only
+    const half_t* h0;     // [H]
+    const half_t* c0;     // [H]
+    half_t* y;            // row t at y + t * y_stride; may be null (inner layers of a wavefront)
+    half_t* hn;           // [H]
+    half_t* cn;           // [H]
+    int reverse;          // 1: this chain processes t = T-1 .. 0 (not in wavefront mode)
+};
+
 struct LstmSeqArgs {
-    const half_t* w_hh;       // [4H, H]
-    const float* xproj;       // [T, 4H] fp32, biases included
-    const half_t* h0;         // [H]
-    const half_t* c0;         // [H]
-    half_t* y;                // row t at y + t * y_stride
-    half_t* hn;               // [H]
-    half_t* cn;               // [H]
-    unsigned int* hx;         // [2][NB][kSeqEntryWords]
-    unsigned int* abort_flag; // set to 1 when a wait gives up
-    long y_stride;            // elements between consecutive time steps of y
+    LstmSeqChain chain[kSeqMaxChains];
+    unsigned int* hx;          // [2][NB][kSeqEntryWords]
+    unsigned int* abort_flag;  // set to 1 when a wait gives up
+    long y_stride;             // elements between consecutive time steps of y
     int H;
     int T;
-    int reverse;              // 1: process t = T-1 .. 0
     unsigned int tag_base;
     unsigned int spin_limit;
 };
 
+template <int NC, bool WAVEFRONT>
 __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
 {
-    __shared__ __align__(16) half_t hbuf[2][kSeqMaxH];  // h of the previous step, double buffered by step parity
+    static_assert(NC >= 1 && NC <= kSeqMaxChains && 4 * NC <= kSeqEntryWords, "entry holds 4 words per chain");
+    __shared__ __align__(16) half_t hbuf[2][NC][kSeqMaxH];  // published h per chain, double buffered by parity
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int H = p.H;
+    const int T = p.T;
     const int nb = gridDim.x;
     const int j = blockIdx.x * kSeqUnits + wave;  // this wavefront's hidden unit
     const bool unit_ok = j < H;
+    const int n_super = WAVEFRONT ? T + NC - 1 : T;
 
-    // ---- this wavefront's four gate rows, columns 16 * lane .. + 15, into registers ----
+    // ---- weights into registers: per chain the four gate rows of unit j, columns 16 * lane .. + 15 ----
     // Accumulator slot v holds gate {i, g, f, o}[v]: the transpose-sum below then leaves gate k in lane k.
-    half8_t w[4][2];
+    half8_t w_hh[NC][4][2];
+    half8_t w_ih[WAVEFRONT ? NC : 1][4][2];  // entry 0 unused
     {
         const int gate_of_slot[4] = {0, 2, 1, 3};
+        half8_t zero;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
+        for (int e = 0; e < 8; ++e) zero[e] = (half_t)0.0f;
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const int col = lane * 16 + c * 8;
+        for (int k = 0; k < NC; ++k) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) w[v][c][e] = (half_t)0.0f;
-                if (unit_ok && col < H)  // H % 8 == 0: an 8-wide chunk is entirely inside or outside the row
-                    w[v][c] = *reinterpret_cast<const half8_t*>(p.w_hh + ((long)gate_of_slot[v] * H + j) * H + col);
+            for (int v = 0; v < 4; ++v) {
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const int col = lane * 16 + c * 8;
+                    const bool ok = unit_ok && col < H;  // H % 8 == 0: a chunk is entirely inside or outside the row
+                    const long off = ((long)gate_of_slot[v] * H + j) * H + col;
+                    w_hh[k][v][c] = ok ? *reinterpret_cast<const half8_t*>(p.chain[k].w_hh + off) : zero;
+                    if (WAVEFRONT && k > 0) w_ih[k][v][c] = ok ? *reinterpret_cast<const half8_t*>(p.chain[k].w_ih + off) : zero;
+                }
             }
         }
-    }
-    // Columns at and past H stay zero in both h buffers for the whole kernel.
-    for (int i = tid; i < 2 * kSeqMaxH / 8; i += 256) {
-        half8_t z;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) z[e] = (half_t)0.0f;
-        reinterpret_cast<half8_t*>(&hbuf[0][0])[i] = z;
+        // Columns at and past H stay zero in all h buffers for the whole kernel.
+        for (int i = tid; i < 2 * NC * kSeqMaxH / 8; i += 256) reinterpret_cast<half8_t*>(&hbuf[0][0][0])[i] = zero;
     }
     __syncthreads();
 
-    const bool has_entry = tid < nb;            // lane t fetches the h values of block t
-    const int my_gate = lane & 3;               // role of lanes 0..3 after the transpose-sum
-    const bool gate_lane = lane < 4 && unit_ok;
-    float c_reg = gate_lane ? (float)p.c0[j] : 0.0f;
+    const bool has_entry = tid < nb;  // lane t fetches what block t published
+    const int my_gate = lane & 3;     // role of lanes 0..3 after the transpose-sum
+    const int jc = unit_ok ? j : H - 1;
+    float c_reg[NC];
+    float bias_reg[NC];               // wavefront chains k > 0: b_ih + b_hh of (gate my_gate, unit j)
+    const float* xp_ptr[NC];
+    long xp_step[NC];
+    float xp_even[NC], xp_odd[NC];
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+        c_reg[k] = (float)p.chain[k].c0[jc];
+        bias_reg[k] = 0.0f;
+        xp_ptr[k] = nullptr;
+        xp_step[k] = 0;
+        xp_even[k] = xp_odd[k] = 0.0f;
+        if (WAVEFRONT && k > 0) {
+            bias_reg[k] = p.chain[k].bsum[(long)my_gate * H + jc];
+        } else {
+            // The input-projection term does not depend on h: it is fetched two steps ahead into two registers
+            // that alternate between even and odd steps (the loop is unrolled by two).  Every lane loads (lanes
+            // 4..63 repeat the addresses of lanes 0..3; steps past the end are clamped to the last one): an
+            // unconditional load keeps the registers free of copies, and with them of waits at the back edge.
+            const bool rev = p.chain[k].reverse != 0;
+            xp_ptr[k] = p.chain[k].xproj + (long)my_gate * H + jc + (rev ? (long)(T - 1) * 4 * H : 0);
+            xp_step[k] = rev ? -(long)4 * H : (long)4 * H;
+            xp_even[k] = xp_ptr[k][0];
+            xp_odd[k] = xp_ptr[k][T > 1 ? xp_step[k] : 0];
+        }
+    }
     bool gave_up = false;
 
-    // The input-projection term does not depend on h: it is fetched two steps ahead, into two registers that
-    // alternate between even and odd steps (the step loop is unrolled by two so that no copy of a pending
-    // load, and hence no wait for it, is needed at the loop's back edge).
-    // Every lane loads (lanes 4..63 repeat the addresses of lanes 0..3, units past H are clamped to H - 1 and
-    // steps past the end to the last step): an unconditional load keeps the two registers free of copies.
-    const float* xp_ptr = p.xproj + (long)my_gate * H + (unit_ok ? j : H - 1);
-    const long xp_step = p.reverse ? -(long)4 * H : (long)4 * H;
-    if (p.reverse) xp_ptr += (long)(p.T - 1) * 4 * H;
-    float xp_even = xp_ptr[0];
-    float xp_odd = xp_ptr[p.T > 1 ? xp_step : 0];
+    auto super_step = [&](const int tau, float (&xp_slot)[NC]) __attribute__((always_inline)) {
+        half_t(*hb)[kSeqMaxH] = hbuf[tau & 1];
 
-    auto step = [&](const int s, float& xp_slot) __attribute__((always_inline)) {
-        const int t = p.reverse ? (p.T - 1 - s) : s;
-        half_t* hb = hbuf[s & 1];
-
-        // ---- 1. h_{s-1} of block `tid` into LDS ----
+        // ---- 1. what block `tid` published at super-step tau - 1 (or the initial state) into LDS ----
         if (has_entry) {
-            half4_t hv;
-            if (s == 0) {
+            unsigned int words[4 * NC];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) hv[e] = (tid * 4 + e < H) ? p.h0[tid * 4 + e] : (half_t)0.0f;
-            } else {
-                const unsigned int want = (p.tag_base + (unsigned int)s) & 0xffffu;
+            for (int i = 0; i < 4 * NC; ++i) words[i] = 0u;
+            if (tau > 0) {
+                const unsigned int want = (p.tag_base + (unsigned int)tau) & 0xffffu;
                 unsigned long long* src =
-                    reinterpret_cast<unsigned long long*>(p.hx + ((long)((s - 1) & 1) * nb + tid) * kSeqEntryWords);
-                unsigned long long w0 = 0, w1 = 0;
+                    reinterpret_cast<unsigned long long*>(p.hx + ((long)((tau - 1) & 1) * nb + tid) * kSeqEntryWords);
                 unsigned int spins = 0;
                 while (true) {
-                    w0 = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    w1 = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    const bool ok = ((unsigned int)(w0 >> 16) & 0xffffu) == want && (unsigned int)(w0 >> 48) == want &&
-                                    ((unsigned int)(w1 >> 16) & 0xffffu) == want && (unsigned int)(w1 >> 48) == want;
+                    bool ok = true;
+#pragma unroll
+                    for (int i = 0; i < 2 * NC; ++i) {
+                        const unsigned long long q = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        words[2 * i] = (unsigned int)q;
+                        words[2 * i + 1] = (unsigned int)(q >> 32);
+                        ok = ok && (words[2 * i] >> 16) == want && (words[2 * i + 1] >> 16) == want;
+                    }
                     if (ok || gave_up) break;
                     ++spins;
                     if ((spins & 255u) == 0u) {
@@ -278,67 +317,112 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
                         gave_up = true;
                     }
                 }
-                hv[0] = __builtin_bit_cast(half_t, (unsigned short)(w0 & 0xffffu));
-                hv[1] = __builtin_bit_cast(half_t, (unsigned short)((w0 >> 32) & 0xffffu));
-                hv[2] = __builtin_bit_cast(half_t, (unsigned short)(w1 & 0xffffu));
-                hv[3] = __builtin_bit_cast(half_t, (unsigned short)((w1 >> 32) & 0xffffu));
             }
-            *reinterpret_cast<half4_t*>(hb + tid * 4) = hv;
+#pragma unroll
+            for (int k = 0; k < NC; ++k) {
+                const int s_k = WAVEFRONT ? tau - k : tau;  // the time step chain k computes now
+                half4_t hv;
+                if (s_k == 0) {
+                    // First step of this chain: its previous h is the caller's initial state.
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) hv[e] = (tid * 4 + e < H) ? p.chain[k].h0[tid * 4 + e] : (half_t)0.0f;
+                } else {
+                    // words[w * NC + k] is unit w of chain k in block `tid`.
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) hv[e] = __builtin_bit_cast(half_t, (unsigned short)(words[e * NC + k] & 0xffffu));
+                }
+                *reinterpret_cast<half4_t*>(&hb[k][tid * 4]) = hv;
+            }
         }
         __syncthreads();
 
-        // ---- 2. gates: 4 rows x 16 columns per lane, then over the wavefront ----
-        const half8_t ha = *reinterpret_cast<const half8_t*>(hb + lane * 16);
-        const half8_t hc = *reinterpret_cast<const half8_t*>(hb + lane * 16 + 8);
-        float acc[4];
+        // ---- 2. gates per chain ----
+        half_t h_new[NC];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) acc[v] = dot8(w[v][1], hc, dot8(w[v][0], ha, 0.0f));
+        for (int k = 0; k < NC; ++k) {
+            const int s_k = WAVEFRONT ? tau - k : tau;
+            h_new[k] = (half_t)0.0f;
+            if (s_k < 0 || s_k >= T) continue;  // uniform: this chain has not started yet, or has finished
 
-        // Transpose-sum: after the two halving exchanges lane l holds slot 2 * (l & 1) + ((l >> 1) & 1) summed
-        // over its quad, i.e. gate (l & 3); wave_sum_mod4 then adds the 16 quads.
-        const bool b0 = lane & 1, b1 = lane & 2;
-        const float a0 = (b0 ? acc[2] : acc[0]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[0] : acc[2]);
-        const float a1 = (b0 ? acc[3] : acc[1]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[1] : acc[3]);
-        const float a = wave_sum_mod4((b1 ? a1 : a0) + dpp_mov_f32<kDppQuadXor2>(b1 ? a0 : a1)) + xp_slot;
-        // The term fetched two steps ago has been consumed: refill the same register for two steps ahead.  (Issued
-        // only now so that the old and the new value never live at once, which would cost a copy, and with it a
-        // wait for this load and for the stores below, at the loop's back edge.)
-        xp_slot = xp_ptr[(long)min(s + 2, p.T - 1) * xp_step];
+            const half8_t ha = *reinterpret_cast<const half8_t*>(&hb[k][lane * 16]);
+            const half8_t hc = *reinterpret_cast<const half8_t*>(&hb[k][lane * 16 + 8]);
+            float acc[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[v] = dot8(w_hh[k][v][1], hc, dot8(w_hh[k][v][0], ha, 0.0f));
+            if (WAVEFRONT && k > 0) {
+                // Input of layer k at this time step: h of layer k - 1 at the same time step, published one
+                // super-step ago.  At s_k == 0 chain k - 1's buffer holds exactly that (its s = 1 input).
+                const half8_t xa = *reinterpret_cast<const half8_t*>(&hb[k - 1][lane * 16]);
+                const half8_t xc = *reinterpret_cast<const half8_t*>(&hb[k - 1][lane * 16 + 8]);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[v] = dot8(w_ih[k][v][1], xc, dot8(w_ih[k][v][0], xa, acc[v]));
+            }
 
-        // Each of lanes 0..3 activates its own gate: sigmoid for i, f, o and tanh(a) = 2 * sigmoid(2a) - 1 for g.
-        const bool is_g = my_gate == 2;
-        const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
-        const float act = is_g ? 2.0f * sg - 1.0f : sg;
-        const float g_i = dpp_mov_f32<0x00>(act);  // quad_perm broadcasts of lanes 0, 1, 2, 3 of the quad
-        const float g_f = dpp_mov_f32<0x55>(act);
-        const float g_g = dpp_mov_f32<0xAA>(act);
-        const float g_o = dpp_mov_f32<0xFF>(act);
-        const float c_new = g_f * c_reg + g_i * g_g;
-        const half_t h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
-        c_reg = c_new;
+            // Transpose-sum: after the two halving exchanges lane l holds slot 2 * (l & 1) + ((l >> 1) & 1) summed
+            // over its quad, i.e. gate (l & 3); wave_sum_mod4 then adds the 16 quads.
+            const bool b0 = lane & 1, b1 = lane & 2;
+            const float a0 = (b0 ? acc[2] : acc[0]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[0] : acc[2]);
+            const float a1 = (b0 ? acc[3] : acc[1]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[1] : acc[3]);
+            float a = wave_sum_mod4((b1 ? a1 : a0) + dpp_mov_f32<kDppQuadXor2>(b1 ? a0 : a1));
+            if (WAVEFRONT && k > 0) {
+                a += bias_reg[k];
+            } else {
+                a += xp_slot[k];
+                // The term fetched two steps ago has been consumed: refill the same register for two steps ahead.
+                // (Issued only now so that the old and the new value never live at once, which would cost a copy,
+                // and with it a wait for this load and for the stores below, at the loop's back edge.)
+                xp_slot[k] = xp_ptr[k][(long)min(s_k + 2, T - 1) * xp_step[k]];
+            }
 
-        // ---- 3. publish ----
-        if (lane == 0) {
-            const unsigned int hbits = unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new) : 0u;
-            const unsigned int word = hbits | (((p.tag_base + (unsigned int)s + 1u) & 0xffffu) << 16);
-            __hip_atomic_store(p.hx + ((long)(s & 1) * nb + blockIdx.x) * kSeqEntryWords + wave, word, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-            if (unit_ok) {
-                p.y[(long)t * p.y_stride + j] = h_new;
-                if (s == p.T - 1) {
-                    p.hn[j] = h_new;
-                    p.cn[j] = (half_t)c_new;
+            // Each of lanes 0..3 activates its own gate: sigmoid for i, f, o and tanh(a) = 2 * sigmoid(2a) - 1 for g.
+            const bool is_g = my_gate == 2;
+            const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
+            const float act = is_g ? 2.0f * sg - 1.0f : sg;
+            const float g_i = dpp_mov_f32<0x00>(act);  // quad_perm broadcasts of lanes 0, 1, 2, 3 of the quad
+            const float g_f = dpp_mov_f32<0x55>(act);
+            const float g_g = dpp_mov_f32<0xAA>(act);
+            const float g_o = dpp_mov_f32<0xFF>(act);
+            const float c_new = g_f * c_reg[k] + g_i * g_g;
+            h_new[k] = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
+            c_reg[k] = c_new;
+
+            if (lane == 0 && unit_ok) {
+                const int t = p.chain[k].reverse ? (T - 1 - s_k) : s_k;
+                if (p.chain[k].y) p.chain[k].y[(long)t * p.y_stride + j] = h_new[k];
+                if (s_k == T - 1) {
+                    p.chain[k].hn[j] = h_new[k];
+                    p.chain[k].cn[j] = (half_t)c_new;
                 }
+            }
+        }
+
+        // ---- 3. publish: words [wave * NC + k] of this block's entry, 8 bytes per store where possible ----
+        if (lane == 0) {
+            const unsigned int tag = ((p.tag_base + (unsigned int)tau + 1u) & 0xffffu) << 16;
+            unsigned int* dst = p.hx + ((long)(tau & 1) * nb + blockIdx.x) * kSeqEntryWords + wave * NC;
+            unsigned int word[NC];
+#pragma unroll
+            for (int k = 0; k < NC; ++k)
+                word[k] = (unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new[k]) : 0u) | tag;
+            if (NC % 2 == 0) {
+#pragma unroll
+                for (int k = 0; k < NC; k += 2)
+                    __hip_atomic_store(reinterpret_cast<unsigned long long*>(dst + k),
+                                       (unsigned long long)word[k] | ((unsigned long long)word[k + 1] << 32), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+#pragma unroll
+                for (int k = 0; k < NC; ++k) __hip_atomic_store(dst + k, word[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     };
 
-    int s = 0;
-    for (; s + 1 < p.T; s += 2) {
-        step(s, xp_even);
-        step(s + 1, xp_odd);
+    int tau = 0;
+    for (; tau + 1 < n_super; tau += 2) {
+        super_step(tau, xp_even);
+        super_step(tau + 1, xp_odd);
     }
-    if (s < p.T) step(s, xp_even);
+    if (tau < n_super) super_step(tau, xp_even);
 }
 
 }  // namespace pimhip

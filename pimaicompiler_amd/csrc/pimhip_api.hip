@@ -375,6 +375,7 @@ struct PimHipLstmPlan {
     bool seq_kernel_ok = false;      // shape fits the persistent sequence kernel
     unsigned int spin_limit = 1u << 22;
     unsigned int tag_base = 0;
+    int max_wavefront = kSeqMaxChains;  // layers of a unidirectional stack advanced by one persistent launch
 
     struct Cell {
         const half_t* w_ih = nullptr;
@@ -529,11 +530,11 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
     plan->seq_kernel_ok = false;
     if (H <= kSeqMaxH) {
         int per_cu = 0;
-        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_seq_f16_kernel, 256, 0));
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_seq_f16_kernel<kSeqMaxChains, true>, 256, 0));
         plan->seq_kernel_ok = (int64_t)per_cu * plan->num_cus >= plan->seq_blocks;
     }
     if (plan->seq_kernel_ok) {
-        const size_t words = (size_t)D * 2 * plan->seq_blocks * kSeqEntryWords;
+        const size_t words = (size_t)2 * plan->seq_blocks * kSeqEntryWords;
         PLAN_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned int)));
         PLAN_HIP_CHECK(hipMemsetAsync(plan->hx, 0, words * sizeof(unsigned int), s));
     }
@@ -621,50 +622,86 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 0u);
         *plan->abort_host = 0u;
     }
-    const bool use_seq = (plan->mode == 2 && T <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T <= kSeqMaxT);
+    const bool use_seq = (plan->mode == 2 && T + kSeqMaxChains <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T + kSeqMaxChains <= kSeqMaxT);
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
     // seq_len == 1: fuse the input projection into the step (one launch per layer and direction).
     const bool fuse_xproj = !use_seq && T == 1;
 
     const half_t* layer_in = (const half_t*)x;
-    for (int l = 0; l < L; ++l) {
-        half_t* layer_out = (l == L - 1) ? (half_t*)y : plan->ybuf[l & 1];
-        const int64_t in_w = plan->cells[(size_t)l * D].in_w;
-        for (int d = 0; d < D; ++d) {
-            const int ci = l * D + d;
-            const PimHipLstmPlan::Cell& c = plan->cells[ci];
-            float* xp = plan->xproj + (size_t)d * plan->max_seq_len * 4 * H;
-            half_t* yd = layer_out + (size_t)d * H;
-            const long y_stride = (long)D * H;
-            const half_t* h0c = h0p + (size_t)ci * H;
-            const half_t* c0c = c0p + (size_t)ci * H;
-            half_t* hnc = hnp + (size_t)ci * H;
-            half_t* cnc = cnp + (size_t)ci * H;
-
-            if (!fuse_xproj) {
-                rc = launch_input_projection(xp, layer_in, c.w_ih, c.bsum, T, in_w, 4 * H, s);
-                if (rc != PIMHIP_OK) return rc;
+    const long y_stride = (long)D * H;
+    if (use_seq) {
+        // Layers are taken in groups that one persistent launch advances together: the two directions of a
+        // bidirectional layer, or up to kSeqMaxChains consecutive layers of a unidirectional stack as a wavefront.
+        int l = 0;
+        while (l < L) {
+            const int group_layers = (D == 2) ? 1 : ((L - l) < plan->max_wavefront ? (L - l) : plan->max_wavefront);
+            const int nc = (D == 2) ? 2 : group_layers;
+            const int last = l + group_layers - 1;
+            half_t* group_out = (last == L - 1) ? (half_t*)y : plan->ybuf[last & 1];
+            const int64_t in_w = plan->cells[(size_t)l * D].in_w;
+            LstmSeqArgs a;
+            memset(&a, 0, sizeof(a));
+            for (int k = 0; k < nc; ++k) {
+                const int ci = (D == 2) ? (l * D + k) : (l + k);
+                const PimHipLstmPlan::Cell& c = plan->cells[ci];
+                LstmSeqChain& ch = a.chain[k];
+                ch.w_hh = c.w_hh;
+                ch.h0 = h0p + (size_t)ci * H;
+                ch.c0 = c0p + (size_t)ci * H;
+                ch.hn = hnp + (size_t)ci * H;
+                ch.cn = cnp + (size_t)ci * H;
+                if (D == 2 || k == 0) {
+                    float* xp = plan->xproj + (size_t)((D == 2) ? k : 0) * plan->max_seq_len * 4 * H;
+                    rc = launch_input_projection(xp, layer_in, c.w_ih, c.bsum, T, in_w, 4 * H, s);
+                    if (rc != PIMHIP_OK) return rc;
+                    ch.xproj = xp;
+                } else {
+                    ch.w_ih = c.w_ih;
+                    ch.bsum = c.bsum;
+                }
+                ch.reverse = (D == 2) ? k : 0;
+                ch.y = (D == 2) ? group_out + (size_t)k * H : ((k == nc - 1) ? group_out : nullptr);
             }
-            if (use_seq) {
-                LstmSeqArgs a;
-                a.w_hh = c.w_hh;
-                a.xproj = xp;
-                a.h0 = h0c;
-                a.c0 = c0c;
-                a.y = yd;
-                a.hn = hnc;
-                a.cn = cnc;
-                a.hx = plan->hx + (size_t)d * 2 * plan->seq_blocks * kSeqEntryWords;
-                a.abort_flag = plan->abort_flag;
-                a.y_stride = y_stride;
-                a.H = (int)H;
-                a.T = (int)T;
-                a.reverse = d;
-                a.tag_base = plan->tag_base;
-                a.spin_limit = plan->spin_limit;
-                plan->tag_base += (unsigned int)T;
-                lstm_seq_f16_kernel<<<plan->seq_blocks, 256, 0, s>>>(a);
+            a.hx = plan->hx;
+            a.abort_flag = plan->abort_flag;
+            a.y_stride = y_stride;
+            a.H = (int)H;
+            a.T = (int)T;
+            a.tag_base = plan->tag_base;
+            a.spin_limit = plan->spin_limit;
+            plan->tag_base += (unsigned int)((D == 2) ? T : T + nc - 1);
+            const dim3 grid(plan->seq_blocks), block(256);
+            if (D == 2) {
+                lstm_seq_f16_kernel<2, false><<<grid, block, 0, s>>>(a);
             } else {
+                switch (nc) {
+                    case 1: lstm_seq_f16_kernel<1, true><<<grid, block, 0, s>>>(a); break;
+                    case 2: lstm_seq_f16_kernel<2, true><<<grid, block, 0, s>>>(a); break;
+                    case 3: lstm_seq_f16_kernel<3, true><<<grid, block, 0, s>>>(a); break;
+                    default: lstm_seq_f16_kernel<4, true><<<grid, block, 0, s>>>(a); break;
+                }
+            }
+            PIMHIP_HIP_CHECK(hipGetLastError());
+            layer_in = group_out;
+            l += group_layers;
+        }
+    } else {
+        for (int l = 0; l < L; ++l) {
+            half_t* layer_out = (l == L - 1) ? (half_t*)y : plan->ybuf[l & 1];
+            const int64_t in_w = plan->cells[(size_t)l * D].in_w;
+            for (int d = 0; d < D; ++d) {
+                const int ci = l * D + d;
+                const PimHipLstmPlan::Cell& c = plan->cells[ci];
+                float* xp = plan->xproj + (size_t)d * plan->max_seq_len * 4 * H;
+                half_t* yd = layer_out + (size_t)d * H;
+                const half_t* h0c = h0p + (size_t)ci * H;
+                const half_t* c0c = c0p + (size_t)ci * H;
+                half_t* hnc = hnp + (size_t)ci * H;
+                half_t* cnc = cnp + (size_t)ci * H;
+                if (!fuse_xproj) {
+                    rc = launch_input_projection(xp, layer_in, c.w_ih, c.bsum, T, in_w, 4 * H, s);
+                    if (rc != PIMHIP_OK) return rc;
+                }
                 float* cst = plan->c_state + (size_t)d * H;
                 const unsigned grid = (unsigned)((H + 3) / 4);
                 for (int64_t step = 0; step < T; ++step) {
@@ -677,10 +714,10 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                         (step == 0) ? c0c : nullptr, cst, yd + t * y_stride, last ? hnc : nullptr, last ? cnc : nullptr,
                         (int)in_w, (int)H);
                 }
+                PIMHIP_HIP_CHECK(hipGetLastError());
             }
-            PIMHIP_HIP_CHECK(hipGetLastError());
+            layer_in = layer_out;
         }
-        layer_in = layer_out;
     }
     if (use_seq)
         PIMHIP_HIP_CHECK(hipMemcpyAsync(plan->abort_host, plan->abort_flag, sizeof(unsigned int), hipMemcpyDeviceToHost, s));

@@ -54,6 +54,8 @@ CASES = [  # I, H, L, bidirectional, T, biases
     (8, 8, 1, False, 1, True), (8, 8, 1, False, 2, True), (24, 40, 1, False, 9, True), (64, 320, 1, False, 13, True),
     (16, 72, 2, True, 6, True), (32, 128, 3, False, 5, False), (32, 128, 3, True, 4, True), (240, 512, 2, False, 17, True),
     (8, 1024, 1, False, 3, True), (40, 1032, 1, False, 3, True), (16, 2048, 1, True, 2, False),
+    (16, 64, 4, False, 7, True), (16, 64, 5, False, 6, True), (24, 136, 7, False, 3, False), (16, 64, 4, False, 1, True),
+    (16, 64, 2, False, 2, True), (32, 1024, 4, False, 5, True),
 ]
 
 
@@ -204,8 +206,10 @@ def test_lstm_bidirectional_equals_forward_on_reversed_input(ops):
     y, hn, cn = run_plan(ops, params, x, h0, c0, True, 1, True, 2)
     yf, hf, cf = run_plan(ops, params[:4], x, h0[:1], c0[:1], True, 1, False, 2)
     yb, hb, cb = run_plan(ops, params[4:], x.flip(0), h0[1:], c0[1:], True, 1, False, 2)
-    assert torch.equal(y[:, :1024], yf) and torch.equal(y[:, 1024:], yb.flip(0))
-    assert torch.equal(hn[0], hf[0]) and torch.equal(hn[1], hb[0]) and torch.equal(cn[1], cb[0])
+    # The fused two-direction launch and the single-chain launch are different instantiations of the kernel: the
+    # compiler may contract multiply-adds differently, so agreement is to a rounding of h, not to the bit.
+    assert maxabs(y[:, :1024], yf.cpu()) <= 1e-3 and maxabs(y[:, 1024:], yb.flip(0).cpu()) <= 1e-3
+    assert maxabs(hn[0], hf[0].cpu()) <= 1e-3 and maxabs(hn[1], hb[0].cpu()) <= 1e-3 and maxabs(cn[1], cb[0].cpu()) <= 1e-3
     assert torch.equal(hn[1], y[0, 1024:]) and torch.equal(hn[0], y[-1, :1024])
 
 
