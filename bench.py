@@ -27,6 +27,10 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix rate
 SWEEP = [(4096, 4096), (16384, 4096), (4096, 16384), (32000, 1024)]
 POOL_BYTES_PER_SHAPE = 512 << 20
+# HBM bytes per launch of the dominant kernel, mean over its three shapes, from two rocprofv3 --pmc runs of this
+# script (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch, factors from --calibration-copy); the figures and the
+# commands are in profiles/gemv_sweep_pmc.md.  A counter reading, not something this script can measure itself.
+DOMINANT_KERNEL_TRAFFIC_BYTES = int((131425.0 + 131425.0 + 32929.0) / 3 * 1024 + (256.0 + 64.0 + 64.0) / 3 * 1024)
 
 
 def gemv_bytes(n, k, bias=True):
@@ -144,7 +148,7 @@ def main():
     dom_us = sum(p["us"] for p, _ in dom) / len(dom)
     achieved = dom_bytes / dom_us / 1e3
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=DOMINANT_KERNEL_TRAFFIC_BYTES,
                     kernel="gemv_mv_f16_kernel<2,4,4,4>", bytes_per_launch=int(dom_bytes), us_per_launch=round(dom_us, 3))
 
     # ---- LSTM: RNNT-style 2 layers, I=240, H=1024, T=200 (400 layer-steps per call) ------------------------------
@@ -203,7 +207,8 @@ def main():
             detail.append(f"{s['n']}x{s['k']}: {med * 1e3:.2f} ms")
         cpu = dict(value=round(b_total / t_total / 1e9, 2), unit="GB/s", cores=threads, kind="reference",
                    sample="LibTorch CPU at::addmm(b, x, W^T) in fp16, the op atenAddmm passes through to: median of <= 20 "
-                          "runs (<= 4 s) per sweep shape after 2 warm-ups, one pass of the same 4-GEMV sweep; " + "; ".join(detail))
+                          "runs (<= 4 s) per sweep shape after 2 warm-ups, same weight every run (cache-warm), one pass of the "
+                          "same 4-GEMV sweep; " + "; ".join(detail))
 
     out = {
         "metric": "fp16 GEMV HBM GB/s (% of peak) at 1 GPU; LSTM us/layer-step at H=1024",

@@ -42,8 +42,35 @@ def build_pimhip(verbose=True):
     return LIB_PATH
 
 
+ATEN_LIB_PATH = os.path.join(PKG_DIR, "_aten_ops_pimhip.so")
+
+
+def build_aten_ops(verbose=True):
+    """The C++ operator bodies with the reference's signatures (cpp/aten_ops_pimhip.cpp) plus their pybind module,
+    compiled with g++ against this image's LibTorch and linked to libpimhip.so next to it."""
+    import sysconfig
+
+    from torch.utils import cpp_extension as ce
+    import torch
+
+    cpp = os.path.join(PKG_DIR, "cpp")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-DTORCH_EXTENSION_NAME=_aten_ops_pimhip",
+           "-DTORCH_API_INCLUDE_EXTENSION_H"]
+    cmd += [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}"]
+    cmd += [os.path.join(cpp, "aten_ops_pimhip.cpp"), os.path.join(cpp, "aten_ops_pybind.cpp"), "-o", ATEN_LIB_PATH]
+    cmd += [f"-L{p}" for p in ce.library_paths()] + ["-lc10", "-ltorch", "-ltorch_cpu", "-ltorch_python"]
+    cmd += [f"-L{PKG_DIR}", "-lpimhip", "-Wl,-rpath,$ORIGIN"] + [f"-Wl,-rpath,{p}" for p in ce.library_paths()]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + res.stdout)
+    return ATEN_LIB_PATH
+
+
 def build_all(verbose=True):
-    return [build_pimhip(verbose)]
+    return [build_pimhip(verbose), build_aten_ops(verbose)]
 
 
 if __name__ == "__main__":

@@ -1,0 +1,112 @@
+"""The C++ operator bodies with the reference's signatures (pimaicompiler_amd/cpp/aten_ops_pimhip.cpp), driven through
+their pybind module.  CPU part: the module loads and its shape logic equals the oracle's.  GPU part: the same
+checks the reference's unit test makes (runtime/unit-tests/custom_op_ut.cpp) plus LibTorch CPU parity for the LSTM."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def cpp():
+    from pimaicompiler_amd import _aten_ops_pimhip as m
+    return m
+
+
+@pytest.fixture(scope="module")
+def cpp_gpu(cpp):
+    assert torch.cuda.is_available()
+    cpp.initialize(0)
+    return cpp
+
+
+def maxabs(a, b):
+    b = b if isinstance(b, torch.Tensor) else torch.as_tensor(np.asarray(b, dtype=np.float32))
+    return float((a.detach().float().cpu().reshape(-1) - b.float().reshape(-1)).abs().max())
+
+
+def test_cpp_shape_logic_matches_oracle(cpp):
+    shapes = [s for r in range(1, 5) for s in itertools.product((1, 2, 3), repeat=r)]
+    checked = 0
+    for s1 in shapes[::3]:
+        for s2 in shapes[::2]:
+            rc, o1, o2 = oracle.gemm_broadcast(s1, s2)
+            if rc != 0 or len(o1) != 4 or len(o2) != 4:
+                with pytest.raises(Exception):
+                    cpp.gemmBroadcast(list(s1), list(s2))
+                continue
+            p1, p2 = cpp.gemmBroadcast(list(s1), list(s2))
+            assert (p1, p2) == (o1, o2)
+            assert cpp.getGemmType(p1, p2) == oracle.get_gemm_type(o1, o2)
+            checked += 1
+    assert checked > 1000
+
+
+@pytest.mark.gpu
+def test_cpp_custom_gemv_unit_test(cpp_gpu):
+    """custom_op_ut.cpp:20-69 through customAtenMatmul, on seeded inputs scaled so that fp16 rounding of the result
+    is below the reference's atol 1e-3."""
+    g = torch.Generator().manual_seed(3)
+    a = (torch.rand(1, 1, 1, 1024, generator=g) / 32).half()
+    b = (torch.rand(1024, 4096, generator=g) / 32).half()
+    out = cpp_gpu.customAtenMatmul(a.to(DEV), b.to(DEV))
+    want = torch.matmul(a.double(), b.double())
+    assert list(out.shape) == [1, 1, 1, 4096]
+    assert torch.allclose(out.double().cpu(), want, atol=1e-3, rtol=1e-5)
+    a = (torch.rand(4096, 1024, generator=g) / 32).half()
+    b = (torch.rand(1, 1, 1024, 1, generator=g) / 32).half()
+    out = cpp_gpu.customAtenMatmul(a.to(DEV), b.to(DEV))
+    want = torch.matmul(a.double(), b.double())
+    assert list(out.shape) == [1, 1, 4096, 1]
+    assert torch.allclose(out.double().cpu(), want, atol=1e-3, rtol=1e-5)
+
+
+@pytest.mark.gpu
+def test_cpp_addmm_matches_libtorch_cpu_and_python_mirror(cpp_gpu, ops):
+    W, x, b = oracle.gemv_inputs(2001, 4096, 4096)
+    want = oracle.torch_addmm(b, x, W).reshape(-1)
+    y = cpp_gpu.customAtenAddmm("none", b.to(DEV), W.to(DEV), x.to(DEV).t(), 1.0, 1.0)
+    assert list(y.shape) == [4096, 1] and maxabs(y, want) <= 2e-3
+    y_py = ops.custom_aten_addmm("none", b.to(DEV), W.to(DEV), x.to(DEV).t())
+    assert torch.equal(y, y_py)
+    y = cpp_gpu.customAtenAddmm("aten::relu", b.to(DEV), x.to(DEV), W.to(DEV).t(), 1.0, 1.0)     # VM on a transposed view
+    assert list(y.shape) == [1, 4096] and maxabs(y, torch.relu(want)) <= 2e-3
+    y = cpp_gpu.atenLinear(x.to(DEV), W.to(DEV), b.to(DEV))
+    assert list(y.shape) == [1, 4096] and maxabs(y, want) <= 2e-3
+    y = cpp_gpu.atenLinear(x.to(DEV), W.to(DEV), None)
+    assert maxabs(y, want.float() - b.float()) <= 2e-3
+    v = (0.3 * torch.randn(4096, 1)).half()
+    y = cpp_gpu.customAtenMatmul(x.to(DEV), v.to(DEV))
+    assert list(y.shape) == [1, 1] and maxabs(y, x.float() @ v.float()) <= 2e-2
+    X = torch.randn(5, 4096).half()
+    y = cpp_gpu.customAtenMatmul(X.to(DEV), W.to(DEV).t())                                        # MM passthrough
+    assert list(y.shape) == [5, 4096] and maxabs(y, X.float() @ W.float().t()) <= 3e-2
+    with pytest.raises(Exception):
+        cpp_gpu.customAtenMatmul(x, W)                                                            # CPU tensors
+
+
+@pytest.mark.gpu
+def test_cpp_lstm_matches_libtorch_cpu(cpp_gpu):
+    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    wy, whn, wcn = oracle.torch_lstm(x, h0, c0, params, True, 2, False)
+    pd = [p.to(DEV) for p in params]
+    y, hn, cn = cpp_gpu.atenLstm1(x.to(DEV), [h0.to(DEV), c0.to(DEV)], pd, True, 2, 0.0, False, False, False)
+    assert list(y.shape) == [200, 1, 1024] and list(hn.shape) == [2, 1, 1024]
+    assert maxabs(y, wy) <= 5e-3 and maxabs(hn, whn) <= 5e-3 and maxabs(cn, wcn) <= 5e-3
+    yb, hnb, cnb = cpp_gpu.atenLstm1(x.to(DEV).transpose(0, 1), [h0.to(DEV), c0.to(DEV)], pd, True, 2, 0.0, False, False, True)
+    assert list(yb.shape) == [1, 200, 1024] and torch.equal(yb.reshape(-1), y.reshape(-1))
+    yp, hnp, cnp = cpp_gpu.atenLstm2(x.to(DEV).reshape(200, 240), torch.ones(200, dtype=torch.int64), [h0.to(DEV), c0.to(DEV)],
+                                     pd, True, 2, 0.0, False, False)
+    assert list(yp.shape) == [200, 1024] and torch.equal(yp.reshape(-1), y.reshape(-1)) and torch.equal(hnp, hn)
+    # bidirectional, one step at a time as the decoders call it
+    params, x, h0, c0 = oracle.lstm_inputs(77, 64, 128, 1, True, 6)
+    wy, whn, wcn = oracle.torch_lstm(x, h0, c0, params, True, 1, True)
+    y, hn, cn = cpp_gpu.atenLstm1(x.to(DEV), [h0.to(DEV), c0.to(DEV)], [p.to(DEV) for p in params], True, 1, 0.0, False, True, False)
+    assert maxabs(y, wy) <= 2e-3 and maxabs(hn, whn) <= 2e-3 and maxabs(cn, wcn) <= 2e-3
+    with pytest.raises(Exception):
+        cpp_gpu.atenLstm1(x.to(DEV).repeat(1, 2, 1), [h0.to(DEV), c0.to(DEV)], [p.to(DEV) for p in params], True, 1, 0.0, False, True, False)
