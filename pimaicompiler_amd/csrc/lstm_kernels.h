@@ -137,17 +137,22 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 //   2. per chain: 4 rows x 16 columns of dot products per lane (twice that with W_ih), a transpose-sum over
 //      the 64 lanes (6 exchanges) that leaves gate k in lane k, the four activations in parallel in lanes 0..3,
 //      the cell update;
-//   3. lane 0 of each wavefront publishes its h values of all chains with one store per 8 bytes, and stores y.
+//   3. lane 0 of each wavefront stores y and hands its h values to LDS; one barrier; one lane publishes the block's
+//      entry with one store per 16 bytes.
 //
-// Exchange buffer: hx[2][NB][16] 32-bit words; block b uses words [w * NC + k] (wavefront w, chain k) of its
-// 64-byte entry (entries of different blocks do not share a 64-byte segment, which measurably shortens the
-// exchange).  word = fp16 bits | tag << 16.  Super-step tau publishes under tag (tag_base + tau + 1) & 0xffff
-// into parity tau & 1; super-step tau >= 1 waits until all 4 * NC words of an entry in parity (tau - 1) & 1
-// carry tag (tag_base + tau) & 0xffff.  Data and flag travel in one word, written and read with device-scope
-// relaxed atomics, so one store / load round trip through memory publishes a super-step.  A block cannot
-// overwrite parity p before every block has consumed it: publishing super-step tau + 2 needs the words of
-// tau + 1 from all blocks, which they publish only after reading tau.  The host advances tag_base by the
-// number of super-steps per launch (at most 65000), so tags left by earlier launches never equal an expected one.
+// Exchange buffer: hx[2][NB] entries of 64 bytes (entries of different blocks do not share a 64-byte segment,
+// which measurably shortens the exchange); chain k of block b uses the 8-byte word k of the entry, one fp16 per
+// wavefront.  |h| <= 1, so bit 14 of its fp16 pattern is always 0 and carries the flag: with g = g_base + tau
+// counting super-steps over all launches of a plan, super-step g publishes into parity g & 1 with flag bit
+// (g >> 1) & 1, i.e. the bit flips every time a slot is rewritten.  A slot can only hold what was published two
+// super-steps earlier or the current values (publishing g + 2 needs the words of g + 1 from all blocks, which
+// they publish only after reading g), so one bit tells them apart; every fp16 carries it, so a reader validates
+// each 8-byte word on its own.  A block gathers its values in LDS and publishes them with ONE store (8 bytes for
+// one chain, 16 for two); a waiting lane reads a block's entry with ONE load of the same size.  The round trip of
+// that pair through the memory side is the cost of a super-step: measured at 256 blocks, every further load per
+// poll and every further store per block adds about 0.3 us.  The buffer is zero when g = 2, the first value
+// the host uses; every launch writes every fp16 of every entry in every super-step, so the sequence of flag bits
+// per slot stays alternating across launches.  After a time-out the host clears the buffer and restarts at g = 2.
 //
 // Every wait is bounded: after `spin_limit` polls a lane raises *abort_flag and stops waiting; lanes poll
 // the flag every 256 spins and stop waiting once it is set.  The kernel then runs to the end with
@@ -156,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 static constexpr int kSeqUnits = 4;        // hidden units per block, one per wavefront
 static constexpr int kSeqMaxH = 1024;      // 64 lanes x 16 columns
 static constexpr int kSeqEntryWords = 16;  // 32-bit words between the entries of consecutive blocks (64 bytes)
-static constexpr int kSeqMaxT = 65000;       // super-steps per launch
+static constexpr int kSeqMaxT = 1 << 30;    // super-steps per launch (the counters are 32-bit)
 static constexpr int kSeqMaxChains = 4;
 
 template <int CTRL>
@@ -201,20 +206,40 @@ struct LstmSeqChain {
 
 struct LstmSeqArgs {
     LstmSeqChain chain[kSeqMaxChains];
-    unsigned int* hx;          // [2][NB][kSeqEntryWords]
+    unsigned int* hx;          // [2][NB][kSeqEntryWords]; zero when g_base == 2
     unsigned int* abort_flag;  // set to 1 when a wait gives up
     long y_stride;             // elements between consecutive time steps of y
     int H;
     int T;
-    unsigned int tag_base;
+    unsigned int g_base;       // super-steps this buffer has seen so far, plus 2
     unsigned int spin_limit;
 };
+
+// One 16-byte device-scope load.  Each 8-byte half is validated on its own by the caller, so nothing depends on the
+// 16 bytes being read as a unit.
+__device__ __forceinline__ void load16_device_scope(const void* p, unsigned long long& lo, unsigned long long& hi)
+{
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    lo = (unsigned long long)v[0] | ((unsigned long long)v[1] << 32);
+    hi = (unsigned long long)v[2] | ((unsigned long long)v[3] << 32);
+}
+
+// One 16-byte device-scope store of two 8-byte words (each validated on its own by the readers).
+__device__ __forceinline__ void store16_device_scope(void* p, unsigned long long lo, unsigned long long hi)
+{
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 v = {(unsigned int)lo, (unsigned int)(lo >> 32), (unsigned int)hi, (unsigned int)(hi >> 32)};
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
 
 template <int NC, bool WAVEFRONT>
 __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
 {
-    static_assert(NC >= 1 && NC <= kSeqMaxChains && 4 * NC <= kSeqEntryWords, "entry holds 4 words per chain");
+    static_assert(NC >= 1 && NC <= kSeqMaxChains && 2 * NC <= kSeqEntryWords, "an entry holds one 8-byte word per chain");
     __shared__ __align__(16) half_t hbuf[2][NC][kSeqMaxH];  // published h per chain, double buffered by parity
+    __shared__ __align__(16) unsigned short pub[NC][4];     // this block's next entry: chain k, wavefront w
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -290,23 +315,24 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
 
         // ---- 1. what block `tid` published at super-step tau - 1 (or the initial state) into LDS ----
         if (has_entry) {
-            unsigned int words[4 * NC];
+            unsigned long long words[NC];  // word k: the four fp16 of chain k published by block `tid`
 #pragma unroll
-            for (int i = 0; i < 4 * NC; ++i) words[i] = 0u;
+            for (int k = 0; k < NC; ++k) words[k] = 0ull;
             if (tau > 0) {
-                const unsigned int want = (p.tag_base + (unsigned int)tau) & 0xffffu;
-                unsigned long long* src =
-                    reinterpret_cast<unsigned long long*>(p.hx + ((long)((tau - 1) & 1) * nb + tid) * kSeqEntryWords);
+                const unsigned int gp = p.g_base + (unsigned int)tau - 1u;  // the super-step whose values are awaited
+                const unsigned long long want = ((gp >> 1) & 1u) ? 0x4000400040004000ull : 0ull;
+                const unsigned long long* src =
+                    reinterpret_cast<const unsigned long long*>(p.hx + ((long)(gp & 1u) * nb + tid) * kSeqEntryWords);
                 unsigned int spins = 0;
                 while (true) {
                     bool ok = true;
 #pragma unroll
-                    for (int i = 0; i < 2 * NC; ++i) {
-                        const unsigned long long q = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        words[2 * i] = (unsigned int)q;
-                        words[2 * i + 1] = (unsigned int)(q >> 32);
-                        ok = ok && (words[2 * i] >> 16) == want && (words[2 * i + 1] >> 16) == want;
-                    }
+                    for (int k = 0; k + 1 < NC; k += 2) load16_device_scope(src + k, words[k], words[k + 1]);
+                    if (NC & 1)
+                        words[NC - 1] = __hip_atomic_load(const_cast<unsigned long long*>(src) + (NC - 1), __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int k = 0; k < NC; ++k) ok = ok && (words[k] & 0x4000400040004000ull) == want;
                     if (ok || gave_up) break;
                     ++spins;
                     if ((spins & 255u) == 0u) {
@@ -327,93 +353,111 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) hv[e] = (tid * 4 + e < H) ? p.chain[k].h0[tid * 4 + e] : (half_t)0.0f;
                 } else {
-                    // words[w * NC + k] is unit w of chain k in block `tid`.
+                    // Unit e of chain k in block `tid`, flag bit removed.
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) hv[e] = __builtin_bit_cast(half_t, (unsigned short)(words[e * NC + k] & 0xffffu));
+                    for (int e = 0; e < 4; ++e) hv[e] = __builtin_bit_cast(half_t, (unsigned short)((words[k] >> (16 * e)) & 0xbfffu));
                 }
                 *reinterpret_cast<half4_t*>(&hb[k][tid * 4]) = hv;
             }
         }
         __syncthreads();
 
-        // ---- 2. gates per chain ----
-        half_t h_new[NC];
+        // ---- 2. gates of all chains ----
+        // Written without branches and phase by phase over the chains, so that the chains' dependency chains
+        // (LDS read, dot products, six exchange steps, exp / rcp) overlap instead of running one after another.  A
+        // chain that has not started or has finished computes on whatever its buffer holds; the result is dropped.
+        float acc[NC][4];
 #pragma unroll
         for (int k = 0; k < NC; ++k) {
-            const int s_k = WAVEFRONT ? tau - k : tau;
-            h_new[k] = (half_t)0.0f;
-            if (s_k < 0 || s_k >= T) continue;  // uniform: this chain has not started yet, or has finished
-
             const half8_t ha = *reinterpret_cast<const half8_t*>(&hb[k][lane * 16]);
             const half8_t hc = *reinterpret_cast<const half8_t*>(&hb[k][lane * 16 + 8]);
-            float acc[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[v] = dot8(w_hh[k][v][1], hc, dot8(w_hh[k][v][0], ha, 0.0f));
+            for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_hh[k][v][1], hc, dot8(w_hh[k][v][0], ha, 0.0f));
             if (WAVEFRONT && k > 0) {
-                // Input of layer k at this time step: h of layer k - 1 at the same time step, published one
-                // super-step ago.  At s_k == 0 chain k - 1's buffer holds exactly that (its s = 1 input).
+                // Input of layer k at its time step: h of layer k - 1 at the same time step, published one
+                // super-step ago, which is what chain k - 1's buffer holds now.
                 const half8_t xa = *reinterpret_cast<const half8_t*>(&hb[k - 1][lane * 16]);
                 const half8_t xc = *reinterpret_cast<const half8_t*>(&hb[k - 1][lane * 16 + 8]);
 #pragma unroll
-                for (int v = 0; v < 4; ++v) acc[v] = dot8(w_ih[k][v][1], xc, dot8(w_ih[k][v][0], xa, acc[v]));
+                for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_ih[k][v][1], xc, dot8(w_ih[k][v][0], xa, acc[k][v]));
             }
+        }
 
-            // Transpose-sum: after the two halving exchanges lane l holds slot 2 * (l & 1) + ((l >> 1) & 1) summed
-            // over its quad, i.e. gate (l & 3); wave_sum_mod4 then adds the 16 quads.
-            const bool b0 = lane & 1, b1 = lane & 2;
-            const float a0 = (b0 ? acc[2] : acc[0]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[0] : acc[2]);
-            const float a1 = (b0 ? acc[3] : acc[1]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[1] : acc[3]);
-            float a = wave_sum_mod4((b1 ? a1 : a0) + dpp_mov_f32<kDppQuadXor2>(b1 ? a0 : a1));
+        // Transpose-sum: after the two halving exchanges lane l holds slot 2 * (l & 1) + ((l >> 1) & 1) summed over
+        // its quad, i.e. gate (l & 3); wave_sum_mod4 then adds the 16 quads.
+        const bool b0 = lane & 1, b1 = lane & 2;
+        float a[NC];
+#pragma unroll
+        for (int k = 0; k < NC; ++k) {
+            const float a0 = (b0 ? acc[k][2] : acc[k][0]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[k][0] : acc[k][2]);
+            const float a1 = (b0 ? acc[k][3] : acc[k][1]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[k][1] : acc[k][3]);
+            a[k] = (b1 ? a1 : a0) + dpp_mov_f32<kDppQuadXor2>(b1 ? a0 : a1);
+        }
+#pragma unroll
+        for (int k = 0; k < NC; ++k) a[k] = wave_sum_mod4(a[k]);
+
+        half_t h_new[NC];
+        float c_out[NC];
+        const bool is_g = my_gate == 2;
+#pragma unroll
+        for (int k = 0; k < NC; ++k) {
+            const int s_k = WAVEFRONT ? tau - k : tau;
+            const bool active = s_k >= 0 && s_k < T;
             if (WAVEFRONT && k > 0) {
-                a += bias_reg[k];
+                a[k] += bias_reg[k];
             } else {
-                a += xp_slot[k];
+                a[k] += xp_slot[k];
                 // The term fetched two steps ago has been consumed: refill the same register for two steps ahead.
                 // (Issued only now so that the old and the new value never live at once, which would cost a copy,
                 // and with it a wait for this load and for the stores below, at the loop's back edge.)
-                xp_slot[k] = xp_ptr[k][(long)min(s_k + 2, T - 1) * xp_step[k]];
+                xp_slot[k] = xp_ptr[k][(long)max(0, min(s_k + 2, T - 1)) * xp_step[k]];
             }
-
             // Each of lanes 0..3 activates its own gate: sigmoid for i, f, o and tanh(a) = 2 * sigmoid(2a) - 1 for g.
-            const bool is_g = my_gate == 2;
-            const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
+            const float sg = fast_sigmoid_f32(is_g ? 2.0f * a[k] : a[k]);
             const float act = is_g ? 2.0f * sg - 1.0f : sg;
             const float g_i = dpp_mov_f32<0x00>(act);  // quad_perm broadcasts of lanes 0, 1, 2, 3 of the quad
             const float g_f = dpp_mov_f32<0x55>(act);
             const float g_g = dpp_mov_f32<0xAA>(act);
             const float g_o = dpp_mov_f32<0xFF>(act);
             const float c_new = g_f * c_reg[k] + g_i * g_g;
-            h_new[k] = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
-            c_reg[k] = c_new;
+            const half_t h = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
+            h_new[k] = active ? h : (half_t)0.0f;
+            c_reg[k] = active ? c_new : c_reg[k];
+            c_out[k] = c_new;
+        }
 
-            if (lane == 0 && unit_ok) {
-                const int t = p.chain[k].reverse ? (T - 1 - s_k) : s_k;
-                if (p.chain[k].y) p.chain[k].y[(long)t * p.y_stride + j] = h_new[k];
-                if (s_k == T - 1) {
-                    p.chain[k].hn[j] = h_new[k];
-                    p.chain[k].cn[j] = (half_t)c_new;
+        // ---- 3. outputs, then publish ----
+        // The block's values are gathered in LDS and published by ONE lane with ONE store per 16 bytes: the time
+        // until every block has seen a super-step grows by about 0.3 us with every further store per block.
+        if (lane == 0) {
+            const unsigned int flag = (((p.g_base + (unsigned int)tau) >> 1) & 1u) << 14;
+#pragma unroll
+            for (int k = 0; k < NC; ++k) {
+                const unsigned int hbits = unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new[k]) : 0u;
+                pub[k][wave] = (unsigned short)(hbits | flag);
+            }
+            if (unit_ok) {
+#pragma unroll
+                for (int k = 0; k < NC; ++k) {
+                    const int s_k = WAVEFRONT ? tau - k : tau;
+                    if (s_k < 0 || s_k >= T) continue;
+                    const int t = p.chain[k].reverse ? (T - 1 - s_k) : s_k;
+                    if (p.chain[k].y) p.chain[k].y[(long)t * p.y_stride + j] = h_new[k];
+                    if (s_k == T - 1) {
+                        p.chain[k].hn[j] = h_new[k];
+                        p.chain[k].cn[j] = (half_t)c_out[k];
+                    }
                 }
             }
         }
-
-        // ---- 3. publish: words [wave * NC + k] of this block's entry, 8 bytes per store where possible ----
-        if (lane == 0) {
-            const unsigned int tag = ((p.tag_base + (unsigned int)tau + 1u) & 0xffffu) << 16;
-            unsigned int* dst = p.hx + ((long)(tau & 1) * nb + blockIdx.x) * kSeqEntryWords + wave * NC;
-            unsigned int word[NC];
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned int g = p.g_base + (unsigned int)tau;
+            unsigned long long* dst = reinterpret_cast<unsigned long long*>(p.hx + ((long)(g & 1u) * nb + blockIdx.x) * kSeqEntryWords);
+            const unsigned long long* src = reinterpret_cast<const unsigned long long*>(&pub[0][0]);
 #pragma unroll
-            for (int k = 0; k < NC; ++k)
-                word[k] = (unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new[k]) : 0u) | tag;
-            if (NC % 2 == 0) {
-#pragma unroll
-                for (int k = 0; k < NC; k += 2)
-                    __hip_atomic_store(reinterpret_cast<unsigned long long*>(dst + k),
-                                       (unsigned long long)word[k] | ((unsigned long long)word[k + 1] << 32), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-            } else {
-#pragma unroll
-                for (int k = 0; k < NC; ++k) __hip_atomic_store(dst + k, word[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            for (int k = 0; k + 1 < NC; k += 2) store16_device_scope(dst + k, src[k], src[k + 1]);
+            if (NC & 1) __hip_atomic_store(dst + (NC - 1), src[NC - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
 

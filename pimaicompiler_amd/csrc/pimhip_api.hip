@@ -321,7 +321,11 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
 // ================================================================================================
 namespace
 {
-__global__ void fill_u32_kernel(unsigned int* p, unsigned int v) { *p = v; }
+__global__ void fill_u32_kernel(unsigned int* p, size_t n, unsigned int v)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
 
 int launch_input_projection(float* out, const half_t* x, const half_t* w, const float* bias, int64_t T, int64_t K,
                             int64_t N, hipStream_t s)
@@ -374,7 +378,8 @@ struct PimHipLstmPlan {
     int mode = 0;
     bool seq_kernel_ok = false;      // shape fits the persistent sequence kernel
     unsigned int spin_limit = 1u << 22;
-    unsigned int tag_base = 0;
+    unsigned int g_count[kSeqMaxChains + 1] = {2, 2, 2, 2, 2};  // per chain count: super-steps its buffer region has seen, plus 2
+    size_t hx_region_words = 0;      // 32-bit words of one region of hx (one region per chain count)
     int max_wavefront = kSeqMaxChains;  // layers of a unidirectional stack advanced by one persistent launch
 
     struct Cell {
@@ -391,7 +396,7 @@ struct PimHipLstmPlan {
     float* xproj = nullptr;           // [num_dirs][max_seq_len][4H] fp32
     half_t* ybuf[2] = {nullptr, nullptr};  // inter-layer sequences [max_seq_len][num_dirs * H]
     float* c_state = nullptr;         // [num_dirs][H] fp32, per-step kernel's cell state
-    unsigned int* hx = nullptr;       // [num_dirs][2][NB][kSeqEntryWords] exchange words of the sequence kernel
+    unsigned int* hx = nullptr;       // [kSeqMaxChains][2][NB][kSeqEntryWords] exchange entries of the sequence kernel
     unsigned int* abort_flag = nullptr;
     unsigned int* abort_host = nullptr;  // pinned copy read by pimhip_lstm_plan_status
     int seq_blocks = 0;
@@ -534,7 +539,10 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         plan->seq_kernel_ok = (int64_t)per_cu * plan->num_cus >= plan->seq_blocks;
     }
     if (plan->seq_kernel_ok) {
-        const size_t words = (size_t)2 * plan->seq_blocks * kSeqEntryWords;
+        // One region per number of chains a launch can advance: a launch writes exactly the words of its chains,
+        // and the flag bits of a region must see every super-step that uses it.
+        plan->hx_region_words = (size_t)2 * plan->seq_blocks * kSeqEntryWords;
+        const size_t words = plan->hx_region_words * kSeqMaxChains;
         PLAN_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned int)));
         PLAN_HIP_CHECK(hipMemsetAsync(plan->hx, 0, words * sizeof(unsigned int), s));
     }
@@ -617,9 +625,14 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     }
 
     if (*plan->abort_host != 0u) {
-        // The previous forward of this plan timed out: re-arm the flag (a fill kernel, not a memset node, so
-        // that callers may capture this call).
-        fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 0u);
+        // The previous forward of this plan timed out: re-arm the flag and bring the exchange buffer back to its
+        // initial state (fill kernels, not memset nodes, so that callers may capture this call).
+        fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 1, 0u);
+        if (plan->hx) {
+            const size_t words = plan->hx_region_words * kSeqMaxChains;
+            fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->hx, words, 0u);
+        }
+        for (int i = 0; i <= kSeqMaxChains; ++i) plan->g_count[i] = 2;
         *plan->abort_host = 0u;
     }
     const bool use_seq = (plan->mode == 2 && T + kSeqMaxChains <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T + kSeqMaxChains <= kSeqMaxT);
@@ -662,14 +675,14 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                 ch.reverse = (D == 2) ? k : 0;
                 ch.y = (D == 2) ? group_out + (size_t)k * H : ((k == nc - 1) ? group_out : nullptr);
             }
-            a.hx = plan->hx;
+            a.hx = plan->hx + plan->hx_region_words * (size_t)(nc - 1);
             a.abort_flag = plan->abort_flag;
             a.y_stride = y_stride;
             a.H = (int)H;
             a.T = (int)T;
-            a.tag_base = plan->tag_base;
+            a.g_base = plan->g_count[nc];
             a.spin_limit = plan->spin_limit;
-            plan->tag_base += (unsigned int)((D == 2) ? T : T + nc - 1);
+            plan->g_count[nc] += (unsigned int)((D == 2) ? T : T + nc - 1);
             const dim3 grid(plan->seq_blocks), block(256);
             if (D == 2) {
                 lstm_seq_f16_kernel<2, false><<<grid, block, 0, s>>>(a);
