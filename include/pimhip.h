@@ -110,6 +110,18 @@ int pimhip_execute_gemv_group(int count, void* const* outs, const void* const* i
                               const void* const* biases, const int64_t* in_ws, const int64_t* out_ws,
                               const int* acts, void* stream);
 
+/* Replaces rocblas_bmm_template_xAy and the two device copies that follow it in executeAtenBmm
+ * (runtime/include/executor/op_executor/custom_ops.h:435-466,
+ *  runtime/source/executor/op_executor/aten_ops_executor.cpp:668-747): y[1, n] = x[1, k] . A[k, n], A row-major and
+ * dense, fp32 accumulation (the reference accumulates in fp16), the result stored to every one of the n_outs
+ * (1..4) buffers of the host array `outs` (the GNMT attention context lands in three concatenation buffers). */
+int pimhip_execute_bmm(void* const* outs, int n_outs, const void* x, const void* A, int64_t k, int64_t n, void* stream);
+
+/* Replaces custom_add (custom_ops.h:383-433; executeAtenAdd, aten_ops_executor.cpp:43-179):
+ * c[m, n] = a[m, n] + b, with b [m, n] (b_broadcast == 0) or one row [n] added to every row (b_broadcast != 0).
+ * fp16 in and out, each sum rounded once; c may alias a or b; any n (the reference needs n % 4 == 0). */
+int pimhip_execute_add(void* c, const void* a, const void* b, int64_t m, int64_t n, int b_broadcast, void* stream);
+
 /* ---- LSTM ----------------------------------------------------------------------------------- */
 
 typedef struct PimHipLstmPlan PimHipLstmPlan;

@@ -56,6 +56,8 @@ def lib():
         l.oracle_gemv_vm.argtypes = [_u16p, _u16p, _u16p, _u16p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
         l.oracle_dot.restype = None
         l.oracle_dot.argtypes = [_u16p, _u16p, _u16p, ctypes.c_int64]
+        l.oracle_add.restype = None
+        l.oracle_add.argtypes = [_u16p, _u16p, _u16p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int]
         l.oracle_gemv_mv_f32.restype = None
         l.oracle_gemv_mv_f32.argtypes = [ctypes.POINTER(ctypes.c_float)] * 4 + [ctypes.c_int64, ctypes.c_int64]
         l.oracle_lstm.restype = None
@@ -123,6 +125,17 @@ def dot(a, b):
     y = np.empty(1, dtype=np.uint16)
     lib().oracle_dot(ap, bp, y.ctypes.data_as(_u16p), au.size)
     return y.view(np.float16)
+
+
+def add(a, b):
+    """c = a[m, n] + b with b [m, n] or [n] (fp16, one rounding)."""
+    au, ap = _h(a)
+    bu, bp = _h(b)
+    n = au.shape[-1]
+    m = au.size // n
+    c = np.empty(au.size, dtype=np.uint16)
+    lib().oracle_add(ap, bp, c.ctypes.data_as(_u16p), m, n, int(bu.size != au.size))
+    return c.view(np.float16).reshape(au.shape)
 
 
 def gemv_mv_f32(W, x, bias=None):

@@ -15,6 +15,8 @@ from .ops import (  # noqa: F401
     custom_aten_addmm,
     custom_aten_matmul,
     aten_linear,
+    aten_bmm,
+    aten_add,
     aten_lstm1,
     aten_lstm2,
     execute_gemv_group,

@@ -27,6 +27,10 @@ SIGNATURES = {
                                           ctypes.c_void_p]),
     "pimhip_execute_gemv_group": (ctypes.c_int, [ctypes.c_int, c_void_pp, c_void_pp, c_void_pp, c_void_pp,
                                                  c_int64_p, c_int64_p, c_int_p, ctypes.c_void_p]),
+    "pimhip_execute_bmm": (ctypes.c_int, [c_void_pp, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                          ctypes.c_int64, ctypes.c_void_p]),
+    "pimhip_execute_add": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                          ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "pimhip_lstm_plan_create": (ctypes.c_int, [c_void_pp, c_void_pp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                                ctypes.c_void_p]),

@@ -184,11 +184,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_generic_kernel(const h
 // the result does not depend on which block finishes last), applies the epilogue and re-arms the
 // ticket counter for the next launch.
 // ---------------------------------------------------------------------------------------------
+// Destinations of a VM product: the same result is stored to `count` buffers (the GNMT attention context goes
+// straight into three concatenation buffers, runtime/source/executor/op_executor/aten_ops_executor.cpp:694-737).
+static constexpr int kGemvMaxOuts = 4;
+struct GemvOuts {
+    half_t* y[kGemvMaxOuts];
+    int count;
+};
+
 template <int WAVES, int U>
 __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* __restrict__ x,
                                                                  const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ bias,
-                                                                 half_t* __restrict__ y, int K, int N, long lda,
+                                                                 GemvOuts outs, int K, int N, long lda,
                                                                  int relu, int k_per_slice,
                                                                  float* __restrict__ partial,
                                                                  unsigned int* __restrict__ tickets)
@@ -257,7 +265,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
                 if (relu) v = fmaxf(v, 0.0f);
                 out[j] = (half_t)v;
             }
-            *reinterpret_cast<half8_t*>(y + col0) = out;
+            for (int o = 0; o < outs.count; ++o) *reinterpret_cast<half8_t*>(outs.y[o] + col0) = out;
         }
         return;
     }
@@ -287,7 +295,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
             if (relu) v = fmaxf(v, 0.0f);
             out[j] = (half_t)v;
         }
-        *reinterpret_cast<half8_t*>(y + col0) = out;
+        for (int o = 0; o < outs.count; ++o) *reinterpret_cast<half8_t*>(outs.y[o] + col0) = out;
     }
     if (threadIdx.x == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -296,7 +304,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
 __global__ __launch_bounds__(256) void gemv_vm_f16_generic_kernel(const half_t* __restrict__ x,
                                                                   const half_t* __restrict__ A,
                                                                   const half_t* __restrict__ bias,
-                                                                  half_t* __restrict__ y, int K, int N, long lda,
+                                                                  GemvOuts outs, int K, int N, long lda,
                                                                   int relu)
 {
     const long col = (long)blockIdx.x * 256 + threadIdx.x;
@@ -305,7 +313,35 @@ __global__ __launch_bounds__(256) void gemv_vm_f16_generic_kernel(const half_t* 
     for (int k = 0; k < K; ++k) acc = fmaf((float)A[(long)k * lda + col], (float)x[k], acc);
     if (bias) acc += (float)bias[col];
     if (relu) acc = fmaxf(acc, 0.0f);
-    y[col] = (half_t)acc;
+    for (int o = 0; o < outs.count; ++o) outs.y[o][col] = (half_t)acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// C[m][n] = A[m][n] + B, B either [m][n] or one row [n] added to every row (the reference's custom_add,
+// runtime/include/executor/op_executor/custom_ops.h:383-433).  The exact sum of two fp16 values rounded once to
+// fp16, which is also what the reference's half2 addition yields.  C may alias A or B.  HBM-bound: 6 bytes per element.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void add_f16_vec_kernel(const half_t* A, const half_t* B, half_t* C, long total8,
+                                                          long row8, int b_broadcast)
+{
+    // Units of 8 halves (16 bytes); row8 = n / 8.
+    const long stride = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total8; i += stride) {
+        const half8_t a = reinterpret_cast<const half8_t*>(A)[i];
+        const half8_t b = reinterpret_cast<const half8_t*>(B)[b_broadcast ? (i % row8) : i];
+        half8_t c;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) c[e] = (half_t)((float)a[e] + (float)b[e]);
+        reinterpret_cast<half8_t*>(C)[i] = c;
+    }
+}
+
+__global__ __launch_bounds__(256) void add_f16_generic_kernel(const half_t* A, const half_t* B, half_t* C, long total,
+                                                              long n, int b_broadcast)
+{
+    const long stride = (long)gridDim.x * 256;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
+        C[i] = (half_t)((float)A[i] + (float)B[b_broadcast ? (i % n) : i]);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -134,13 +134,14 @@ int gemv_mv(const half_t* W, const half_t* x, const half_t* bias, half_t* y, int
     return PIMHIP_OK;
 }
 
-int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bias, half_t* y, int64_t K, int64_t N,
-            int64_t lda, int relu, hipStream_t s)
+int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bias, const GemvOuts& outs, int64_t K,
+            int64_t N, int64_t lda, int relu, hipStream_t s)
 {
-    const bool vec_ok = (N % 8 == 0) && (lda % 8 == 0) && aligned16(A) && aligned16(y);
+    bool vec_ok = (N % 8 == 0) && (lda % 8 == 0) && aligned16(A);
+    for (int o = 0; o < outs.count; ++o) vec_ok = vec_ok && aligned16(outs.y[o]);
     if (!vec_ok) {
         const int grid = (int)((N + 255) / 256);
-        gemv_vm_f16_generic_kernel<<<grid, 256, 0, s>>>(x, A, bias, y, (int)K, (int)N, (long)lda, relu);
+        gemv_vm_f16_generic_kernel<<<grid, 256, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu);
         return PIMHIP_OK;
     }
     constexpr int WAVES = 4;
@@ -165,7 +166,7 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
         tickets = ws->tickets;
     }
     dim3 grid(col_blocks, slices);
-    gemv_vm_f16_kernel<WAVES, 4><<<grid, WAVES * 64, 0, s>>>(x, A, bias, y, (int)K, (int)N, (long)lda, relu,
+    gemv_vm_f16_kernel<WAVES, 4><<<grid, WAVES * 64, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu,
                                                              k_per_slice, partial, tickets);
     return PIMHIP_OK;
 }
@@ -251,9 +252,65 @@ extern "C" int pimhip_execute_gemv(void* out, const void* in, const void* weight
     const int relu = act == PIMHIP_ACT_RELU;
     if (order == PIMHIP_W_X_I)
         rc = gemv_mv((const half_t*)weight, (const half_t*)in, (const half_t*)bias, (half_t*)out, out_w, in_w, ld_weight, relu, s);
-    else
-        rc = gemv_vm(st, (const half_t*)in, (const half_t*)weight, (const half_t*)bias, (half_t*)out, in_w, out_w, ld_weight, relu, s);
+    else {
+        GemvOuts outs;
+        memset(&outs, 0, sizeof(outs));
+        outs.y[0] = (half_t*)out;
+        outs.count = 1;
+        rc = gemv_vm(st, (const half_t*)in, (const half_t*)weight, (const half_t*)bias, outs, in_w, out_w, ld_weight, relu, s);
+    }
     if (rc != PIMHIP_OK) return rc;
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_execute_bmm(void* const* outs, int n_outs, const void* x, const void* A, int64_t k, int64_t n,
+                                  void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!outs || !x || !A) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "outs, x and A must be non-null");
+    if (n_outs < 1 || n_outs > kGemvMaxOuts) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "n_outs=%d not in [1, %d]", n_outs, kGemvMaxOuts);
+    if (k < 0 || n < 0 || k > INT32_MAX || n > INT32_MAX) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "k=%lld n=%lld out of range", (long long)k, (long long)n);
+    GemvOuts o;
+    memset(&o, 0, sizeof(o));
+    for (int i = 0; i < n_outs; ++i) {
+        if (!outs[i]) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "outs[%d] is null", i);
+        o.y[i] = (half_t*)outs[i];
+    }
+    o.count = n_outs;
+    if (n == 0) return PIMHIP_OK;
+    rc = gemv_vm(st, (const half_t*)x, (const half_t*)A, nullptr, o, k, n, n, 0, static_cast<hipStream_t>(stream));
+    if (rc != PIMHIP_OK) return rc;
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_execute_add(void* c, const void* a, const void* b, int64_t m, int64_t n, int b_broadcast, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!c || !a || !b) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "c, a and b must be non-null");
+    if (m < 0 || n < 0) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "m=%lld n=%lld must not be negative", (long long)m, (long long)n);
+    const int64_t total = m * n;
+    if (total == 0) return PIMHIP_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // About 8 blocks per CU, each lane 16 bytes per operand and trip.
+    const bool vec_ok = (n % 8 == 0) && aligned16(a) && aligned16(b) && aligned16(c);
+    if (vec_ok) {
+        const int64_t total8 = total / 8;
+        int64_t grid = (total8 + 255) / 256;
+        if (grid > 8LL * st->num_cus) grid = 8LL * st->num_cus;
+        add_f16_vec_kernel<<<(unsigned)grid, 256, 0, s>>>((const half_t*)a, (const half_t*)b, (half_t*)c, (long)total8,
+                                                            (long)(n / 8), b_broadcast ? 1 : 0);
+    } else {
+        int64_t grid = (total + 255) / 256;
+        if (grid > 8LL * st->num_cus) grid = 8LL * st->num_cus;
+        add_f16_generic_kernel<<<(unsigned)grid, 256, 0, s>>>((const half_t*)a, (const half_t*)b, (half_t*)c, (long)total, (long)n,
+                                                                b_broadcast ? 1 : 0);
+    }
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
 }

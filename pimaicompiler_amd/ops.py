@@ -310,6 +310,76 @@ def execute_gemv_group(inputs, weights, biases=None, act_types=None, stream=None
     return outs
 
 
+def aten_bmm(self_tensor, other_tensor, outs=None, stream=None):
+    """executeAtenBmm's custom path (runtime/source/executor/op_executor/aten_ops_executor.cpp:668-747): for a single
+    row, y[..., 1, n] = x[..., 1, k] . A[..., k, n] on the VM kernel.  `outs` may list up to four preallocated fp16
+    buffers of n elements (views into concatenation buffers, as the GNMT decoder uses them, :694-737): the result is
+    stored to each of them by the one launch and the first is returned.  More than one row or batch: LibTorch."""
+    _require_half_cuda(self_tensor, other_tensor)
+    m, k = self_tensor.size(-2), self_tensor.size(-1)
+    n, k2 = other_tensor.size(-1), other_tensor.size(-2)
+    if k != k2:
+        raise NNRuntimeException(f"bmm operands disagree on the reduction width ({k} vs {k2})")
+    if m != 1 or self_tensor.numel() != k or other_tensor.numel() != k * n:
+        if outs:
+            raise NNRuntimeException("preallocated outputs need the single-row product")
+        return torch.bmm(self_tensor, other_tensor) if self_tensor.dim() == 3 else torch.matmul(self_tensor, other_tensor)
+    lib = L.load()
+    _ensure_init(other_tensor)
+    x, A = self_tensor.contiguous(), other_tensor.contiguous()
+    shape = list(self_tensor.shape)
+    shape[-1], shape[-2] = n, m
+    if not outs:
+        outs = [torch.empty(shape, dtype=torch.float16, device=A.device)]
+    if len(outs) > 4:
+        raise NNRuntimeException("at most four destinations")
+    for o in outs:
+        _require_half_cuda(o)
+        if o.numel() != n or not o.is_contiguous():
+            raise NNRuntimeException(f"every destination must be a contiguous fp16 buffer of {n} elements")
+    arr = (ctypes.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
+    _check(lib.pimhip_execute_bmm(arr, len(outs), x.data_ptr(), A.data_ptr(), k, n, _stream_handle(stream)))
+    return outs[0]
+
+
+def aten_add(self_tensor, other_tensor, alpha=1, out=None, stream=None):
+    """executeAtenAdd's custom path (aten_ops_executor.cpp:43-179): fp16 tensors of equal rank (element-wise) or
+    with `other` one row broadcast over the rows of `self`; the reference's kernel ignores alpha (custom_ops.h:415-433)
+    and so does this path.  The reference writes the sum into `self` (or, in the GNMT decoder, into a concatenation
+    buffer): pass `out` for that; by default a new tensor is returned.  Anything else goes to LibTorch."""
+    if (not isinstance(other_tensor, torch.Tensor) or self_tensor.dtype != torch.float16 or
+            other_tensor.dtype != torch.float16 or not self_tensor.is_cuda or not other_tensor.is_cuda or
+            not _custom_add_dims_ok(self_tensor, other_tensor)):
+        return torch.add(self_tensor, other_tensor, alpha=alpha, out=out)
+    lib = L.load()
+    _ensure_init(self_tensor)
+    a, b = self_tensor.contiguous(), other_tensor.contiguous()
+    n = a.size(-1)
+    m = a.numel() // n if n else 0
+    sym = a.dim() == b.dim()
+    if (sym and b.numel() != a.numel()) or (not sym and b.numel() != n):
+        return torch.add(self_tensor, other_tensor, alpha=alpha, out=out)
+    if out is None:
+        out = torch.empty_like(a)
+    elif out.dtype != torch.float16 or not out.is_cuda or out.numel() != a.numel() or not out.is_contiguous():
+        raise NNRuntimeException("`out` must be a contiguous fp16 GPU buffer with as many elements as `self`")
+    _check(lib.pimhip_execute_add(out.data_ptr(), a.data_ptr(), b.data_ptr(), m, n, int(not sym), _stream_handle(stream)))
+    return out
+
+
+def _custom_add_dims_ok(t1, t2):
+    """customAddDimensionsCheck (aten_ops_executor.cpp:87-109) on the larger-rank operand first."""
+    s1, s2 = (t1.shape, t2.shape) if t1.dim() >= t2.dim() else (t2.shape, t1.shape)
+    if len(s1) in (1, 2):
+        return True
+    if len(s1) == 3:
+        return not (s1[0] != 1 or (len(s2) == 3 and s2[0] != 1))
+    if len(s1) == 4:
+        return not ((len(s2) == 4 and s1[0] != s2[0]) or s1[1] != 1 or (len(s2) == 4 and s2[1] != 1) or
+                    (len(s2) == 3 and s2[0] != 1))
+    return False
+
+
 def input_projection(x, w, bias=None, stream=None):
     """out[T, N] fp32 = x[T, K] . w[N, K]^T + bias[N] (fp32) on the matrix cores."""
     lib = L.load()
@@ -396,8 +466,11 @@ class LstmPlan:
         torch.cuda.synchronize(self.device)
         _check(L.load().pimhip_lstm_plan_status(self._handle))
 
-    def forward(self, x2d, h0, c0, stream=None):
-        """x2d [T, I]; h0, c0 [L*D, H] (any shape with those elements).  Returns y [T, D*H], hn, cn [L*D, H]."""
+    def forward(self, x2d, h0, c0, stream=None, out=None):
+        """x2d [T, I]; h0, c0 [L*D, H] (any shape with those elements).  Returns y [T, D*H], hn, cn [L*D, H].
+
+        `out` = (y, hn, cn) preallocated contiguous fp16 buffers lets a decoder step write its results straight into
+        the buffers that consume them (the GNMT concatenation buffers, miopen_ops_executor.cpp:170-228)."""
         lib = L.load()
         _require_half_cuda(x2d, h0, c0)
         T = x2d.size(0)
@@ -407,9 +480,16 @@ class LstmPlan:
         if h0.numel() != n_state or c0.numel() != n_state:
             raise NNRuntimeException(f"h0 / c0 must have {n_state} elements")
         x2d, h0, c0 = x2d.contiguous(), h0.contiguous(), c0.contiguous()
-        y = torch.empty((T, self.num_dirs * self.hidden), dtype=torch.float16, device=self.device)
-        hn = torch.empty((self.num_layers * self.num_dirs, self.hidden), dtype=torch.float16, device=self.device)
-        cn = torch.empty_like(hn)
+        if out is not None:
+            y, hn, cn = out
+            _require_half_cuda(y, hn, cn)
+            if (y.numel() != T * self.num_dirs * self.hidden or hn.numel() != n_state or cn.numel() != n_state or
+                    not (y.is_contiguous() and hn.is_contiguous() and cn.is_contiguous())):
+                raise NNRuntimeException("`out` buffers must be contiguous with the sizes of y, hn and cn")
+        else:
+            y = torch.empty((T, self.num_dirs * self.hidden), dtype=torch.float16, device=self.device)
+            hn = torch.empty((self.num_layers * self.num_dirs, self.hidden), dtype=torch.float16, device=self.device)
+            cn = torch.empty_like(hn)
         _check(lib.pimhip_lstm_forward(self._handle, x2d.data_ptr(), h0.data_ptr(), c0.data_ptr(), y.data_ptr(),
                                        hn.data_ptr(), cn.data_ptr(), T, _stream_handle(stream)))
         return y, hn, cn
@@ -428,7 +508,8 @@ def _plan_for(params, has_biases, num_layers, bidirectional, seq_len):
     return plan
 
 
-def aten_lstm1(input, hx, params, has_biases, num_layers, dropout, train, bidirectional, batch_first, stream=None):
+def aten_lstm1(input, hx, params, has_biases, num_layers, dropout, train, bidirectional, batch_first, stream=None,
+               out=None):
     """atenLstm1: padded-sequence aten::lstm, batch 1 (the reference's GPU LSTM hard-codes batch 1,
     miopen_ops_executor.cpp:117).  dropout is ignored as in the reference (aten_ops.cpp:333); train must be false.
     Returns (output, hy, cy) shaped like at::lstm's results."""
@@ -443,10 +524,10 @@ def aten_lstm1(input, hx, params, has_biases, num_layers, dropout, train, bidire
     T = input.size(1) if batch_first else input.size(0)
     h0, c0 = hx[0], hx[1]
     plan = _plan_for(list(params), has_biases, num_layers, bidirectional, T)
-    y, hn, cn = plan.forward(input.reshape(T, input.size(2)), h0, c0, stream)
+    y, hn, cn = plan.forward(input.reshape(T, input.size(2)), h0, c0, stream, out=out)
     D, H = plan.num_dirs, plan.hidden
-    out = y.view(1, T, D * H) if batch_first else y.view(T, 1, D * H)
-    return out, hn.view(num_layers * D, 1, H), cn.view(num_layers * D, 1, H)
+    seq = y.view(1, T, D * H) if batch_first else y.view(T, 1, D * H)
+    return seq, hn.view(num_layers * D, 1, H), cn.view(num_layers * D, 1, H)
 
 
 def aten_lstm2(data, batch_sizes, hx, params, has_biases, num_layers, dropout, train, bidirectional, stream=None):

@@ -126,3 +126,111 @@ def test_rnnt_joint_split_gemvs(ops):
     assert lib.pimhip_execute_gemv(y1.data_ptr(), fd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), 1024, 512, 1344, 0, 1, s) == 0
     assert lib.pimhip_execute_gemv(y2.data_ptr(), gd.data_ptr(), Wd.data_ptr() + 2 * 1024, None, 320, 512, 1344, 0, 1, s) == 0
     assert maxabs(y1.float() + y2.float(), want) <= 2 * TOL
+
+
+# ---- the decoder loop's other custom kernels: residual add and attention-context bmm ---------------------------
+@pytest.mark.parametrize("shape_a,shape_b", [((1, 1, 1024), (1, 1, 1024)), ((4, 1024), (4, 1024)), ((50, 1, 2048), (50, 1, 2048)),
+                                             ((4, 1024), (1024,)), ((1, 13, 768), (768,)), ((7, 20), (7, 20)), ((3, 17), (17,)),
+                                             ((1, 1, 33, 8), (1, 1, 33, 8)), ((1, 5), (1, 5))])
+def test_add_matches_oracle_and_torch(ops, shape_a, shape_b):
+    g = torch.Generator().manual_seed(sum(shape_a))
+    a, b = rnd(g, *shape_a, scale=1.0), rnd(g, *shape_b, scale=1.0)
+    want = oracle.add(a.numpy(), b.numpy())
+    c = ops.aten_add(a.to(DEV), b.to(DEV), alpha=1)
+    assert list(c.shape) == list(a.shape)
+    assert np.array_equal(c.cpu().numpy().view(np.uint16).reshape(-1), want.view(np.uint16).reshape(-1))   # bit-exact
+    assert torch.equal(c.cpu(), a + b)                                                                      # LibTorch CPU
+    # in place, as the reference does (C = A) and into a separate buffer (the GNMT concatenation buffer)
+    ad = a.to(DEV).clone()
+    assert ops.aten_add(ad, b.to(DEV), out=ad) is ad and torch.equal(ad, c)
+
+
+def test_add_falls_back_like_the_reference(ops):
+    a, b = torch.randn(2, 3, 4, 8).half().to(DEV), torch.randn(2, 3, 4, 8).half().to(DEV)   # channel != 1: not the custom path
+    assert torch.equal(ops.aten_add(a, b), a + b)
+    af = torch.randn(4, 8).to(DEV)
+    assert torch.equal(ops.aten_add(af, af, alpha=2), af + 2 * af)                            # fp32: LibTorch with alpha
+
+
+def test_add_against_the_references_own_kernel(ops):
+    ref = oracle.ref_lib()
+    if ref is None:
+        pytest.skip("oracle/_ref was not built (reference tree absent at build time)")
+    g = torch.Generator().manual_seed(2)
+    a, b, row = rnd(g, 8, 2048, scale=1.0).to(DEV), rnd(g, 8, 2048, scale=1.0).to(DEV), rnd(g, 2048, scale=1.0).to(DEV)
+    s = torch.cuda.current_stream().cuda_stream
+    out = torch.zeros_like(a)
+    ref.ref_custom_add(s, a.data_ptr(), b.data_ptr(), out.data_ptr(), 8, 2048, 1)
+    assert torch.equal(out, ops.aten_add(a, b))
+    ref.ref_custom_add(s, a.data_ptr(), row.data_ptr(), out.data_ptr(), 8, 2048, 0)
+    assert torch.equal(out, ops.aten_add(a, row))
+
+
+@pytest.mark.parametrize("k,n", [(12, 1024), (50, 1024), (341, 2048), (7, 24), (13, 1000), (1, 8)])
+def test_bmm_single_row_matches_oracle(ops, k, n):
+    g = torch.Generator().manual_seed(k + n)
+    x, A = torch.softmax(torch.randn(1, 1, k, generator=g), -1).half(), rnd(g, 1, k, n, scale=1.0)
+    want = oracle.gemv_vm(x.numpy().reshape(-1), A.numpy().reshape(k, n))
+    y = ops.aten_bmm(x.to(DEV), A.to(DEV))
+    assert list(y.shape) == [1, 1, n] and maxabs(y, torch.as_tensor(want)) <= TOL
+    assert maxabs(y, torch.bmm(x.float(), A.float())) <= TOL
+    # three destinations in one launch: what executeAtenBmm + two atenCopy_ do in the GNMT decoder
+    cat = [torch.zeros(1, 1, 2 * n, dtype=torch.float16, device=DEV) for _ in range(3)]
+    outs = [c[0, 0, n:] for c in cat]
+    first = ops.aten_bmm(x.to(DEV), A.to(DEV), outs=outs)
+    assert first is outs[0]
+    for c in cat:
+        assert torch.equal(c[0, 0, n:], y.reshape(-1)) and float(c[0, 0, :n].abs().max()) == 0.0
+
+
+def test_bmm_is_more_accurate_than_the_references_fp16_accumulation(ops):
+    ref = oracle.ref_lib()
+    if ref is None:
+        pytest.skip("oracle/_ref was not built (reference tree absent at build time)")
+    g = torch.Generator().manual_seed(4)
+    k, n = 341, 1024
+    x, A = torch.rand(1, 1, k, generator=g).half(), rnd(g, 1, k, n, scale=1.0)
+    exact = torch.bmm(x.double(), A.double()).reshape(-1)
+    y = ops.aten_bmm(x.to(DEV), A.to(DEV)).reshape(-1)
+    out = torch.zeros(n, dtype=torch.float16, device=DEV)
+    ref.ref_bmm_xAy(torch.cuda.current_stream().cuda_stream, x.to(DEV).data_ptr(), A.to(DEV).data_ptr(), out.data_ptr(), n, k)
+    err_ours = float((y.double().cpu() - exact).abs().max())
+    err_ref = float((out.double().cpu() - exact).abs().max())
+    assert err_ours <= err_ref and err_ours <= 1e-2      # outputs are of order 10: one fp16 ulp there is 7.8e-3
+    # the two differ by no more than the reference's own distance from the exact product (plus ours)
+    assert float((y.double().cpu() - out.double().cpu()).abs().max()) <= err_ref + err_ours + 1e-9
+
+
+def test_bmm_with_rows_or_batches_takes_libtorch(ops):
+    a, b = torch.randn(2, 3, 8).half().to(DEV), torch.randn(2, 8, 5).half().to(DEV)
+    assert torch.equal(ops.aten_bmm(a, b), torch.bmm(a, b))
+
+
+def test_decoder_step_writes_into_consumer_buffers(ops):
+    """seq_len == 1 LSTM step with hy / cy / y placed straight into preallocated buffers (the GNMT decoder's
+    [8, 1, 1024] state buffer and [1, 1, 2048] concatenation buffer, miopen_ops_executor.cpp:170-228)."""
+    params, x, h0, c0 = oracle.lstm_inputs(5, 1024, 1024, 1, False, 1)
+    g = torch.Generator().manual_seed(5)
+    h0, c0 = (0.3 * torch.randn(1, 1, 1024, generator=g)).half(), (0.3 * torch.randn(1, 1, 1024, generator=g)).half()
+    want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
+    state = torch.zeros(8, 1, 1024, dtype=torch.float16, device=DEV)     # (h, c) of four decoder layers
+    cat = torch.zeros(1, 1, 2048, dtype=torch.float16, device=DEV)       # [lstm output | attention context]
+    pd = [p.to(DEV) for p in params]
+    y, hy, cy = ops.aten_lstm1(x.to(DEV), (h0.to(DEV), c0.to(DEV)), pd, True, 1, 0.0, False, False, False,
+                               out=(cat[0, 0, :1024], state[2], state[3]))
+    assert y.data_ptr() == cat.data_ptr() and hy.data_ptr() == state[2].data_ptr()
+    assert maxabs(cat[0, 0, :1024], want[0]) <= 2e-3 and maxabs(state[2], want[1]) <= 2e-3 and maxabs(state[3], want[2]) <= 2e-3
+    assert float(state[:2].abs().max()) == 0.0 and float(state[4:].abs().max()) == 0.0 and float(cat[0, 0, 1024:].abs().max()) == 0.0
+
+
+def test_rnnt_encoder_lstm_on_the_references_feature_file(ops):
+    """The reference's RNNT input (examples/runtime/resource/rnnt/inputs/feature.bin, fp16 [341, 1, 240]) through a
+    2-layer H=1024 LSTM with seeded weights, against LibTorch CPU on the same tensors."""
+    import os
+    from pimaicompiler_amd import io
+    feat = io.load_tensor(os.path.join(os.path.dirname(__file__), "golden", "rnnt_feature_341x1x240_f16.bin"), [341, 1, 240], "FLOAT16")
+    params, _, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 1)
+    want = oracle.torch_lstm(feat, h0, c0, params, True, 2, False)
+    y, hn, cn = ops.aten_lstm1(feat.to(DEV), (h0.to(DEV), c0.to(DEV)), [p.to(DEV) for p in params], True, 2, 0.0, False, False, False)
+    assert list(y.shape) == [341, 1, 1024]
+    assert maxabs(y, want[0]) <= 5e-3 and maxabs(hn, want[1]) <= 5e-3 and maxabs(cn, want[2]) <= 5e-3
