@@ -184,6 +184,79 @@ def main():
     xp_us = e0.elapsed_time(e1) * 1e3 / 50
     xp_tflops = 2 * 200 * 1024 * 4096 / xp_us / 1e6
 
+    # ---- the other kernels of the path (reported beside the headline figures, not part of `value`) ---------------
+    def timed_us(fn, reps, warm=5):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(reps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    other = {}
+    # GNMT-style stack: four at::lstm calls (L0 bidirectional I=1024, L1 I=2048, L2, L3 I=1024), T=50: 250 layer-steps
+    gn = []
+    seq = torch.randn(50, 1024, device=dev).half()
+    for li, (in_w, bidir) in enumerate([(1024, True), (2048, False), (1024, False), (1024, False)]):
+        prm, _, h0g, c0g = oracle.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
+        gn.append((P.LstmPlan([q.to(dev) for q in prm], True, 1, bidir, 50), h0g.to(dev), c0g.to(dev)))
+
+    def gnmt_stack():
+        cur = seq
+        for plan_g, hg, cg in gn:
+            cur, _, _ = plan_g.forward(cur, hg, cg)
+
+    other["gnmt_lstm_stack_us_per_layer_step"] = round(timed_us(gnmt_stack, 30) / 250, 3)
+    # one decoder step (seq_len 1, I = H = 1024): the fused step kernel, W_ih and W_hh streamed once (16.8 MB)
+    prm, _, h0d, c0d = oracle.lstm_inputs(4101, 1024, 1024, 1, False, 1)
+    plan_d = P.LstmPlan([q.to(dev) for q in prm], True, 1, False, 1)
+    xd1, h0d, c0d = torch.randn(1, 1024, device=dev).half(), h0d.to(dev).contiguous(), c0d.to(dev).contiguous()
+    yd1, hnd, cnd = torch.empty(1024, dtype=torch.float16, device=dev), torch.empty_like(h0d), torch.empty_like(c0d)
+    # (these small launches are timed through the C ABI on preallocated buffers: the operator layer's Python
+    # bookkeeping costs more than the kernels)
+    us = timed_us(lambda: lib.pimhip_lstm_forward(plan_d._handle, xd1.data_ptr(), h0d.data_ptr(), c0d.data_ptr(), yd1.data_ptr(),
+                                                  hnd.data_ptr(), cnd.data_ptr(), 1, sh), 200)
+    other["lstm_decode_step"] = {"us": round(us, 3), "gbs": round((2 * 4096 * 2048 + 8 * 4096) / us / 1e3, 1)}
+    # the same sweep as ONE grouped launch (executeMultiStream's siblings in one grid), cold
+    def grouped():
+        ws = []
+        for s_ in shapes:
+            ws.append(s_["pool"][s_["it"] % s_["copies"]])
+            s_["it"] += 1
+        P.execute_gemv_group([s_["x"] for s_ in shapes], ws, [s_["b"] for s_ in shapes])
+    us = timed_us(grouped, 100)
+    other["gemv_sweep_grouped_launch"] = {"us": round(us, 2), "gbs": round(step_bytes / us / 1e3, 1)}
+    # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
+    big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
+    big_c = torch.empty_like(big_a)
+    us = timed_us(lambda: P.aten_add(big_a, big_b, out=big_c), 50)
+    other["add_32Mi"] = {"us": round(us, 2), "gbs": round(6 * (32 << 20) / us / 1e3, 1)}
+    sa, sb = big_a[:1].reshape(1, 1, 1024), big_b[:1].reshape(1, 1, 1024)
+    other["add_1024_us"] = round(timed_us(lambda: lib.pimhip_execute_add(sa.data_ptr(), sa.data_ptr(), sb.data_ptr(), 1, 1024, 0, sh), 200), 3)
+    del big_a, big_b, big_c
+    # attention context: y[1, 1024] = p[1, 50] . enc[50, 1024], stored to three buffers
+    pa, enc = torch.rand(1, 1, 50, device=dev).half(), torch.randn(1, 50, 1024, device=dev).half()
+    dsts = [torch.empty(1024, dtype=torch.float16, device=dev) for _ in range(3)]
+    import ctypes
+    dst_arr = (ctypes.c_void_p * 3)(*[d_.data_ptr() for d_ in dsts])
+    other["bmm_50x1024_three_destinations_us"] = round(
+        timed_us(lambda: lib.pimhip_execute_bmm(dst_arr, 3, pa.data_ptr(), enc.data_ptr(), 50, 1024, sh), 200), 3)
+    # the reference's own HIP GEMV (custom_ops.h addmv_kernel_Axy, compiled from its tree) on the same cold weights
+    ref = oracle.ref_lib()
+    if ref is not None:
+        ref_times = []
+        for s_ in shapes:
+            def ref_launch(s_=s_):
+                w = s_["pool"][s_["it"] % s_["copies"]]
+                s_["it"] += 1
+                ref.ref_addmv_Axy(sh, s_["b"].data_ptr(), w.data_ptr(), s_["x"].data_ptr(), s_["y"].data_ptr(), s_["n"], s_["k"], 0)
+            us = timed_us(ref_launch, 30)
+            ref_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
+        other["reference_hip_gemv_kernel"] = ref_times
+
     # ---- CPU baseline: LibTorch CPU at::addmm in fp16 on the same sweep, bounded sample ---------------------------
     cpu = None
     if not args.no_cpu_baseline:
@@ -205,6 +278,13 @@ def main():
             t_total += med
             b_total += gemv_bytes(s["n"], s["k"])
             detail.append(f"{s['n']}x{s['k']}: {med * 1e3:.2f} ms")
+        # LibTorch CPU at::lstm on the LSTM configuration (fp16, as the reference's atenLstm1 calls it)
+        pc = [q for q in params]
+        torch.lstm(x, (h0, c0), pc, True, 2, 0.0, False, False, False)
+        t = time.perf_counter()
+        for _ in range(3):
+            torch.lstm(x, (h0, c0), pc, True, 2, 0.0, False, False, False)
+        other["cpu_libtorch_lstm_us_per_layer_step"] = round((time.perf_counter() - t) / 3 / 400 * 1e6, 1)
         cpu = dict(value=round(b_total / t_total / 1e9, 2), unit="GB/s", cores=threads, kind="reference",
                    sample="LibTorch CPU at::addmm(b, x, W^T) in fp16, the op atenAddmm passes through to: median of <= 20 "
                           "runs (<= 4 s) per sweep shape after 2 warm-ups, same weight every run (cache-warm), one pass of the "
@@ -233,6 +313,7 @@ def main():
         "lstm_config": "2 layers unidirectional, I=240, H=1024, T=200, batch 1 (400 layer-steps per call, input projection included)",
         "input_projection": {"shape": "T=200, I=1024, 4H=4096", "us": round(xp_us, 2), "tflops": round(xp_tflops, 2),
                              "mfma_utilisation": round(xp_tflops / MFMA_FP16_PEAK_TFLOPS, 5)},
+        "other_kernels": other,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": roofline,
         "cpu_baseline": cpu,

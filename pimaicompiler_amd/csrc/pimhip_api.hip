@@ -150,6 +150,8 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     int slices = (4 * st->num_cus + col_blocks - 1) / col_blocks;
     const int max_slices = (int)((K + 31) / 32);
     if (slices > max_slices) slices = max_slices;
+    // A weight of a few hundred KB is latency-bound: the cross-block reduction would cost more than it spreads.
+    if ((int64_t)K * N * (int64_t)sizeof(half_t) <= 256 * 1024) slices = 1;
     if (slices < 1) slices = 1;
     int k_per_slice = (int)((K + slices - 1) / slices);
     k_per_slice = (k_per_slice + WAVES - 1) / WAVES * WAVES;
