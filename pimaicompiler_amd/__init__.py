@@ -5,6 +5,7 @@ The compute lives in libpimhip.so (hand-written HIP kernels behind the C ABI of 
 which are used for device memory and streams only.
 """
 from . import _lib  # noqa: F401
+from . import executor, io, rewrite  # noqa: F401
 from .ops import (  # noqa: F401
     NNRuntimeException,
     GemmType,

@@ -1,0 +1,366 @@
+"""Executor-level entry points of the hot path: layer records, the blob store and the `execute*` functions.
+
+Mirrors, for the layer types on this path only, what the reference's interpreter does per layer
+(paths relative to the reference tree):
+
+    StreamExecutor.update_blob / find_blob   runtime/source/executor/stream_executor.cpp:260-280
+    execute_aten_addmm[_with_stream]         runtime/source/executor/op_executor/aten_ops_executor.cpp:181-254
+    execute_aten_matmul[_with_stream]        aten_ops_executor.cpp:2488-2525
+    execute_aten_linear                      aten_ops_executor.cpp:2029-2059
+    execute_aten_lstm1 / execute_aten_lstm2  aten_ops_executor.cpp:2135-2399 (without the GNMT concatenation-buffer
+                                             side effects, :2238-2302, which belong to the model-specific glue)
+    execute_aten_add / execute_aten_bmm      aten_ops_executor.cpp:43-179, 668-747 (custom-kernel branches)
+    execute_multi_stream                     runtime/source/executor/op_executor/stream_ops_executor.cpp:27-50
+    StreamExecutor.inference                 the dispatch loop, stream_executor.cpp:153-186, for these layer types
+
+A layer attribute that holds the reference's "unset" sentinel (ir/include/common/utils.hpp:19-23: INT32_MAX for
+int, INT64_MIN for int64, DBL_MAX for double) is taken from the next input blob instead, in the reference's order.
+Tensors are torch tensors on the GPU; the arithmetic is in libpimhip.so via pimaicompiler_amd.ops.
+"""
+import enum
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+import torch
+
+from . import ops
+from .ops import NNRuntimeException
+
+INT32_MAX = 2 ** 31 - 1
+INT64_MIN = -2 ** 63
+DBL_MAX = 1.7976931348623157e308
+
+
+def is_default_int(v):
+    return v == INT32_MAX
+
+
+def is_default_int64(v):
+    return v == INT64_MIN
+
+
+def is_default_double(v):
+    return abs(v - DBL_MAX) <= 2.220446049250313e-16
+
+
+class LayerType(enum.Enum):
+    """The LayerType values of ir/include/types.h that reach this path."""
+    ATENADD = "aten::add"
+    ATENADDMM = "aten::addmm"
+    ATENBMM = "aten::bmm"
+    ATENLINEAR = "aten::linear"
+    ATENLSTM1 = "aten::lstm1"
+    ATENLSTM2 = "aten::lstm2"
+    ATENMATMUL = "aten::matmul"
+    MULTISTREAM = "multi_stream"
+
+
+class DataType(enum.Enum):
+    UNDEFINED = 0
+    TENSOR = 1
+    INT64 = 2
+    FLOAT64 = 3
+    LIST = 4
+    NONE = 5
+
+
+@dataclass
+class NNLayer:
+    """ir::NNLayer reduced to what the executors read: type, id (= position), input / output STensor ids."""
+    type: LayerType
+    id: int = 0
+    in_stensor_ids: List[int] = field(default_factory=list)
+    out_stensor_ids: List[int] = field(default_factory=list)
+    name: str = ""
+
+
+@dataclass
+class AtenAddmmLayer(NNLayer):          # ir/include/layers/aten_addmm_layer.h
+    act_type: str = "none"              # "none" | "aten::relu" | "aten::max", set by FuseActivation
+
+
+@dataclass
+class AtenLinearLayer(NNLayer):         # ir/include/layers/aten_linear_layer.h
+    weight_ids: List[int] = field(default_factory=list)
+    bias_ids: List[int] = field(default_factory=list)
+
+
+@dataclass
+class AtenLSTM1Layer(NNLayer):          # ir/include/layers/aten_lstm1_layer.h
+    has_biases: int = INT32_MAX
+    num_layers: int = INT64_MIN
+    dropout: float = DBL_MAX
+    train: int = INT32_MAX
+    bidirectional: int = INT32_MAX
+    batch_first: int = INT32_MAX
+    param_vector: List[torch.Tensor] = field(default_factory=list)   # LibTorch order, built at model-build time
+
+
+@dataclass
+class AtenLSTM2Layer(NNLayer):          # ir/include/layers/aten_lstm2_layer.h
+    has_biases: int = INT32_MAX
+    num_layers: int = INT64_MIN
+    dropout: float = DBL_MAX
+    train: int = INT32_MAX
+    bidirectional: int = INT32_MAX
+    param_vector: List[torch.Tensor] = field(default_factory=list)
+
+
+@dataclass
+class AtenAddLayer(NNLayer):            # ir/include/layers/aten_add_layer.h
+    alpha: int = INT64_MIN
+
+
+@dataclass
+class MultiStreamLayer(NNLayer):        # ir/include/layers/multi_stream_layer.h
+    layers: List[NNLayer] = field(default_factory=list)
+
+    @property
+    def layer_num(self):
+        return len(self.layers)
+
+
+class StreamExecutor:
+    """Blob store + streams + cursor, as far as the hot-path executors use them (stream_executor.h:30-179)."""
+
+    def __init__(self, layers: Optional[List[NNLayer]] = None, model_type: str = "", device=0, grouped_multi_stream=False):
+        self.layers = layers or []
+        self.model_type = model_type
+        self.device = device
+        self.global_blobs: Dict[int, Any] = {}     # id -> (DataType, value)
+        self.cursor = 0
+        self.streams: List[torch.cuda.Stream] = []
+        # True: sibling GEMVs of a MULTISTREAM layer go out as one grouped launch instead of one stream each.
+        self.grouped_multi_stream = grouped_multi_stream
+        ops.initialize(device)
+        width = max([l.layer_num for l in self.layers if isinstance(l, MultiStreamLayer)], default=0)
+        self.set_streams(width)
+
+    # stream_executor.h:124-133
+    def set_streams(self, n):
+        with torch.cuda.device(self.device):
+            self.streams = [torch.cuda.Stream() for _ in range(n)]
+
+    def get_streams(self):
+        return self.streams
+
+    def update_blob(self, blob_id, dtype, value):
+        self.global_blobs[blob_id] = (dtype, value)
+
+    def find_blob(self, blob_id):
+        return self.global_blobs.get(blob_id, (DataType.UNDEFINED, None))
+
+    def check_valid_blob_id(self, blob_id):
+        return blob_id in self.global_blobs
+
+    def set_cursor(self, c):
+        self.cursor = c
+
+    def inference(self, executors=None):
+        """The dispatch loop (stream_executor.cpp:153-186) over self.layers; MULTISTREAM sets the cursor itself."""
+        table = executors or OP_EXECUTORS
+        self.cursor = 0
+        while self.cursor < len(self.layers):
+            layer = self.layers[self.cursor]
+            table[layer.type](layer, self)
+            self.cursor += 1
+        if self.streams:
+            # The reference relies on legacy default-stream ordering after its multi-stream launches; torch streams
+            # do not block the default stream implicitly, so results are joined here.
+            cur = torch.cuda.current_stream()
+            for s in self.streams:
+                cur.wait_stream(s)
+
+
+def _tensor(executor, blob_id, what):
+    dtype, v = executor.find_blob(blob_id)
+    if not isinstance(v, torch.Tensor):
+        raise NNRuntimeException(f"{what}: blob {blob_id} is not a tensor ({dtype})")
+    return v
+
+
+# ---- GEMV family ---------------------------------------------------------------------------------------------------
+def execute_aten_addmm_with_stream(layer, executor, stream):
+    ids = layer.in_stensor_ids
+    _, iv_self = executor.find_blob(ids[0])
+    mat1, mat2 = _tensor(executor, ids[1], "addmm mat1"), _tensor(executor, ids[2], "addmm mat2")
+    alpha = beta = 1
+    if len(ids) == 5:
+        beta, alpha = int(executor.find_blob(ids[3])[1]), int(executor.find_blob(ids[4])[1])
+    if iv_self is None:
+        out = ops.custom_aten_matmul(mat1, mat2, stream=stream)
+    else:
+        out = ops.custom_aten_addmm(layer.act_type, iv_self, mat1, mat2, beta, alpha, stream=stream)
+    executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, out)
+
+
+def execute_aten_addmm(layer, executor):
+    execute_aten_addmm_with_stream(layer, executor, None)
+
+
+def execute_aten_matmul_with_stream(layer, executor, stream):
+    ids = layer.in_stensor_ids
+    out = ops.custom_aten_matmul(_tensor(executor, ids[0], "matmul self"), _tensor(executor, ids[1], "matmul other"), stream=stream)
+    executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, out)
+
+
+def execute_aten_matmul(layer, executor):
+    execute_aten_matmul_with_stream(layer, executor, None)
+
+
+def execute_aten_linear(layer, executor):
+    x = _tensor(executor, layer.in_stensor_ids[0], "linear input")
+    w = _tensor(executor, layer.weight_ids[0], "linear weight")
+    b = _tensor(executor, layer.bias_ids[0], "linear bias") if layer.bias_ids else None
+    executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, ops.aten_linear(x, w, b))
+
+
+def execute_multi_stream(layer, executor):
+    subs = layer.layers
+    for sub in subs:
+        if sub.type not in (LayerType.ATENADDMM, LayerType.ATENMATMUL):
+            raise NNRuntimeException(f"Unsupported layer type: {sub.type.value} found in multi-stream execution.")
+    if executor.grouped_multi_stream and _groupable(subs, executor):
+        _execute_grouped(subs, executor)
+    else:
+        streams = executor.get_streams()
+        cur = torch.cuda.current_stream()
+        for i, sub in enumerate(subs):
+            streams[i].wait_stream(cur)   # the siblings' inputs were produced on the current stream
+            with torch.cuda.stream(streams[i]):
+                if sub.type == LayerType.ATENADDMM:
+                    execute_aten_addmm_with_stream(sub, executor, streams[i])
+                else:
+                    execute_aten_matmul_with_stream(sub, executor, streams[i])
+    # The graph keeps the duplicated sub-layers right after this one; the main loop's increment skips the last of them.
+    executor.set_cursor(layer.id + layer.layer_num)
+
+
+def _mv_operands(sub, executor):
+    """(x, W, bias, act) if the sub-layer is an MV product W[out,in] . x[in,1] on dense 2-D weights, else None."""
+    ids = sub.in_stensor_ids
+    if sub.type == LayerType.ATENADDMM:
+        bias, w, x, act = executor.find_blob(ids[0])[1], executor.find_blob(ids[1])[1], executor.find_blob(ids[2])[1], sub.act_type
+        if len(ids) == 5:
+            return None
+    else:
+        bias, w, x, act = None, executor.find_blob(ids[0])[1], executor.find_blob(ids[1])[1], "none"
+    if not (isinstance(w, torch.Tensor) and isinstance(x, torch.Tensor)) or w.dim() != 2 or not w.is_contiguous():
+        return None
+    if x.dim() != 2 or x.size(1) != 1 or x.size(0) != w.size(1) or w.size(1) % 8 != 0:
+        return None
+    if bias is not None and not (isinstance(bias, torch.Tensor) and bias.numel() == w.size(0)):
+        return None
+    if any(t is not None and (t.dtype != torch.float16 or not t.is_cuda) for t in (x, w, bias)):
+        return None
+    if act not in ("none", "aten::relu"):
+        act = "none"            # only ReLU is an activation for the kernels (aten_ops.cpp:641-643)
+    return x, w, bias, act
+
+
+def _groupable(subs, executor):
+    return all(_mv_operands(s, executor) is not None for s in subs)
+
+
+def _execute_grouped(subs, executor):
+    quad = [_mv_operands(s, executor) for s in subs]
+    outs = ops.execute_gemv_group([q[0] for q in quad], [q[1] for q in quad], [q[2] for q in quad], [q[3] for q in quad])
+    for s, o in zip(subs, outs):
+        executor.update_blob(s.out_stensor_ids[0], DataType.TENSOR, o.view(-1, 1))
+
+
+# ---- LSTM ----------------------------------------------------------------------------------------------------------
+def _lstm_flags(layer, executor, in_id, with_batch_first):
+    ids = layer.in_stensor_ids
+    # A TensorList of parameters may sit in the inputs; the layer's own param_vector is used instead (:2162-2168).
+    if len(ids) > in_id and isinstance(executor.find_blob(ids[in_id])[1], (list, tuple)):
+        in_id += 1
+
+    def take(value, is_default):
+        nonlocal in_id
+        if is_default(value):
+            value = executor.find_blob(ids[in_id])[1]
+            in_id += 1
+        return value
+
+    has_biases = int(take(layer.has_biases, is_default_int))
+    num_layers = int(take(layer.num_layers, is_default_int64))
+    dropout = float(take(layer.dropout, is_default_double))
+    train = int(take(layer.train, is_default_int))
+    bidirectional = int(take(layer.bidirectional, is_default_int))
+    batch_first = int(take(layer.batch_first, is_default_int)) if with_batch_first else 0
+    return has_biases, num_layers, dropout, train, bidirectional, batch_first
+
+
+def _unique_in_order(ids):
+    out = []
+    for i in ids:
+        if not out or out[-1] != i:
+            out.append(i)
+    return out
+
+
+def execute_aten_lstm1(layer, executor):
+    ids = layer.in_stensor_ids
+    x = _tensor(executor, ids[0], "lstm input")
+    hx = executor.find_blob(ids[1])[1]
+    if not isinstance(hx, (list, tuple)) or len(hx) != 2:
+        raise NNRuntimeException("lstm hx must be a TensorList (h0, c0)")
+    has_biases, num_layers, dropout, train, bidirectional, batch_first = _lstm_flags(layer, executor, 2, True)
+    out_ids = _unique_in_order(layer.out_stensor_ids)
+    if len(out_ids) != 3:
+        raise NNRuntimeException("lstm needs three output ids")
+    y, hy, cy = ops.aten_lstm1(x, tuple(hx), layer.param_vector, bool(has_biases), num_layers, dropout, bool(train),
+                               bool(bidirectional), bool(batch_first))
+    for i, v in zip(out_ids, (y, hy, cy)):
+        executor.update_blob(i, DataType.TENSOR, v)
+
+
+def execute_aten_lstm2(layer, executor):
+    ids = layer.in_stensor_ids
+    data = _tensor(executor, ids[0], "lstm data")
+    batch_sizes = _tensor(executor, ids[1], "lstm batch_sizes")
+    hx = executor.find_blob(ids[2])[1]
+    if not isinstance(hx, (list, tuple)) or len(hx) != 2:
+        raise NNRuntimeException("lstm hx must be a TensorList (h0, c0)")
+    has_biases, num_layers, dropout, train, bidirectional, _ = _lstm_flags(layer, executor, 3, False)
+    y, hy, cy = ops.aten_lstm2(data, batch_sizes, tuple(hx), layer.param_vector, bool(has_biases), num_layers, dropout,
+                               bool(train), bool(bidirectional))
+    for i, v in zip(layer.out_stensor_ids[:3], (y, hy, cy)):
+        executor.update_blob(i, DataType.TENSOR, v)
+
+
+# ---- the decoder loop's custom-kernel users ---------------------------------------------------------------------------
+def execute_aten_add(layer, executor):
+    ids = layer.in_stensor_ids
+    a, b = executor.find_blob(ids[0])[1], executor.find_blob(ids[1])[1]
+    alpha = layer.alpha
+    if is_default_int64(alpha):
+        alpha = int(executor.find_blob(ids[2])[1]) if len(ids) == 3 and executor.check_valid_blob_id(ids[2]) else 1
+    if isinstance(a, int) and isinstance(b, int):
+        executor.update_blob(layer.out_stensor_ids[0], DataType.INT64, a + b * alpha)
+        return
+    if isinstance(b, torch.Tensor):
+        out = ops.aten_add(a, b, alpha=alpha)
+    else:
+        out = torch.add(a, b, alpha=alpha)
+    executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, out)
+
+
+def execute_aten_bmm(layer, executor):
+    ids = layer.in_stensor_ids
+    out = ops.aten_bmm(_tensor(executor, ids[0], "bmm self"), _tensor(executor, ids[1], "bmm other"))
+    executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, out)
+
+
+# registerOp (stream_executor.cpp:433-576) for the layer types of this path
+OP_EXECUTORS = {
+    LayerType.ATENADD: execute_aten_add,
+    LayerType.ATENADDMM: execute_aten_addmm,
+    LayerType.ATENBMM: execute_aten_bmm,
+    LayerType.ATENLINEAR: execute_aten_linear,
+    LayerType.ATENLSTM1: execute_aten_lstm1,
+    LayerType.ATENLSTM2: execute_aten_lstm2,
+    LayerType.ATENMATMUL: execute_aten_matmul,
+    LayerType.MULTISTREAM: execute_multi_stream,
+}

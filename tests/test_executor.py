@@ -1,0 +1,332 @@
+"""The executor level of the path: blob store, attribute-or-blob unboxing, cursor handling and the execute* functions.
+
+CPU tests replace the operator layer by a recorder and check which operands each executor unboxes, in the order of
+runtime/source/executor/op_executor/aten_ops_executor.cpp (addmm :181-254, linear :2029-2059, LSTM1 :2135-2307,
+LSTM2 :2309-2399, matmul :2488-2525) and stream_ops_executor.cpp:27-50.  GPU tests run the same layers for real and
+compare with the oracle and LibTorch CPU.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from pimaicompiler_amd import executor as E
+from pimaicompiler_amd.executor import DataType, LayerType
+
+TOL_GEMV = 2e-3
+TOL_LSTM = 5e-3
+
+
+class Recorder:
+    """Stands in for pimaicompiler_amd.ops: records each call, returns a marker."""
+
+    def __init__(self):
+        self.calls = []
+
+    def __getattr__(self, name):
+        def f(*a, **k):
+            self.calls.append((name, a, k))
+            if name in ("aten_lstm1", "aten_lstm2"):
+                return ("y", "hy", "cy")
+            return name
+        return f
+
+
+@pytest.fixture
+def rec(monkeypatch):
+    r = Recorder()
+    monkeypatch.setattr(E, "ops", r)
+    monkeypatch.setattr(E.torch.cuda, "Stream", lambda *a, **k: object())
+    return r
+
+
+def _blobs(ex, **kv):
+    for k, v in kv.items():
+        i = int(k[1:])
+        if isinstance(v, torch.Tensor):
+            ex.update_blob(i, DataType.TENSOR, v)
+        elif isinstance(v, (list, tuple)):
+            ex.update_blob(i, DataType.LIST, v)
+        elif v is None:
+            ex.update_blob(i, DataType.NONE, None)
+        elif isinstance(v, float):
+            ex.update_blob(i, DataType.FLOAT64, v)
+        else:
+            ex.update_blob(i, DataType.INT64, v)
+
+
+class _NoDevice:
+    def __init__(self, device):
+        pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        return False
+
+
+@pytest.fixture
+def ex(rec, monkeypatch):
+    monkeypatch.setattr(E.torch.cuda, "device", _NoDevice)
+    return E.StreamExecutor([])
+
+
+# ---- host logic (CPU) -----------------------------------------------------------------------------------------------
+def test_sentinels_are_the_reference_values():
+    assert E.is_default_int(2 ** 31 - 1) and not E.is_default_int(0)
+    assert E.is_default_int64(-2 ** 63) and not E.is_default_int64(1)
+    assert E.is_default_double(1.7976931348623157e308) and not E.is_default_double(0.0)
+
+
+def test_blob_store(ex):
+    assert ex.find_blob(7) == (DataType.UNDEFINED, None) and not ex.check_valid_blob_id(7)
+    ex.update_blob(7, DataType.INT64, 3)
+    ex.update_blob(7, DataType.INT64, 4)        # update overwrites
+    assert ex.find_blob(7) == (DataType.INT64, 4) and ex.check_valid_blob_id(7)
+
+
+def test_addmm_unboxes_three_or_five_inputs_and_routes_none_bias_to_matmul(ex, rec):
+    b, m1, m2 = torch.zeros(4), torch.zeros(1, 3), torch.zeros(3, 4)
+    _blobs(ex, b0=b, b1=m1, b2=m2, b3=2, b4=5, b9=None)
+    E.execute_aten_addmm(E.AtenAddmmLayer(LayerType.ATENADDMM, 0, [0, 1, 2], [10], act_type="aten::relu"), ex)
+    name, a, k = rec.calls[-1]
+    assert name == "custom_aten_addmm" and a[0] == "aten::relu" and a[1] is b and a[2] is m1 and a[3] is m2
+    assert a[4:] == (1, 1) and k == {"stream": None} and ex.find_blob(10) == (DataType.TENSOR, "custom_aten_addmm")
+    E.execute_aten_addmm(E.AtenAddmmLayer(LayerType.ATENADDMM, 0, [0, 1, 2, 3, 4], [11]), ex)
+    assert rec.calls[-1][1][4:] == (2, 5)       # (beta, alpha) = inputs 3 and 4
+    E.execute_aten_addmm(E.AtenAddmmLayer(LayerType.ATENADDMM, 0, [9, 1, 2], [12]), ex)
+    assert rec.calls[-1][0] == "custom_aten_matmul" and rec.calls[-1][1] == (m1, m2)
+
+
+def test_addmm_rejects_non_tensor_operands(ex):
+    _blobs(ex, b0=torch.zeros(4), b1=3, b2=torch.zeros(3, 4))
+    with pytest.raises(E.NNRuntimeException):
+        E.execute_aten_addmm(E.AtenAddmmLayer(LayerType.ATENADDMM, 0, [0, 1, 2], [10]), ex)
+
+
+def test_linear_takes_weight_and_bias_from_the_layer_ids(ex, rec):
+    x, w, b = torch.zeros(1, 3), torch.zeros(4, 3), torch.zeros(4)
+    _blobs(ex, b0=x, b20=w, b21=b)
+    E.execute_aten_linear(E.AtenLinearLayer(LayerType.ATENLINEAR, 0, [0], [5], weight_ids=[20], bias_ids=[21]), ex)
+    assert rec.calls[-1][1] == (x, w, b)
+    E.execute_aten_linear(E.AtenLinearLayer(LayerType.ATENLINEAR, 0, [0], [5], weight_ids=[20]), ex)
+    assert rec.calls[-1][1] == (x, w, None)
+
+
+def test_lstm1_flags_from_attributes(ex, rec):
+    x, h, c = torch.zeros(5, 1, 8), torch.zeros(2, 1, 8), torch.zeros(2, 1, 8)
+    _blobs(ex, b0=x, b1=[h, c])
+    params = [torch.zeros(1)]
+    layer = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1], [7, 8, 9], has_biases=1, num_layers=2, dropout=0.0, train=0,
+                             bidirectional=0, batch_first=0, param_vector=params)
+    E.execute_aten_lstm1(layer, ex)
+    name, a, _ = rec.calls[-1]
+    assert name == "aten_lstm1" and a[0] is x and a[1] == (h, c) and a[2] is params
+    assert a[3:] == (True, 2, 0.0, False, False, False)
+    assert [ex.find_blob(i)[1] for i in (7, 8, 9)] == ["y", "hy", "cy"]
+
+
+def test_lstm1_unset_attributes_come_from_the_following_blobs_in_order(ex, rec):
+    """has_biases, num_layers, dropout, train, bidirectional, batch_first — each one only if its attribute is the
+    sentinel; a parameter TensorList in slot 2 is skipped (aten_ops_executor.cpp:2162-2206)."""
+    x, h, c = torch.zeros(5, 1, 8), torch.zeros(1, 1, 8), torch.zeros(1, 1, 8)
+    _blobs(ex, b0=x, b1=[h, c], b2=[torch.zeros(1)], b3=1, b4=3, b5=0.25, b6=0, b7=1, b8=1)
+    layer = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1, 2, 3, 4, 5, 6, 7, 8], [7, 7, 8, 9])
+    E.execute_aten_lstm1(layer, ex)
+    assert rec.calls[-1][1][3:] == (True, 3, 0.25, False, True, True)
+    # mixed: num_layers and train fixed in the layer, the others from blobs 2.. in order
+    _blobs(ex, b2=0, b3=0.5, b4=1, b5=0)
+    layer = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1, 2, 3, 4, 5], [7, 8, 9], num_layers=4, train=0)
+    E.execute_aten_lstm1(layer, ex)
+    assert rec.calls[-1][1][3:] == (False, 4, 0.5, False, True, False)
+
+
+def test_lstm1_needs_a_pair_of_states_and_three_outputs(ex):
+    _blobs(ex, b0=torch.zeros(5, 1, 8), b1=torch.zeros(1, 1, 8), b2=[torch.zeros(1, 1, 8)] * 2)
+    full = dict(has_biases=1, num_layers=1, dropout=0.0, train=0, bidirectional=0, batch_first=0)
+    with pytest.raises(E.NNRuntimeException):
+        E.execute_aten_lstm1(E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1], [7, 8, 9], **full), ex)
+    with pytest.raises(E.NNRuntimeException):
+        E.execute_aten_lstm1(E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 2], [7, 8], **full), ex)
+
+
+def test_lstm2_operand_order(ex, rec):
+    data, bs, h, c = torch.zeros(5, 8), torch.ones(5, dtype=torch.int64), torch.zeros(1, 1, 8), torch.zeros(1, 1, 8)
+    _blobs(ex, b0=data, b1=bs, b2=[h, c], b3=1, b4=1, b5=0.0, b6=0, b7=0)
+    E.execute_aten_lstm2(E.AtenLSTM2Layer(LayerType.ATENLSTM2, 0, [0, 1, 2, 3, 4, 5, 6, 7], [10, 11, 12]), ex)
+    name, a, _ = rec.calls[-1]
+    assert name == "aten_lstm2" and a[0] is data and a[1] is bs and a[2] == (h, c)
+    assert a[4:] == (True, 1, 0.0, False, False)
+
+
+def test_multi_stream_issues_each_sibling_on_its_own_stream_and_moves_the_cursor(rec, monkeypatch):
+    monkeypatch.setattr(E.torch.cuda, "device", _NoDevice)
+
+    class FakeStream:
+        def wait_stream(self, other):
+            pass
+
+    class FakeCtx(_NoDevice):
+        pass
+
+    monkeypatch.setattr(E.torch.cuda, "Stream", lambda *a, **k: FakeStream())
+    monkeypatch.setattr(E.torch.cuda, "current_stream", lambda *a, **k: FakeStream())
+    monkeypatch.setattr(E.torch.cuda, "stream", FakeCtx)
+    subs = [E.AtenAddmmLayer(LayerType.ATENADDMM, 4, [0, 1, 2], [10]), E.NNLayer(LayerType.ATENMATMUL, 5, [1, 2], [11]),
+            E.AtenAddmmLayer(LayerType.ATENADDMM, 6, [0, 1, 2], [12])]
+    ms = E.MultiStreamLayer(LayerType.MULTISTREAM, 3, layers=subs)
+    ex = E.StreamExecutor([ms])
+    assert len(ex.get_streams()) == 3
+    _blobs(ex, b0=torch.zeros(4), b1=torch.zeros(4, 3), b2=torch.zeros(3, 1))
+    E.execute_multi_stream(ms, ex)
+    assert [c[0] for c in rec.calls if c[0] != "initialize"] == ["custom_aten_addmm", "custom_aten_matmul", "custom_aten_addmm"]
+    used = [c[2]["stream"] for c in rec.calls if c[0] != "initialize"]
+    assert used == ex.get_streams()
+    assert ex.cursor == 3 + 3                   # the loop's own increment then steps past the last duplicate
+    bad = E.MultiStreamLayer(LayerType.MULTISTREAM, 0, layers=[E.NNLayer(LayerType.ATENBMM, 1, [1, 2], [11])])
+    with pytest.raises(E.NNRuntimeException):
+        E.execute_multi_stream(bad, ex)
+
+
+def test_integer_add_stays_on_the_host(ex):
+    _blobs(ex, b0=3, b1=4)
+    E.execute_aten_add(E.AtenAddLayer(LayerType.ATENADD, 0, [0, 1], [2], alpha=2), ex)
+    assert ex.find_blob(2) == (DataType.INT64, 11)
+
+
+# ---- on the GPU -------------------------------------------------------------------------------------------------------
+DEV = "cuda:0"
+
+
+def maxabs(a, b):
+    return float((torch.as_tensor(a).detach().float().cpu().reshape(-1) - torch.as_tensor(b).detach().float().cpu().reshape(-1)).abs().max())
+
+
+def _gate_graph(seed, n_gates, out_w, in_w):
+    """T(x) already applied: x_t [in,1]; per gate an addmm(b_i, W_i, x_t) (odd gates: matmul(W_i, x_t)); the graph
+    lists the MULTISTREAM layer followed by its duplicated sub-layers, as the reference's builder leaves them."""
+    Ws, bs, x = [], [], None
+    for i in range(n_gates):
+        W, x, b = oracle.gemv_inputs(seed + i, out_w, in_w)
+        Ws.append(W)
+        bs.append(b)
+    subs, blobs = [], {"b0": x.t().to(DEV)}
+    for i in range(n_gates):
+        blobs[f"b{10 + i}"] = Ws[i].to(DEV)
+        blobs[f"b{20 + i}"] = bs[i].to(DEV)
+        if i % 2 == 0:
+            subs.append(E.AtenAddmmLayer(LayerType.ATENADDMM, 2 + i, [20 + i, 10 + i, 0], [30 + i],
+                                         act_type="aten::relu" if i == 2 else "none"))
+        else:
+            subs.append(E.NNLayer(LayerType.ATENMATMUL, 2 + i, [10 + i, 0], [30 + i]))
+    layers = [E.AtenLinearLayer(LayerType.ATENLINEAR, 0, [1], [2], weight_ids=[10], bias_ids=[20]),
+              E.MultiStreamLayer(LayerType.MULTISTREAM, 1, layers=subs)] + subs
+    layers.append(E.AtenLinearLayer(LayerType.ATENLINEAR, 2 + n_gates, [1], [3], weight_ids=[11]))
+    blobs["b1"] = x.to(DEV)
+    want = []
+    for i in range(n_gates):
+        want.append(oracle.gemv_mv(Ws[i].numpy(), x.numpy().reshape(-1), bs[i].numpy() if i % 2 == 0 else None, relu=(i == 2)))
+    lin = [oracle.gemv_mv(Ws[0].numpy(), x.numpy().reshape(-1), bs[0].numpy()),
+           oracle.gemv_mv(Ws[1].numpy(), x.numpy().reshape(-1), None)]
+    return layers, blobs, want, lin
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("grouped", [False, True])
+def test_inference_loop_with_a_multi_stream_layer(ops, grouped):
+    layers, blobs, want, lin = _gate_graph(100, 4, 512, 1024)
+    ex = E.StreamExecutor(layers, device=0, grouped_multi_stream=grouped)
+    _blobs(ex, **blobs)
+    calls = []
+    table = dict(E.OP_EXECUTORS)
+    for t in (LayerType.ATENADDMM, LayerType.ATENMATMUL):
+        table[t] = (lambda f: lambda l, e: (calls.append(l.id), f(l, e)))(E.OP_EXECUTORS[t])
+    ex.inference(table)
+    torch.cuda.synchronize()
+    assert calls == []                          # the duplicated sub-layers are skipped by the cursor move
+    for i, w in enumerate(want):
+        y = ex.find_blob(30 + i)[1]
+        assert list(y.shape) == [512, 1] and maxabs(y, w) <= TOL_GEMV
+    assert list(ex.find_blob(2)[1].shape) == [1, 512]
+    assert maxabs(ex.find_blob(2)[1], lin[0]) <= TOL_GEMV and maxabs(ex.find_blob(3)[1], lin[1]) <= TOL_GEMV
+
+
+@pytest.mark.gpu
+def test_grouped_and_streamed_multi_stream_agree_bit_for_bit(ops):
+    outs = []
+    for grouped in (False, True):
+        layers, blobs, _, _ = _gate_graph(7, 4, 1024, 1024)
+        ex = E.StreamExecutor(layers, device=0, grouped_multi_stream=grouped)
+        _blobs(ex, **blobs)
+        ex.inference()
+        torch.cuda.synchronize()
+        outs.append([ex.find_blob(30 + i)[1].cpu() for i in range(4)])
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+def test_addmm_vm_order_and_none_bias(ops):
+    W, x, b = oracle.gemv_inputs(3, 320, 256)
+    A = W.t().contiguous()
+    ex = E.StreamExecutor([], device=0)
+    _blobs(ex, b0=b.to(DEV), b1=x.to(DEV), b2=A.to(DEV), b3=None)
+    E.execute_aten_addmm(E.AtenAddmmLayer(LayerType.ATENADDMM, 0, [0, 1, 2], [5]), ex)
+    E.execute_aten_addmm(E.AtenAddmmLayer(LayerType.ATENADDMM, 0, [3, 1, 2], [6]), ex)
+    E.execute_aten_matmul(E.NNLayer(LayerType.ATENMATMUL, 0, [1, 2], [7]), ex)
+    assert list(ex.find_blob(5)[1].shape) == [1, 320]
+    assert maxabs(ex.find_blob(5)[1], oracle.gemv_vm(x.numpy().reshape(-1), A.numpy(), b.numpy())) <= TOL_GEMV
+    no_bias = oracle.gemv_vm(x.numpy().reshape(-1), A.numpy(), None)
+    assert maxabs(ex.find_blob(6)[1], no_bias) <= TOL_GEMV and torch.equal(ex.find_blob(6)[1], ex.find_blob(7)[1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bidirectional,num_layers", [(False, 2), (True, 1)])
+def test_lstm1_layer_with_flags_from_blobs(ops, bidirectional, num_layers):
+    params, x, h0, c0 = oracle.lstm_inputs(11, 64, 128, num_layers, bidirectional, 9)
+    g = torch.Generator().manual_seed(5)
+    h0 = (0.1 * torch.randn(h0.shape, generator=g)).half()
+    c0 = (0.1 * torch.randn(c0.shape, generator=g)).half()
+    ex = E.StreamExecutor([], device=0)
+    _blobs(ex, b0=x.to(DEV), b1=[h0.to(DEV), c0.to(DEV)], b2=[p.to(DEV) for p in params], b3=1, b4=num_layers, b5=0.0, b6=0,
+           b7=int(bidirectional), b8=0)
+    layer = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, list(range(9)), [20, 21, 22], param_vector=[p.to(DEV) for p in params])
+    E.execute_aten_lstm1(layer, ex)
+    D = 2 if bidirectional else 1
+    y, hn, cn = oracle.lstm(x.numpy().reshape(9, 64), h0.numpy(), c0.numpy(), [p.numpy() for p in params], True, num_layers,
+                            bidirectional)
+    ty, thn, tcn = oracle.torch_lstm(x, h0, c0, params, True, num_layers, bidirectional)
+    got = [ex.find_blob(i)[1] for i in (20, 21, 22)]
+    assert list(got[0].shape) == [9, 1, D * 128] and list(got[1].shape) == [num_layers * D, 1, 128]
+    for g_, o_, t_ in zip(got, (y, hn, cn), (ty, thn, tcn)):
+        assert maxabs(g_, o_) <= TOL_LSTM and maxabs(g_, t_) <= TOL_LSTM
+
+
+@pytest.mark.gpu
+def test_lstm2_layer_on_the_rnnt_feature_shape(ops):
+    params, x, h0, c0 = oracle.lstm_inputs(12, 240, 256, 2, False, 21)
+    ex = E.StreamExecutor([], device=0)
+    _blobs(ex, b0=x.reshape(21, 240).to(DEV), b1=torch.ones(21, dtype=torch.int64), b2=[h0.to(DEV), c0.to(DEV)])
+    layer = E.AtenLSTM2Layer(LayerType.ATENLSTM2, 0, [0, 1, 2], [20, 21, 22], has_biases=1, num_layers=2, dropout=0.0,
+                             train=0, bidirectional=0, param_vector=[p.to(DEV) for p in params])
+    E.execute_aten_lstm2(layer, ex)
+    y, hn, cn = oracle.lstm(x.numpy().reshape(21, 240), h0.numpy(), c0.numpy(), [p.numpy() for p in params], True, 2, False)
+    got = [ex.find_blob(i)[1] for i in (20, 21, 22)]
+    assert list(got[0].shape) == [21, 256]
+    for g_, o_ in zip(got, (y, hn, cn)):
+        assert maxabs(g_, o_) <= TOL_LSTM
+
+
+@pytest.mark.gpu
+def test_add_and_bmm_layers(ops):
+    g = torch.Generator().manual_seed(9)
+    a, b = torch.randn(1, 1, 1024, generator=g).half(), torch.randn(1, 1, 1024, generator=g).half()
+    q, keys = (0.1 * torch.randn(1, 1, 40, generator=g)).half(), torch.randn(1, 40, 1024, generator=g).half()
+    ex = E.StreamExecutor([], device=0)
+    _blobs(ex, b0=a.to(DEV), b1=b.to(DEV), b2=q.to(DEV), b3=keys.to(DEV), b4=1)
+    E.execute_aten_add(E.AtenAddLayer(LayerType.ATENADD, 0, [0, 1, 4], [5]), ex)
+    E.execute_aten_bmm(E.NNLayer(LayerType.ATENBMM, 0, [2, 3], [6]), ex)
+    assert np.array_equal(ex.find_blob(5)[1].cpu().numpy(), oracle.add(a.numpy(), b.numpy()).reshape(1, 1, 1024))
+    want = oracle.gemv_vm(q.numpy().reshape(-1), keys.numpy().reshape(40, 1024), None)
+    assert list(ex.find_blob(6)[1].shape) == [1, 1, 1024] and maxabs(ex.find_blob(6)[1], want) <= TOL_GEMV
