@@ -81,6 +81,8 @@ class AtenAddmmLayer(NNLayer):          # ir/include/layers/aten_addmm_layer.h
 
 @dataclass
 class AtenLinearLayer(NNLayer):         # ir/include/layers/aten_linear_layer.h
+    weights: List[torch.Tensor] = field(default_factory=list)        # host tensors until the model is preloaded
+    biases: List[torch.Tensor] = field(default_factory=list)
     weight_ids: List[int] = field(default_factory=list)
     bias_ids: List[int] = field(default_factory=list)
 
@@ -93,6 +95,10 @@ class AtenLSTM1Layer(NNLayer):          # ir/include/layers/aten_lstm1_layer.h
     train: int = INT32_MAX
     bidirectional: int = INT32_MAX
     batch_first: int = INT32_MAX
+    weights: List[torch.Tensor] = field(default_factory=list)        # per layer x direction: w_ih, w_hh
+    biases: List[torch.Tensor] = field(default_factory=list)         # per layer x direction: b_ih, b_hh
+    weight_ids: List[int] = field(default_factory=list)
+    bias_ids: List[int] = field(default_factory=list)
     param_vector: List[torch.Tensor] = field(default_factory=list)   # LibTorch order, built at model-build time
 
 
@@ -103,6 +109,10 @@ class AtenLSTM2Layer(NNLayer):          # ir/include/layers/aten_lstm2_layer.h
     dropout: float = DBL_MAX
     train: int = INT32_MAX
     bidirectional: int = INT32_MAX
+    weights: List[torch.Tensor] = field(default_factory=list)
+    biases: List[torch.Tensor] = field(default_factory=list)
+    weight_ids: List[int] = field(default_factory=list)
+    bias_ids: List[int] = field(default_factory=list)
     param_vector: List[torch.Tensor] = field(default_factory=list)
 
 
@@ -164,12 +174,84 @@ class StreamExecutor:
             layer = self.layers[self.cursor]
             table[layer.type](layer, self)
             self.cursor += 1
-        if self.streams:
-            # The reference relies on legacy default-stream ordering after its multi-stream launches; torch streams
-            # do not block the default stream implicitly, so results are joined here.
-            cur = torch.cuda.current_stream()
-            for s in self.streams:
-                cur.wait_stream(s)
+
+
+class ModelBuilder:
+    """Weight preload for the layers of this path (runtime/source/builder/model_builder.cpp:18-224).
+
+    pre_process finds the first free blob id; preload_model moves each LINEAR / LSTM layer's weights and biases to the
+    GPU under fresh ids, and for an LSTM whose flags are all set builds the LibTorch-ordered parameter vector.  Where
+    the reference then packs a MIOpen weight buffer (reArangeLstmWeights, :226-319), this build prepares the recurrence
+    plan (bias sums, projection and exchange buffers) for the layer once, so no call allocates later.
+    """
+
+    def __init__(self, device=0):
+        self.device = torch.device("cuda", device) if isinstance(device, int) else torch.device(device)
+        self.preload_id = 0
+        self.preloaded_data_container: Dict[int, Any] = {}
+
+    def pre_process(self, layers):
+        for layer in _flatten(layers):
+            for i in layer.out_stensor_ids:
+                self.preload_id = max(self.preload_id, i)
+        self.preload_id += 1
+
+    def load_weight_and_bias(self, weight_data, bias_data):
+        ids = ([], [])
+        for dst, group in zip(ids, (weight_data, bias_data)):
+            for t in group:
+                self.preloaded_data_container[self.preload_id] = (DataType.TENSOR, t.to(self.device))
+                dst.append(self.preload_id)
+                self.preload_id += 1
+        return ids
+
+    @staticmethod
+    def feasible_for_lstm_weight_process(layer):
+        unset = [is_default_int(layer.has_biases), is_default_int64(layer.num_layers), is_default_double(layer.dropout),
+                 is_default_int(layer.train), is_default_int(layer.bidirectional)]
+        if isinstance(layer, AtenLSTM1Layer):
+            unset.append(is_default_int(layer.batch_first))
+        return not any(unset)
+
+    def build_lstm_parameter_vector(self, layer):
+        assert layer.bidirectional in (0, 1)
+        params = []
+        for i in range(layer.num_layers * (layer.bidirectional + 1)):
+            params.append(self.preloaded_data_container[layer.weight_ids[2 * i]][1])
+            params.append(self.preloaded_data_container[layer.weight_ids[2 * i + 1]][1])
+            if layer.has_biases:
+                params.append(self.preloaded_data_container[layer.bias_ids[2 * i]][1])
+                params.append(self.preloaded_data_container[layer.bias_ids[2 * i + 1]][1])
+        layer.param_vector = params
+
+    def preload_model(self, layers, lstm_seq_len=64):
+        for layer in _flatten(layers):
+            if layer.type in (LayerType.ATENLSTM1, LayerType.ATENLSTM2, LayerType.ATENLINEAR):
+                if not layer.weights:
+                    continue
+                layer.weight_ids, layer.bias_ids = self.load_weight_and_bias(layer.weights, layer.biases)
+                if layer.type == LayerType.ATENLINEAR:
+                    continue
+                if not self.feasible_for_lstm_weight_process(layer):
+                    raise NNRuntimeException(f"Failed to pre-process weights for: {layer.name}")
+                self.build_lstm_parameter_vector(layer)
+                ops.prepare_lstm(layer.param_vector, bool(layer.has_biases), layer.num_layers, bool(layer.bidirectional),
+                                 lstm_seq_len)
+
+    def build(self, layers, **executor_args):
+        """pre_process + preload_model + a StreamExecutor whose blob store starts from the preloaded container."""
+        self.pre_process(layers)
+        self.preload_model(layers)
+        ex = StreamExecutor(layers, device=self.device.index or 0, **executor_args)
+        ex.global_blobs.update(self.preloaded_data_container)
+        return ex
+
+
+def _flatten(layers):
+    for layer in layers:
+        yield layer
+        if isinstance(layer, MultiStreamLayer):
+            yield from layer.layers
 
 
 def _tensor(executor, blob_id, what):
@@ -232,6 +314,10 @@ def execute_multi_stream(layer, executor):
                     execute_aten_addmm_with_stream(sub, executor, streams[i])
                 else:
                     execute_aten_matmul_with_stream(sub, executor, streams[i])
+        # The reference's streams are ordered against its null stream implicitly; these are not, so the issuing
+        # stream waits (on the GPU, not the host) for the siblings before any consumer is enqueued.
+        for i in range(len(subs)):
+            cur.wait_stream(streams[i])
     # The graph keeps the duplicated sub-layers right after this one; the main loop's increment skips the last of them.
     executor.set_cursor(layer.id + layer.layer_num)
 

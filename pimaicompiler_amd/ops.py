@@ -508,6 +508,13 @@ def _plan_for(params, has_biases, num_layers, bidirectional, seq_len):
     return plan
 
 
+def prepare_lstm(params, has_biases, num_layers, bidirectional, max_seq_len=64):
+    """One-time weight preparation for an LSTM layer stack, done where the reference packs its MIOpen weight buffer
+    (ModelBuilder::reArangeLstmWeights, runtime/source/builder/model_builder.cpp:226-319): later aten_lstm1/2 calls
+    with the same parameter tensors and at most `max_seq_len` steps allocate no plan."""
+    return _plan_for(list(params), has_biases, num_layers, bidirectional, max_seq_len)
+
+
 def aten_lstm1(input, hx, params, has_biases, num_layers, dropout, train, bidirectional, batch_first, stream=None,
                out=None):
     """atenLstm1: padded-sequence aten::lstm, batch 1 (the reference's GPU LSTM hard-codes batch 1,

@@ -195,6 +195,33 @@ def test_integer_add_stays_on_the_host(ex):
     assert ex.find_blob(2) == (DataType.INT64, 11)
 
 
+def test_builder_assigns_fresh_ids_and_orders_lstm_parameters(rec, monkeypatch):
+    """model_builder.cpp:18-224: ids start after the largest output id; weights before biases per layer; the
+    parameter vector is (w_ih, w_hh, b_ih, b_hh) per layer and direction."""
+    monkeypatch.setattr(E.torch.cuda, "device", _NoDevice)
+    w = [torch.full((1,), float(i)) for i in range(4)]      # l0 fwd w_ih, w_hh, l0 bwd w_ih, w_hh
+    b = [torch.full((1,), 10.0 + i) for i in range(4)]
+    lstm = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1], [4, 5, 6], has_biases=1, num_layers=1, dropout=0.0, train=0,
+                            bidirectional=1, batch_first=0, weights=w, biases=b)
+    lin = E.AtenLinearLayer(LayerType.ATENLINEAR, 1, [4], [9], weights=[torch.zeros(2, 2)], biases=[torch.zeros(2)])
+    mb = E.ModelBuilder(device="cpu")
+    ex = mb.build([lstm, lin])
+    assert lstm.weight_ids == [10, 11, 12, 13] and lstm.bias_ids == [14, 15, 16, 17]
+    assert lin.weight_ids == [18] and lin.bias_ids == [19]
+    assert [float(p) for p in lstm.param_vector] == [0, 1, 10, 11, 2, 3, 12, 13]
+    assert ex.find_blob(18)[1] is mb.preloaded_data_container[18][1]
+    prep = [c for c in rec.calls if c[0] == "prepare_lstm"]
+    assert len(prep) == 1 and prep[0][1][1:4] == (True, 1, True)
+
+
+def test_builder_refuses_an_lstm_with_unset_flags(rec, monkeypatch):
+    monkeypatch.setattr(E.torch.cuda, "device", _NoDevice)
+    lstm = E.AtenLSTM2Layer(LayerType.ATENLSTM2, 0, [0, 1, 2], [4, 5, 6], has_biases=1, num_layers=1, train=0,
+                            bidirectional=0, weights=[torch.zeros(1)] * 2, biases=[torch.zeros(1)] * 2)   # dropout unset
+    with pytest.raises(E.NNRuntimeException):
+        E.ModelBuilder(device="cpu").build([lstm])
+
+
 # ---- on the GPU -------------------------------------------------------------------------------------------------------
 DEV = "cuda:0"
 
@@ -330,3 +357,27 @@ def test_add_and_bmm_layers(ops):
     assert np.array_equal(ex.find_blob(5)[1].cpu().numpy(), oracle.add(a.numpy(), b.numpy()).reshape(1, 1, 1024))
     want = oracle.gemv_vm(q.numpy().reshape(-1), keys.numpy().reshape(40, 1024), None)
     assert list(ex.find_blob(6)[1].shape) == [1, 1, 1024] and maxabs(ex.find_blob(6)[1], want) <= TOL_GEMV
+
+
+@pytest.mark.gpu
+def test_built_model_lstm_then_linear_on_the_rnnt_feature(ops):
+    """Preload + inference of a two-layer LSTM followed by a linear on its last output row."""
+    from pimaicompiler_amd import io
+    import os
+    feat = io.load_tensor(os.path.join(os.path.dirname(__file__), "golden", "rnnt_feature_341x1x240_f16.bin"), [341, 1, 240], "FLOAT16")
+    x = feat[:30].contiguous()
+    params, _, h0, c0 = oracle.lstm_inputs(21, 240, 128, 2, False, 30)
+    W, _, b = oracle.gemv_inputs(22, 64, 128)
+    lstm = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1], [2, 3, 4], has_biases=1, num_layers=2, dropout=0.0, train=0,
+                            bidirectional=0, batch_first=0, weights=[params[i] for i in (0, 1, 4, 5)],
+                            biases=[params[i] for i in (2, 3, 6, 7)])
+    lin = E.AtenLinearLayer(LayerType.ATENLINEAR, 1, [3], [5], weights=[W], biases=[b])
+    ex = E.ModelBuilder(device=0).build([lstm, lin])
+    assert [tuple(p.shape) for p in lstm.param_vector] == [tuple(p.shape) for p in params]
+    _blobs(ex, b0=x.to(DEV), b1=[h0.to(DEV), c0.to(DEV)])
+    ex.inference()
+    y, hn, cn = oracle.lstm(x.numpy().reshape(30, 240), h0.numpy(), c0.numpy(), [p.numpy() for p in params], True, 2, False)
+    assert maxabs(ex.find_blob(2)[1], y) <= TOL_LSTM and maxabs(ex.find_blob(3)[1], hn) <= TOL_LSTM
+    want = np.stack([oracle.gemv_mv(W.numpy(), hn[l], b.numpy()) for l in range(2)])
+    got = ex.find_blob(5)[1]
+    assert list(got.shape) == [2, 1, 64] and maxabs(got, want) <= 5e-3
