@@ -5,7 +5,8 @@
 // values of row (l % 16), starting at K offset 8 * (l / 16), for A (x) and for B (w) alike, and
 // receives out rows 4 * (l / 16) .. + 3 of column (l % 16).
 //
-// Grid: one block of 256 lanes per 16 * NT output columns and 64 time steps.  Requirements checked by the launcher:
+// Grid (1-D): one block of 256 lanes per 16 * NT output columns and 64 time steps, 8 * ceil(column tiles / 8) * row
+// blocks in all.  Requirements checked by the launcher:
 // K % 8 == 0, 16-byte aligned x and w, row pitches % 8 == 0.
 #pragma once
 
@@ -13,38 +14,63 @@
 
 namespace pimhip
 {
-// What bounds this kernel is the rate at which one CU can pull bytes in from L2 with fragment-shaped loads (measured:
-// about 32 GB/s per CU on MI355X, whatever the loop structure, unrolling or LDS staging), not the matrix cores.  The run
-// time is therefore (bytes a block reads) / 32 GB/s, and the tiling minimises that at full CU coverage: a block computes
-// 64 time steps x 16 * NT columns and each of its four wavefronts takes a quarter of the K range for the whole tile
-// (4 x NT MFMA tiles), i.e. (64 + 16 * NT) x K halves per block (256 KB at K = 1024, NT = 4, against 448 KB for a
-// 208 x 16 tile); the four K quarters are added through LDS in a fixed order at the end.
-static constexpr int kXprojTile = 64;    // time steps and output columns per block
-static constexpr int kXprojKSplit = 4;   // K quarters per block, one per wavefront
-static constexpr int kXprojUnroll = 2;   // K steps (of 32) whose 16 fragment loads are issued together
+// A fragment-shaped load straight from global memory (16 lanes on 16 different rows) makes the vector cache look up one
+// line per lane, which caps a CU at about 16 bytes per clock (measured: ~35 GB/s per CU, whatever the unrolling).  So
+// the operands go through LDS, which only serves as a layout converter: the block reads 128-column slabs of its 64 x rows
+// and 16 * NT w rows with row-contiguous 16-byte loads (16 adjacent lanes = 256 contiguous bytes), keeps the next slab in
+// registers while the current one is multiplied, and every wavefront reads its fragments from LDS with ds_read_b128 (row
+// pitch 272 bytes: 16 lanes x 16 bytes fall into 64 distinct banks).  The four wavefronts split K inside a slab (one
+// 32-wide MFMA step each) and each accumulates the whole 64 x 16 * NT tile; the four partial tiles are added through LDS
+// in a fixed order at the end.
+static constexpr int kXprojTile = 64;    // time steps per block
+static constexpr int kXprojKSplit = 4;   // wavefronts per block = MFMA K steps per slab
+static constexpr int kXprojSlab = 32 * kXprojKSplit;  // K values per slab (128)
+static constexpr int kXprojPitch = kXprojSlab + 8;    // LDS row pitch in halves (272 bytes)
 
-template <int NT>  // column tiles of 16 per block: 4 for long sequences, fewer when there are too few row blocks to fill the CUs
+// NT: column tiles of 16 per block (2, or 1 when a single row block would leave CUs without work).
+template <int NT>
 __global__ __launch_bounds__(256) void input_projection_f16_kernel(const half_t* __restrict__ x,
                                                                   const half_t* __restrict__ w,
                                                                   const float* __restrict__ bias,
                                                                   float* __restrict__ out, int T, int K, int N, long ldx,
-                                                                  long ldw)
+                                                                  long ldw, int row_blocks)
 {
-    __shared__ __align__(16) float red[kXprojKSplit][4 * NT][64][4];  // [K quarter][4 x NT MFMA tile][lane][4 rows]: up to 64 KB
+    constexpr int ROWS = kXprojTile + 16 * NT;            // LDS rows per slab: x rows first, then w rows
+    constexpr int CHUNKS = ROWS * (kXprojSlab / 8);       // 16-byte pieces per slab
+    constexpr int PER_LANE = CHUNKS / 256;                // 5, 6 or 8
+    static_assert(CHUNKS % 256 == 0, "slab must divide evenly over the block");
+    constexpr int SLAB_BYTES = ROWS * kXprojPitch * 2;
+    constexpr int RED_BYTES = kXprojKSplit * 4 * NT * 64 * 16;
+    constexpr int LDS_BYTES = 2 * SLAB_BYTES > RED_BYTES ? 2 * SLAB_BYTES : RED_BYTES;
+    __shared__ __align__(16) unsigned char lds[LDS_BYTES];  // two slabs while multiplying, the partial tiles afterwards
 
-    const int lane = threadIdx.x & 63;
-    const int ks = threadIdx.x >> 6;  // this wavefront's K quarter
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int ks = tid >> 6;  // this wavefront's MFMA step inside a slab
     const int r16 = lane & 15;
     const int kq = lane >> 4;  // which 8-wide K slice of a 32-wide MFMA step this lane feeds
-    const int n_base = blockIdx.x * (16 * NT);
-    const int t_base = blockIdx.y * kXprojTile;
+    // Workgroups go to the eight XCDs round-robin by linear id, and each XCD has its own L2.  All row blocks of a column
+    // tile are therefore given ids that are equal modulo 8: the tile's slice of w is then pulled into one L2 once and
+    // shared by its row blocks, instead of crossing the fabric once per row block and XCD.
+    const int xcd = blockIdx.x & 7;
+    const int local = blockIdx.x >> 3;
+    const int col_tile = (local / row_blocks) * 8 + xcd;
+    if (col_tile * (16 * NT) >= N) return;  // whole block, before any barrier
+    const int n_base = col_tile * (16 * NT);
+    const int t_base = (local % row_blocks) * kXprojTile;
 
-    const half_t* xrow[4];
-    const half_t* wrow[NT];
+    // Global side of the slab copy: piece i of this lane is row (tid + 256 i) / 16, 8-wide column (tid + 256 i) % 16.
+    const half_t* src[PER_LANE];
+    int dst[PER_LANE];  // LDS offset in halves within a slab
+    const int kcol = (tid & 15) * 8;
 #pragma unroll
-    for (int m = 0; m < 4; ++m) xrow[m] = x + (long)min(t_base + m * 16 + r16, T - 1) * ldx;  // rows past T duplicate the last row; not stored
-#pragma unroll
-    for (int n = 0; n < NT; ++n) wrow[n] = w + (long)min(n_base + n * 16 + r16, N - 1) * ldw;
+    for (int i = 0; i < PER_LANE; ++i) {
+        const int row = (tid >> 4) + 16 * i;
+        // rows past T or N duplicate the last row; their results are never stored
+        src[i] = row < kXprojTile ? x + (long)min(t_base + row, T - 1) * ldx
+                                  : w + (long)min(n_base + row - kXprojTile, N - 1) * ldw;
+        dst[i] = row * kXprojPitch + kcol;
+    }
 
     half8_t zero;
 #pragma unroll
@@ -55,41 +81,47 @@ __global__ __launch_bounds__(256) void input_projection_f16_kernel(const half_t*
 #pragma unroll
         for (int n = 0; n < NT; ++n) acc[m][n] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // This wavefront's K range, in steps of 32: [step_begin, step_end).
-    const int steps = (K + 31) >> 5;
-    const int per_quarter = (steps + kXprojKSplit - 1) / kXprojKSplit;
-    const int step_begin = ks * per_quarter;
-    const int step_end = min(steps, step_begin + per_quarter);
-
-    for (int s0 = step_begin; s0 < step_end; s0 += kXprojUnroll) {
-        half8_t a[kXprojUnroll][4], b[kXprojUnroll][NT];
+    const int slabs = (K + kXprojSlab - 1) / kXprojSlab;
+    // One register stage: the loads of slab s + 1 are issued before slab s is multiplied and written to the other LDS
+    // buffer after it.  (A second register stage, with a barrier that does not wait for global loads, measured slower.)
+    half8_t stage[PER_LANE];
+    auto fetch = [&](int slab) {
+        const int k = slab * kXprojSlab + kcol;
+        const bool ok = k < K;  // K % 8 == 0: an 8-wide piece is entirely in or out of range
+        const int kc = ok ? k : 0;
 #pragma unroll
-        for (int u = 0; u < kXprojUnroll; ++u) {
-            // Within the 32 * kXprojUnroll K values of an iteration lane group kq owns a contiguous run and feeds its
-            // u-th 8-wide piece to the u-th K step (x and w alike, so products still pair equal K indices): the four
-            // lane groups of a row then cover a whole 128-byte line with back-to-back loads instead of half of it.
-            const int k = s0 * 32 + kq * (8 * kXprojUnroll) + u * 8;
-            const bool ok = k < step_end * 32 && k < K;  // K % 8 == 0: an 8-wide slice is entirely in or out of range
-            const int kc = ok ? k : 0;                     // unconditional loads from a valid address, zeroed when out
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                const half8_t av = *reinterpret_cast<const half8_t*>(xrow[m] + kc);
-                a[u][m] = ok ? av : zero;
-            }
-#pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                const half8_t bv = *reinterpret_cast<const half8_t*>(wrow[n] + kc);
-                b[u][n] = ok ? bv : zero;
-            }
+        for (int i = 0; i < PER_LANE; ++i) {
+            const half8_t v = *reinterpret_cast<const half8_t*>(src[i] + kc);
+            stage[i] = ok ? v : zero;
         }
+    };
+    auto deposit = [&](int buf) {
+        half_t* base = reinterpret_cast<half_t*>(lds + buf * SLAB_BYTES);
 #pragma unroll
-        for (int u = 0; u < kXprojUnroll; ++u)
+        for (int i = 0; i < PER_LANE; ++i) *reinterpret_cast<half8_t*>(base + dst[i]) = stage[i];
+    };
+
+    fetch(0);
+    deposit(0);
+    __syncthreads();
+    for (int s = 0; s < slabs; ++s) {
+        if (s + 1 < slabs) fetch(s + 1);
+        const half_t* base = reinterpret_cast<const half_t*>(lds + (s & 1) * SLAB_BYTES) + ks * 32 + kq * 8;
+        half8_t a[4], b[NT];
 #pragma unroll
-            for (int m = 0; m < 4; ++m)
+        for (int m = 0; m < 4; ++m) a[m] = *reinterpret_cast<const half8_t*>(base + (m * 16 + r16) * kXprojPitch);
 #pragma unroll
-                for (int n = 0; n < NT; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][m], b[u][n], acc[m][n], 0, 0, 0);
+        for (int n = 0; n < NT; ++n) b[n] = *reinterpret_cast<const half8_t*>(base + (kXprojTile + n * 16 + r16) * kXprojPitch);
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m], b[n], acc[m][n], 0, 0, 0);
+        // Slab s + 1 goes into the other buffer, which every wavefront stopped reading before the previous barrier.
+        if (s + 1 < slabs) deposit((s + 1) & 1);
+        __syncthreads();
     }
 
+    float(*red)[4 * NT][64][4] = reinterpret_cast<float(*)[4 * NT][64][4]>(lds);  // [K split][tile][lane][4 rows]
 #pragma unroll
     for (int m = 0; m < 4; ++m)
 #pragma unroll
