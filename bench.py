@@ -30,7 +30,7 @@ POOL_BYTES_PER_SHAPE = 512 << 20
 # HBM bytes per launch of the dominant kernel, mean over its three shapes, from two rocprofv3 --pmc runs of this
 # script (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch, factors from --calibration-copy); the figures and the
 # commands are in profiles/gemv_sweep_pmc.md.  A counter reading, not something this script can measure itself.
-DOMINANT_KERNEL_TRAFFIC_BYTES = int((131425.0 + 131425.0 + 32929.0) / 3 * 1024 + (256.0 + 64.0 + 64.0) / 3 * 1024)
+DOMINANT_KERNEL_TRAFFIC_BYTES = int((131431.0 + 131431.0 + 32935.0) / 3 * 1024 + (256.0 + 64.0 + 64.0) / 3 * 1024)
 
 
 def gemv_bytes(n, k, bias=True):
