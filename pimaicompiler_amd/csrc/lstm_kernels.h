@@ -11,10 +11,10 @@
 //   lstm_step_f16_kernel      one launch per (layer, direction, step): streams W_hh (and W_ih when the
 //                             input projection is fused) once, HBM-bound.  Used for seq_len == 1 decode
 //                             steps and as the fallback for shapes the persistent kernel does not take.
-//   lstm_seq_f16_kernel       one launch per (layer, direction) for the whole sequence: every block keeps
-//                             its 16 rows of W_hh in LDS and its cell state in registers for all steps; h_t
-//                             is exchanged between blocks through tagged words in device memory, so
-//                             the per-step cost is one device-scope store/load round trip, not a launch.
+//   lstm_seq_f16_kernel       one launch for whole sequences of up to four recurrences: every wavefront keeps
+//                             the gate rows of its hidden unit and its cell state in registers for all
+//                             steps; h_t is exchanged between blocks through flagged words in device memory,
+//                             so the per-step cost is one device-scope store/load round trip, not a launch.
 #pragma once
 
 #include "device_common.h"
