@@ -161,7 +161,8 @@ int pimhip_lstm_plan_status(PimHipLstmPlan* plan);
 int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limit);
 
 /* Selects how pimhip_lstm_forward runs the recurrence: 0 = automatic, 1 = one fused launch per step,
- * 2 = persistent sequence kernel (fails with PIMHIP_ERR_UNSUPPORTED if the shape does not fit). */
+ * 2 = persistent sequence kernel (fails with PIMHIP_ERR_UNSUPPORTED if the shape does not fit), 3 = as 2 but with
+ * four hidden units per block in every launch (2 runs a single unidirectional layer with eight). */
 int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);
 
 /* The dense input projection of one LSTM layer over all time steps, the only MFMA kernel of the path:

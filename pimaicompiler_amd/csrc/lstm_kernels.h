@@ -126,7 +126,9 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 //   WAVEFRONT = false  the chains are independent (the two directions of a bidirectional layer): every chain
 //                      takes its own precomputed input projection; chain k runs forward or backward in time.
 //
-// Grid: NB = ceil(H / 4) blocks of 256 lanes (H <= 1024, H % 8 == 0), all resident at once.  Block b owns
+// Grid: NB = ceil(H / UNITS) blocks of UNITS wavefronts (H <= 1024, H % 8 == 0; UNITS = 4, or 8 for a single chain,
+// whose entry then still is one 16-byte store and load and whose exchange among half as many blocks is about 0.4 us
+// shorter), all resident at once.  The text below is written for UNITS = 4.  Block b owns
 // hidden units 4b .. 4b+3 of every chain, one unit per wavefront: wavefront w keeps, per chain, the four W_hh
 // gate rows of unit 4b+w (and the four W_ih rows for wavefront chains k > 0) in registers for the whole
 // launch (lane l holds columns 16l .. 16l+15 of each row) and the cell states in registers.
@@ -234,12 +236,15 @@ __device__ __forceinline__ void store16_device_scope(void* p, unsigned long long
     asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
 }
 
-template <int NC, bool WAVEFRONT>
-__global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
+template <int NC, bool WAVEFRONT, int UNITS = kSeqUnits>
+__global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
 {
-    static_assert(NC >= 1 && NC <= kSeqMaxChains && 2 * NC <= kSeqEntryWords, "an entry holds one 8-byte word per chain");
-    __shared__ __align__(16) half_t hbuf[2][NC][kSeqMaxH];  // published h per chain, double buffered by parity
-    __shared__ __align__(16) unsigned short pub[NC][4];     // this block's next entry: chain k, wavefront w
+    static_assert(UNITS == 4 || UNITS == 8, "one or two 8-byte words per chain and block");
+    constexpr int WPC = UNITS / 4;  // 8-byte words per chain in an entry
+    constexpr int NW = NC * WPC;    // 8-byte words of an entry that are in use
+    static_assert(NC >= 1 && NC <= kSeqMaxChains && 2 * NW <= kSeqEntryWords, "an entry is 64 bytes");
+    __shared__ __align__(16) half_t hbuf[2][NC][kSeqMaxH];   // published h per chain, double buffered by parity
+    __shared__ __align__(16) unsigned short pub[NC][UNITS];  // this block's next entry: chain k, wavefront w
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -247,7 +252,7 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
     const int H = p.H;
     const int T = p.T;
     const int nb = gridDim.x;
-    const int j = blockIdx.x * kSeqUnits + wave;  // this wavefront's hidden unit
+    const int j = blockIdx.x * UNITS + wave;  // this wavefront's hidden unit
     const bool unit_ok = j < H;
     const int n_super = WAVEFRONT ? T + NC - 1 : T;
 
@@ -275,7 +280,7 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
             }
         }
         // Columns at and past H stay zero in all h buffers for the whole kernel.
-        for (int i = tid; i < 2 * NC * kSeqMaxH / 8; i += 256) reinterpret_cast<half8_t*>(&hbuf[0][0][0])[i] = zero;
+        for (int i = tid; i < 2 * NC * kSeqMaxH / 8; i += 64 * UNITS) reinterpret_cast<half8_t*>(&hbuf[0][0][0])[i] = zero;
     }
     __syncthreads();
 
@@ -315,9 +320,9 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
 
         // ---- 1. what block `tid` published at super-step tau - 1 (or the initial state) into LDS ----
         if (has_entry) {
-            unsigned long long words[NC];  // word k: the four fp16 of chain k published by block `tid`
+            unsigned long long words[NW];  // words k * WPC ..: the UNITS fp16 of chain k published by block `tid`
 #pragma unroll
-            for (int k = 0; k < NC; ++k) words[k] = 0ull;
+            for (int k = 0; k < NW; ++k) words[k] = 0ull;
             if (tau > 0) {
                 const unsigned int gp = p.g_base + (unsigned int)tau - 1u;  // the super-step whose values are awaited
                 const unsigned long long want = ((gp >> 1) & 1u) ? 0x4000400040004000ull : 0ull;
@@ -327,12 +332,12 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
                 while (true) {
                     bool ok = true;
 #pragma unroll
-                    for (int k = 0; k + 1 < NC; k += 2) load16_device_scope(src + k, words[k], words[k + 1]);
-                    if (NC & 1)
-                        words[NC - 1] = __hip_atomic_load(const_cast<unsigned long long*>(src) + (NC - 1), __ATOMIC_RELAXED,
+                    for (int k = 0; k + 1 < NW; k += 2) load16_device_scope(src + k, words[k], words[k + 1]);
+                    if (NW & 1)
+                        words[NW - 1] = __hip_atomic_load(const_cast<unsigned long long*>(src) + (NW - 1), __ATOMIC_RELAXED,
                                                           __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-                    for (int k = 0; k < NC; ++k) ok = ok && (words[k] & 0x4000400040004000ull) == want;
+                    for (int k = 0; k < NW; ++k) ok = ok && (words[k] & 0x4000400040004000ull) == want;
                     if (ok || gave_up) break;
                     ++spins;
                     if ((spins & 255u) == 0u) {
@@ -347,17 +352,24 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
 #pragma unroll
             for (int k = 0; k < NC; ++k) {
                 const int s_k = WAVEFRONT ? tau - k : tau;  // the time step chain k computes now
-                half4_t hv;
-                if (s_k == 0) {
-                    // First step of this chain: its previous h is the caller's initial state.
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) hv[e] = (tid * 4 + e < H) ? p.chain[k].h0[tid * 4 + e] : (half_t)0.0f;
-                } else {
-                    // Unit e of chain k in block `tid`, flag bit removed.
+                for (int q = 0; q < WPC; ++q) {
+                    half4_t hv;
+                    if (s_k == 0) {
+                        // First step of this chain: its previous h is the caller's initial state.
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) hv[e] = __builtin_bit_cast(half_t, (unsigned short)((words[k] >> (16 * e)) & 0xbfffu));
+                        for (int e = 0; e < 4; ++e) {
+                            const int u = tid * UNITS + q * 4 + e;
+                            hv[e] = (u < H) ? p.chain[k].h0[u] : (half_t)0.0f;
+                        }
+                    } else {
+                        // Units 4q .. 4q+3 of chain k in block `tid`, flag bit removed.
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            hv[e] = __builtin_bit_cast(half_t, (unsigned short)((words[k * WPC + q] >> (16 * e)) & 0xbfffu));
+                    }
+                    *reinterpret_cast<half4_t*>(&hb[k][tid * UNITS + q * 4]) = hv;
                 }
-                *reinterpret_cast<half4_t*>(&hb[k][tid * 4]) = hv;
             }
         }
         __syncthreads();
@@ -456,8 +468,8 @@ __global__ __launch_bounds__(256) void lstm_seq_f16_kernel(LstmSeqArgs p)
             unsigned long long* dst = reinterpret_cast<unsigned long long*>(p.hx + ((long)(g & 1u) * nb + blockIdx.x) * kSeqEntryWords);
             const unsigned long long* src = reinterpret_cast<const unsigned long long*>(&pub[0][0]);
 #pragma unroll
-            for (int k = 0; k + 1 < NC; k += 2) store16_device_scope(dst + k, src[k], src[k + 1]);
-            if (NC & 1) __hip_atomic_store(dst + (NC - 1), src[NC - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int k = 0; k + 1 < NW; k += 2) store16_device_scope(dst + k, src[k], src[k + 1]);
+            if (NW & 1) __hip_atomic_store(dst + (NW - 1), src[NW - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
 

@@ -456,6 +456,8 @@ struct PimHipLstmPlan {
     unsigned int* abort_flag = nullptr;
     unsigned int* abort_host = nullptr;  // pinned copy read by pimhip_lstm_plan_status
     int seq_blocks = 0;
+    bool reset_exchange = false;     // the next forward starts from a cleared exchange buffer (layout change)
+    bool seq_units8_ok = false;      // a single chain may run with 8 hidden units per block (half as many blocks)
 };
 
 namespace
@@ -595,6 +597,11 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         plan->seq_kernel_ok = (int64_t)per_cu * plan->num_cus >= plan->seq_blocks;
     }
     if (plan->seq_kernel_ok) {
+        int per_cu8 = 0;
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu8, lstm_seq_f16_kernel<1, true, 8>, 512, 0));
+        plan->seq_units8_ok = (int64_t)per_cu8 * plan->num_cus >= (plan->seq_blocks + 1) / 2;
+    }
+    if (plan->seq_kernel_ok) {
         // One region per number of chains a launch can advance: a launch writes exactly the words of its chains,
         // and the flag bits of a region must see every super-step that uses it.
         plan->hx_region_words = (size_t)2 * plan->seq_blocks * kSeqEntryWords;
@@ -625,9 +632,11 @@ extern "C" int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan)
 extern "C" int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode)
 {
     if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
-    if (mode < 0 || mode > 2) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "mode %d not in {0, 1, 2}", mode);
-    if (mode == 2 && !plan->seq_kernel_ok)
+    if (mode < 0 || mode > 3) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "mode %d not in {0, 1, 2, 3}", mode);
+    if (mode >= 2 && !plan->seq_kernel_ok)
         return fail(PIMHIP_ERR_UNSUPPORTED, "hidden_size %lld does not fit the persistent sequence kernel", (long long)plan->hidden);
+    // Modes 3 and 0 / 2 lay out a single chain's exchange entries differently: start over from a cleared buffer.
+    if ((plan->mode == 3) != (mode == 3)) plan->reset_exchange = true;
     plan->mode = mode;
     return PIMHIP_OK;
 }
@@ -680,9 +689,9 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         return PIMHIP_OK;
     }
 
-    if (*plan->abort_host != 0u) {
-        // The previous forward of this plan timed out: re-arm the flag and bring the exchange buffer back to its
-        // initial state (fill kernels, not memset nodes, so that callers may capture this call).
+    if (*plan->abort_host != 0u || plan->reset_exchange) {
+        // The previous forward of this plan timed out (or the entry layout changes): re-arm the flag and bring the
+        // exchange buffer back to its initial state (fill kernels, not memset nodes, so that callers may capture this call).
         fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 1, 0u);
         if (plan->hx) {
             const size_t words = plan->hx_region_words * kSeqMaxChains;
@@ -690,8 +699,9 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         }
         for (int i = 0; i <= kSeqMaxChains; ++i) plan->g_count[i] = 2;
         *plan->abort_host = 0u;
+        plan->reset_exchange = false;
     }
-    const bool use_seq = (plan->mode == 2 && T + kSeqMaxChains <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T + kSeqMaxChains <= kSeqMaxT);
+    const bool use_seq = (plan->mode >= 2 && T + kSeqMaxChains <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T + kSeqMaxChains <= kSeqMaxT);
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
     // seq_len == 1: fuse the input projection into the step (one launch per layer and direction).
     const bool fuse_xproj = !use_seq && T == 1;
@@ -744,7 +754,14 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                 lstm_seq_f16_kernel<2, false><<<grid, block, 0, s>>>(a);
             } else {
                 switch (nc) {
-                    case 1: lstm_seq_f16_kernel<1, true><<<grid, block, 0, s>>>(a); break;
+                    case 1:
+                        // A single chain exchanges 2 bytes per unit: eight units per block still fit one 16-byte
+                        // store and one 16-byte load per entry, and half as many blocks finish a round sooner.
+                        if (plan->seq_units8_ok && plan->mode != 3)
+                            lstm_seq_f16_kernel<1, true, 8><<<dim3((unsigned)((H + 7) / 8)), dim3(512), 0, s>>>(a);
+                        else
+                            lstm_seq_f16_kernel<1, true><<<grid, block, 0, s>>>(a);
+                        break;
                     case 2: lstm_seq_f16_kernel<2, true><<<grid, block, 0, s>>>(a); break;
                     case 3: lstm_seq_f16_kernel<3, true><<<grid, block, 0, s>>>(a); break;
                     default: lstm_seq_f16_kernel<4, true><<<grid, block, 0, s>>>(a); break;

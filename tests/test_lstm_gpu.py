@@ -13,7 +13,7 @@ from oracle import oracle
 pytestmark = pytest.mark.gpu
 LSTM_TOL = 5e-3
 DEV = "cuda:0"
-MODES = [1, 2]  # 1: one fused launch per step, 2: persistent sequence kernel
+MODES = [1, 2, 3]  # 1: one fused launch per step, 2: persistent sequence kernel, 3: the same, four units per block always
 
 
 def maxabs(a, b):
@@ -62,7 +62,7 @@ CASES = [  # I, H, L, bidirectional, T, biases
 @pytest.mark.parametrize("mode", [0] + MODES)
 @pytest.mark.parametrize("I,H,L,bidir,T,has_b", CASES)
 def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
-    if mode == 2 and H > 1024:
+    if mode >= 2 and H > 1024:
         pytest.skip("the persistent kernel takes hidden sizes up to 1024; larger ones run step by step")
     params, x, h0, c0 = oracle.lstm_inputs(900 + I + H + T, I, H, L, bidir, T, has_b)
     g = torch.Generator().manual_seed(T)
@@ -218,6 +218,24 @@ def test_step_and_sequence_kernels_agree(ops):
     y1, h1, c1 = run_plan(ops, params, x, h0, c0, True, 1, False, 1)
     y2, h2, c2 = run_plan(ops, params, x, h0, c0, True, 1, False, 2)
     assert maxabs(y1, y2.cpu()) <= 1e-3 and maxabs(c1, c2.cpu()) <= 1e-3
+
+
+def test_switching_the_block_shape_on_one_plan_restarts_the_exchange(ops):
+    """Modes 2 and 3 lay out a single layer's exchange entries differently; a plan that switches must not read what
+    the other layout left behind."""
+    params, x, h0, c0 = oracle.lstm_inputs(77, 64, 1024, 1, False, 23)
+    want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 23)
+    outs = []
+    for mode in (2, 3, 3, 2, 0, 3, 1, 2):
+        plan.set_mode(mode)
+        y, hn, cn = plan.forward(x.reshape(23, 64).to(DEV), h0.to(DEV), c0.to(DEV))
+        plan.status()
+        assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
+        outs.append((mode, y.cpu()))
+    first = {}
+    for mode, y in outs:          # one mode, one instruction stream: repeated runs agree to the bit
+        assert torch.equal(first.setdefault(mode, y), y)
 
 
 # ---- the bounded wait ---------------------------------------------------------------------------------------------
