@@ -144,7 +144,7 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 //
 // Exchange buffer: hx[2][NB] entries of 64 bytes (entries of different blocks do not share a 64-byte segment,
 // which measurably shortens the exchange); chain k of block b uses the 8-byte word k of the entry, one fp16 per
-// wavefront.  |h| <= 1, so bit 14 of its fp16 pattern is always 0 and carries the flag: with g = g_base + tau
+// wavefront.  |h| <= 1, so bit 14 of its fp16 pattern is always 0 (a NaN is published as 0) and carries the flag: with g = g_base + tau
 // counting super-steps over all launches of a plan, super-step g publishes into parity g & 1 with flag bit
 // (g >> 1) & 1, i.e. the bit flips every time a slot is rewritten.  A slot can only hold what was published two
 // super-steps earlier or the current values (publishing g + 2 needs the words of g + 1 from all blocks, which
@@ -445,7 +445,10 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             const unsigned int flag = (((p.g_base + (unsigned int)tau) >> 1) & 1u) << 14;
 #pragma unroll
             for (int k = 0; k < NC; ++k) {
-                const unsigned int hbits = unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new[k]) : 0u;
+                unsigned int hbits = unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new[k]) : 0u;
+                // A NaN (from non-finite inputs or weights) has bit 14 set and cannot travel with the flag: y, hn and
+                // cn below still receive it, the recurrence continues from 0 for this unit instead of waiting forever.
+                if ((hbits & 0x7c00u) == 0x7c00u) hbits = 0u;
                 pub[k][wave] = (unsigned short)(hbits | flag);
             }
             if (unit_ok) {

@@ -256,6 +256,22 @@ def test_persistent_kernel_wait_gives_up_and_reports(ops):
     assert maxabs(y, want[0]) <= 2e-3
 
 
+@pytest.mark.parametrize("mode", [2, 3])
+def test_persistent_kernel_survives_a_nan_input(ops, mode):
+    """A NaN cannot carry the exchange's flag bit, so it is exchanged as 0; the cell state keeps it, and y is NaN from
+    that step on exactly as in LibTorch.  No wait times out."""
+    params, x, h0, c0 = oracle.lstm_inputs(5, 64, 512, 1, False, 12)
+    x = x.clone()
+    x[7, 0, 3] = float("nan")
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 12)
+    plan.set_mode(mode)
+    y, hn, cn = plan.forward(x.reshape(12, 64).to(DEV), h0.to(DEV), c0.to(DEV))
+    plan.status()
+    want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)[0]
+    assert maxabs(y[:7], want[:7]) <= 2e-3
+    assert bool(torch.isnan(want[7:]).all()) and bool(torch.isnan(y[7:]).all()) and bool(torch.isnan(cn).all())
+
+
 # ---- input projection (the MFMA kernel) against fp32 torch on the host ---------------------------------------------
 @pytest.mark.parametrize("T,K,N", [(1, 8, 16), (5, 24, 40), (16, 32, 16), (17, 40, 100), (50, 1024, 4096), (50, 2048, 4096),
                                    (200, 240, 4096), (200, 1024, 4096), (341, 240, 4096), (700, 64, 256)])
