@@ -229,6 +229,22 @@ def main():
         P.execute_gemv_group([s_["x"] for s_ in shapes], ws, [s_["b"] for s_ in shapes])
     us = timed_us(grouped, 100)
     other["gemv_sweep_grouped_launch"] = {"us": round(us, 2), "gbs": round(step_bytes / us / 1e3, 1)}
+    # the sweep in the other operand order (y = x . A, A [in, out] row-major: the un-swapped addmm / matmul route); the
+    # same cold pools, read as [in, out]
+    vm_times = []
+    for s_ in shapes:
+        xv = (2 * torch.rand(s_["k"], generator=g, device=dev) - 1).half()
+
+        def vm_launch(s_=s_, xv=xv):
+            w = s_["pool"][s_["it"] % s_["copies"]]
+            s_["it"] += 1
+            rc = lib.pimhip_execute_gemv(s_["y"].data_ptr(), xv.data_ptr(), w.data_ptr(), s_["b"].data_ptr(), s_["k"], s_["n"], 0,
+                                         L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W, sh)
+            if rc != 0:
+                raise RuntimeError(lib.pimhip_last_error().decode())
+        us = timed_us(vm_launch, 50)
+        vm_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
+    other["gemv_vm_order"] = vm_times
     # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
     big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
     big_c = torch.empty_like(big_a)

@@ -176,13 +176,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_generic_kernel(const h
 // ---------------------------------------------------------------------------------------------
 // VM order, vector path.  Requirements: N % 8 == 0, lda % 8 == 0, A 16-byte aligned.
 //
-// A block owns 512 adjacent outputs (8 per lane, one 16-byte load per weight row) and a slice
-// [k_begin, k_end) of the reduction; its WAVES wavefronts interleave over the rows of the slice.
-// gridDim.y slices cover K.  With one slice the block finishes the outputs itself; with several,
-// each block writes its 512 partial sums (fp32) to `partial[slice][N]` and takes a ticket from
-// `tickets[blockIdx.x]`; the block that draws the last ticket adds the slices in slice order (so
-// the result does not depend on which block finishes last), applies the epilogue and re-arms the
-// ticket counter for the next launch.
+// A block owns CW = 8 * LPR adjacent outputs and a slice [k_begin, k_end) of the reduction.  LPR lanes (8 columns,
+// one 16-byte load each) cover the block's part of one weight row, so a wavefront reads 64 / LPR rows per load
+// instruction and the block's wavefronts interleave over the rows of the slice, U loads in flight per lane.
+// gridDim.y slices cover K.  With one slice the block finishes the outputs itself; with several, each block writes
+// its CW partial sums (fp32) to `partial[slice][N]` and takes a ticket from `tickets[blockIdx.x]`; the block that
+// draws the last ticket adds the slices with all its lanes, in an order that depends on the slice index only (so the
+// result does not depend on which block finishes last), applies the epilogue and re-arms the ticket counter for
+// the next launch.
 // ---------------------------------------------------------------------------------------------
 // Destinations of a VM product: the same result is stored to `count` buffers (the GNMT attention context goes
 // straight into three concatenation buffers, runtime/source/executor/op_executor/aten_ops_executor.cpp:694-737).
@@ -192,21 +193,49 @@ struct GemvOuts {
     int count;
 };
 
-template <int WAVES, int U>
+// 32 contiguous bytes written / read at device scope (partial sums cross CUs and XCDs).  The loads of one call are
+// issued together and waited for once.
+__device__ __forceinline__ void store32_device_scope(float* p, const float (&v)[8])
+{
+    const float4_t lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\tglobal_store_dwordx4 %0, %2, off offset:16 sc1" : : "v"(p), "v"(lo), "v"(hi) : "memory");
+}
+template <int B>
+__device__ __forceinline__ void load32_device_scope(const float* const (&p)[B], float4_t (&lo)[B], float4_t (&hi)[B])
+{
+    static_assert(B == 4, "four slices per batch");
+    asm volatile(
+        "global_load_dwordx4 %0, %8, off sc1\n\tglobal_load_dwordx4 %1, %8, off offset:16 sc1\n\t"
+        "global_load_dwordx4 %2, %9, off sc1\n\tglobal_load_dwordx4 %3, %9, off offset:16 sc1\n\t"
+        "global_load_dwordx4 %4, %10, off sc1\n\tglobal_load_dwordx4 %5, %10, off offset:16 sc1\n\t"
+        "global_load_dwordx4 %6, %11, off sc1\n\tglobal_load_dwordx4 %7, %11, off offset:16 sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(lo[0]), "=&v"(hi[0]), "=&v"(lo[1]), "=&v"(hi[1]), "=&v"(lo[2]), "=&v"(hi[2]), "=&v"(lo[3]), "=&v"(hi[3])
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3])
+        : "memory");
+}
+
+template <int WAVES, int U, int LPR>
 __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* __restrict__ x,
                                                                  const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ bias,
                                                                  GemvOuts outs, int K, int N, long lda,
-                                                                 int relu, int k_per_slice,
-                                                                 float* __restrict__ partial,
-                                                                 unsigned int* __restrict__ tickets)
+                                                                 int relu, int k_per_slice, float* partial,
+                                                                 unsigned int* tickets)
 {
-    __shared__ float red[WAVES][8][64];
+    static_assert(LPR == 16 || LPR == 32 || LPR == 64, "lanes per weight row");
+    constexpr int RPW = 64 / LPR;          // rows per wavefront and load instruction
+    constexpr int GROUPS = WAVES * RPW;    // row groups per block = LDS rows of the reduction
+    constexpr int STEP = GROUPS;           // rows between consecutive loads of one lane
+    __shared__ float red[GROUPS][8][LPR];
     __shared__ unsigned int s_ticket;
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const long col0 = ((long)blockIdx.x * 64 + lane) * 8;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int cg = lane % LPR;             // which 8 columns of the block
+    const int grp = wave * RPW + lane / LPR;
+    const long col0 = ((long)blockIdx.x * LPR + cg) * 8;
     const bool col_ok = col0 < N;
     const int k_begin = blockIdx.y * k_per_slice;
     const int k_end = min(K, k_begin + k_per_slice);
@@ -217,22 +246,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
 
     if (col_ok) {
         const half_t* a = A + col0;
-        int k = k_begin + wave;
-        for (; k + (U - 1) * WAVES < k_end; k += U * WAVES) {
+        int k = k_begin + grp;
+        for (; k + (U - 1) * STEP < k_end; k += U * STEP) {
             half8_t ar[U];
             float xr[U];
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                ar[u] = load_stream(reinterpret_cast<const half8_t*>(a + (long)(k + u * WAVES) * lda));
+                ar[u] = load_stream(reinterpret_cast<const half8_t*>(a + (long)(k + u * STEP) * lda));
 #pragma unroll
-            for (int u = 0; u < U; ++u) xr[u] = (float)x[k + u * WAVES];
+            for (int u = 0; u < U; ++u) xr[u] = (float)x[k + u * STEP];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) acc[j] = fmaf((float)ar[u][j], xr[u], acc[j]);
             }
         }
-        for (; k < k_end; k += WAVES) {
+        for (; k < k_end; k += STEP) {
             const half8_t ar = load_stream(reinterpret_cast<const half8_t*>(a + (long)k * lda));
             const float xr = (float)x[k];
 #pragma unroll
@@ -240,64 +269,93 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
         }
     }
 
-    // Combine the WAVES partial sums of each column in LDS; wave 0 ends up with the block's result.
+    // Combine the GROUPS partial sums of each column in LDS, in group order; lanes tid < LPR end up with the block's result.
 #pragma unroll
-    for (int j = 0; j < 8; ++j) red[wave][j][lane] = acc[j];
+    for (int j = 0; j < 8; ++j) red[grp][j][cg] = acc[j];
     __syncthreads();
-    if (wave == 0) {
+    const bool finisher = tid < LPR && col_ok;  // tid < LPR: cg == tid, grp == 0
+    if (tid < LPR) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            float v = red[0][j][lane];
+            float v = red[0][j][cg];
 #pragma unroll
-            for (int w = 1; w < WAVES; ++w) v += red[w][j][lane];
+            for (int g = 1; g < GROUPS; ++g) v += red[g][j][cg];
             acc[j] = v;
         }
     }
 
-    const int nslices = gridDim.y;
-    if (nslices == 1) {
-        if (wave == 0 && col_ok) {
-            half8_t out;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                float v = acc[j];
-                if (bias) v += (float)bias[col0 + j];
-                if (relu) v = fmaxf(v, 0.0f);
-                out[j] = (half_t)v;
-            }
-            for (int o = 0; o < outs.count; ++o) *reinterpret_cast<half8_t*>(outs.y[o] + col0) = out;
-        }
-        return;
-    }
-
-    if (wave == 0 && col_ok) {
-        float* p = partial + (long)blockIdx.y * N + col0;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) __hip_atomic_store(p + j, acc[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        s_ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (s_ticket != (unsigned int)(nslices - 1)) return;
-
-    __threadfence();
-    if (wave == 0 && col_ok) {
+    auto epilogue_store = [&](const float (&v)[8]) {
         half8_t out;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            float v = 0.0f;
-            for (int s = 0; s < nslices; ++s)
-                v += __hip_atomic_load(partial + (long)s * N + col0 + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (bias) v += (float)bias[col0 + j];
-            if (relu) v = fmaxf(v, 0.0f);
-            out[j] = (half_t)v;
+            float r = v[j];
+            if (bias) r += (float)bias[col0 + j];
+            if (relu) r = fmaxf(r, 0.0f);
+            out[j] = (half_t)r;
         }
         for (int o = 0; o < outs.count; ++o) *reinterpret_cast<half8_t*>(outs.y[o] + col0) = out;
+    };
+
+    const int nslices = gridDim.y;
+    if (nslices == 1) {
+        if (finisher) epilogue_store(acc);
+        return;
     }
-    if (threadIdx.x == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // The partial sums travel with device-scope stores and loads (write-through / read-through the XCD's L2), so no
+    // fence is needed, and none is wanted: a device-scope fence writes back and invalidates the whole L2, once per
+    // block.  The stores are complete (acknowledged) before the block's ticket is drawn; the last block's loads are
+    // issued after it has seen the last ticket.
+    if (finisher) {
+        store32_device_scope(partial + (long)blockIdx.y * N + col0, acc);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != (unsigned int)(nslices - 1)) return;
+
+    // Row group g of the block adds slices g, g + GROUPS, ... (four loads of 32 bytes in flight), then the groups are
+    // added in group order as above.
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    if (col_ok) {
+        const float* base = partial + col0;
+        int sl = grp;
+        for (; sl + 3 * GROUPS < nslices; sl += 4 * GROUPS) {
+            const float* const ptr[4] = {base + (long)sl * N, base + (long)(sl + GROUPS) * N, base + (long)(sl + 2 * GROUPS) * N,
+                                         base + (long)(sl + 3 * GROUPS) * N};
+            float4_t lo[4], hi[4];
+            load32_device_scope<4>(ptr, lo, hi);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[j] += lo[b][j];
+                    acc[4 + j] += hi[b][j];
+                }
+            }
+        }
+        for (; sl < nslices; sl += GROUPS) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                acc[j] += __hip_atomic_load(base + (long)sl * N + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) red[grp][j][cg] = acc[j];
+    __syncthreads();
+    if (finisher) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            v[j] = red[0][j][cg];
+#pragma unroll
+            for (int g = 1; g < GROUPS; ++g) v[j] += red[g][j][cg];
+        }
+        epilogue_store(v);
+    }
+    if (tid == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // VM order, any N / leading dimension / alignment: one lane per output column, 2-byte loads.

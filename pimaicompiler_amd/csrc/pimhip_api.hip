@@ -47,7 +47,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 struct SplitWorkspace {
     float* partial = nullptr;        // [slices][N] fp32 partial sums of the VM kernel
     size_t partial_elems = 0;
-    unsigned int* tickets = nullptr; // one arrival counter per 512-column block, zero between launches
+    unsigned int* tickets = nullptr; // one arrival counter per column block, zero between launches
     size_t ticket_count = 0;
 };
 
@@ -144,18 +144,25 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
         gemv_vm_f16_generic_kernel<<<grid, 256, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu);
         return PIMHIP_OK;
     }
-    constexpr int WAVES = 4;
-    const int col_blocks = (int)((N + 511) / 512);
-    // Enough slices of K that about 4 blocks per CU exist, each slice at least 32 rows deep.
-    int slices = (4 * st->num_cus + col_blocks - 1) / col_blocks;
+    // Measured on MI355X: 128-column blocks (16 lanes per weight row, 4 rows per wavefront and load) with 8 loads in
+    // flight per lane are fastest for every shape tried; a cross-block reduction costs about 3 us, so K is sliced
+    // only as far as needed for roughly one block per CU (64 blocks for a weight of a few MB), and not at all for
+    // weights of up to 256 KB.
+    constexpr int WAVES = 4, U = 8, LPR = 16;
+    constexpr int GROUPS = WAVES * (64 / LPR);
+    const int col_blocks = (int)((N + LPR * 8 - 1) / (LPR * 8));
+    const int64_t weight_bytes = K * N * (int64_t)sizeof(half_t);
+    int64_t target = weight_bytes / 65536;
+    if (target < 64) target = 64;
+    if (target > st->num_cus) target = st->num_cus;
+    int slices = (int)((target + col_blocks - 1) / col_blocks);
     const int max_slices = (int)((K + 31) / 32);
     if (slices > max_slices) slices = max_slices;
-    // A weight of a few hundred KB is latency-bound: the cross-block reduction would cost more than it spreads.
-    if ((int64_t)K * N * (int64_t)sizeof(half_t) <= 256 * 1024) slices = 1;
+    if (weight_bytes <= 256 * 1024) slices = 1;
     if (slices < 1) slices = 1;
     int k_per_slice = (int)((K + slices - 1) / slices);
-    k_per_slice = (k_per_slice + WAVES - 1) / WAVES * WAVES;
-    if (k_per_slice < WAVES) k_per_slice = WAVES;  // K == 0: one empty slice, y = act(bias)
+    k_per_slice = (k_per_slice + GROUPS - 1) / GROUPS * GROUPS;
+    if (k_per_slice < GROUPS) k_per_slice = GROUPS;  // K == 0: one empty slice, y = act(bias)
     slices = (int)((K + k_per_slice - 1) / k_per_slice);
     if (slices < 1) slices = 1;
     SplitWorkspace* ws = nullptr;
@@ -168,8 +175,8 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
         tickets = ws->tickets;
     }
     dim3 grid(col_blocks, slices);
-    gemv_vm_f16_kernel<WAVES, 4><<<grid, WAVES * 64, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu,
-                                                             k_per_slice, partial, tickets);
+    gemv_vm_f16_kernel<WAVES, U, LPR><<<grid, WAVES * 64, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu,
+                                                                    k_per_slice, partial, tickets);
     return PIMHIP_OK;
 }
 
