@@ -155,7 +155,7 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     int64_t target = weight_bytes / 65536;
     if (target < 64) target = 64;
     if (target > st->num_cus) target = st->num_cus;
-    int slices = (int)((target + col_blocks - 1) / col_blocks);
+    int slices = (int)((target + col_blocks / 2) / col_blocks);  // rounded: 250 column blocks on 256 CUs are not sliced
     const int max_slices = (int)((K + 31) / 32);
     if (slices > max_slices) slices = max_slices;
     if (weight_bytes <= 256 * 1024) slices = 1;
