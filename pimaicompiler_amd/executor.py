@@ -7,8 +7,9 @@ Mirrors, for the layer types on this path only, what the reference's interpreter
     execute_aten_addmm[_with_stream]         runtime/source/executor/op_executor/aten_ops_executor.cpp:181-254
     execute_aten_matmul[_with_stream]        aten_ops_executor.cpp:2488-2525
     execute_aten_linear                      aten_ops_executor.cpp:2029-2059
-    execute_aten_lstm1 / execute_aten_lstm2  aten_ops_executor.cpp:2135-2399 (without the GNMT concatenation-buffer
-                                             side effects, :2238-2302, which belong to the model-specific glue)
+    execute_aten_lstm1 / execute_aten_lstm2  aten_ops_executor.cpp:2135-2399; the GNMT decoder's state and attention
+                                             buffers (:2238-2302) are written in place, as the reference's MIOpen
+                                             route does (miopen_ops_executor.cpp:170-228)
     execute_aten_add / execute_aten_bmm      aten_ops_executor.cpp:43-179, 668-747 (custom-kernel branches)
     execute_multi_stream                     runtime/source/executor/op_executor/stream_ops_executor.cpp:27-50
     StreamExecutor.inference                 the dispatch loop, stream_executor.cpp:153-186, for these layer types
@@ -100,6 +101,14 @@ class AtenLSTM1Layer(NNLayer):          # ir/include/layers/aten_lstm1_layer.h
     weight_ids: List[int] = field(default_factory=list)
     bias_ids: List[int] = field(default_factory=list)
     param_vector: List[torch.Tensor] = field(default_factory=list)   # LibTorch order, built at model-build time
+    # GNMT decoder (aten_lstm1_layer.h: match_custom_opt_, custom_opt_number_, custom_cat_mem_id_): layer number k of the
+    # decoder keeps (h, c) in rows 2k, 2k+1 of the state buffer blob `custom_cat_mem_id`; layers 0 and 1 also put their
+    # output into the first H columns of the attention concatenation buffer, whose blob id the reference looks up
+    # through the following cat layer (aten_ops_executor.cpp:2277-2282) and this record carries directly.
+    match_custom_opt: bool = False
+    custom_opt_number: int = 0
+    custom_cat_mem_id: int = -1
+    output_cat_mem_id: int = -1
 
 
 @dataclass
@@ -386,6 +395,39 @@ def _unique_in_order(ids):
     return out
 
 
+def _gnmt_lstm_destinations(layer, executor, x, out_ids, hidden, num_layers, bidirectional, batch_first):
+    """Where a GNMT decoder LSTM writes (y, hy, cy), or None for fresh tensors.
+
+    The reference's LibTorch route rebuilds the concatenation tensors with slice + cat after the call
+    (aten_ops_executor.cpp:2238-2302); its MIOpen route hands the kernel pointers into them
+    (miopen_ops_executor.cpp:170-228).  The latter is what happens here: the step kernel stores straight into the
+    consumers' buffers and no copy is made."""
+    if executor.model_type != "GNMT" or num_layers != 1 or bidirectional:
+        return None
+    seq_len = x.size(1) if batch_first else x.size(0)
+    prev = [executor.find_blob(i)[1] for i in out_ids]
+    if seq_len == 1 and all(isinstance(t, torch.Tensor) and t.is_contiguous() and t.dtype == torch.float16 for t in prev) and \
+            [t.numel() for t in prev] == [hidden, hidden, hidden]:
+        return tuple(prev)                       # the buffers of the previous decoder step are written again
+    if not layer.match_custom_opt:
+        return None
+    k = layer.custom_opt_number
+    state = executor.find_blob(layer.custom_cat_mem_id)[1]
+    if not isinstance(state, torch.Tensor) or not state.is_contiguous() or state.numel() < (2 * k + 2) * hidden:
+        raise NNRuntimeException(f"blob {layer.custom_cat_mem_id} cannot hold the state of decoder layer {k}")
+    flat = state.view(-1)
+    hy = flat[2 * k * hidden:(2 * k + 1) * hidden].view(1, 1, hidden)
+    cy = flat[(2 * k + 1) * hidden:(2 * k + 2) * hidden].view(1, 1, hidden)
+    y = None
+    if k in (0, 1) and layer.output_cat_mem_id >= 0 and seq_len == 1:
+        cat = executor.find_blob(layer.output_cat_mem_id)[1]
+        if isinstance(cat, torch.Tensor) and cat.is_contiguous() and cat.numel() >= hidden:
+            y = cat.view(-1)[:hidden].view(1, 1, hidden)
+    if y is None:
+        y = torch.empty((seq_len, hidden), dtype=torch.float16, device=x.device)
+    return y, hy, cy
+
+
 def execute_aten_lstm1(layer, executor):
     ids = layer.in_stensor_ids
     x = _tensor(executor, ids[0], "lstm input")
@@ -396,8 +438,9 @@ def execute_aten_lstm1(layer, executor):
     out_ids = _unique_in_order(layer.out_stensor_ids)
     if len(out_ids) != 3:
         raise NNRuntimeException("lstm needs three output ids")
+    out = _gnmt_lstm_destinations(layer, executor, x, out_ids, hx[0].size(-1), num_layers, bool(bidirectional), bool(batch_first))
     y, hy, cy = ops.aten_lstm1(x, tuple(hx), layer.param_vector, bool(has_biases), num_layers, dropout, bool(train),
-                               bool(bidirectional), bool(batch_first))
+                               bool(bidirectional), bool(batch_first), out=out)
     for i, v in zip(out_ids, (y, hy, cy)):
         executor.update_blob(i, DataType.TENSOR, v)
 

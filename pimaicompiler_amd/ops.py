@@ -15,6 +15,7 @@ LSTM runs in libpimhip.so.  True matrix-matrix products take the same LibTorch p
 (atenAddmm / atenMatmul, aten_ops.cpp:47-51,362).  Errors are raised as NNRuntimeException
 (runtime/include/executor/utils/utils.h:166-176) instead of being ignored.
 """
+import contextlib
 import ctypes
 import enum
 import weakref
@@ -490,9 +491,25 @@ class LstmPlan:
             y = torch.empty((T, self.num_dirs * self.hidden), dtype=torch.float16, device=self.device)
             hn = torch.empty((self.num_layers * self.num_dirs, self.hidden), dtype=torch.float16, device=self.device)
             cn = torch.empty_like(hn)
-        _check(lib.pimhip_lstm_forward(self._handle, x2d.data_ptr(), h0.data_ptr(), c0.data_ptr(), y.data_ptr(),
-                                       hn.data_ptr(), cn.data_ptr(), T, _stream_handle(stream)))
+        # The kernels read all of h0 while they store hn (and x while they store y): an output that shares memory with
+        # an input, as a decoder's state buffer does when it is both, is computed beside it and copied over afterwards.
+        dests = [y, hn, cn]
+        staged = [t if not any(_overlap(t, i) for i in (x2d, h0, c0)) else torch.empty_like(t) for t in dests]
+        _check(lib.pimhip_lstm_forward(self._handle, x2d.data_ptr(), h0.data_ptr(), c0.data_ptr(), staged[0].data_ptr(),
+                                       staged[1].data_ptr(), staged[2].data_ptr(), T, _stream_handle(stream)))
+        for d, t in zip(dests, staged):
+            if d is not t:
+                if isinstance(stream, int):
+                    stream = torch.cuda.ExternalStream(stream)
+                with torch.cuda.stream(stream) if stream is not None else contextlib.nullcontext():
+                    d.copy_(t)
         return y, hn, cn
+
+
+def _overlap(a, b):
+    """True if the two tensors' storage ranges intersect (both are dense here)."""
+    a0, b0 = a.data_ptr(), b.data_ptr()
+    return a.numel() > 0 and b.numel() > 0 and a0 < b0 + b.numel() * b.element_size() and b0 < a0 + a.numel() * a.element_size()
 
 
 _plan_cache = {}

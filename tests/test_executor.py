@@ -381,3 +381,46 @@ def test_built_model_lstm_then_linear_on_the_rnnt_feature(ops):
     want = np.stack([oracle.gemv_mv(W.numpy(), hn[l], b.numpy()) for l in range(2)])
     got = ex.find_blob(5)[1]
     assert list(got.shape) == [2, 1, 64] and maxabs(got, want) <= 5e-3
+
+
+@pytest.mark.gpu
+def test_gnmt_decoder_steps_write_into_the_state_and_attention_buffers(ops):
+    """Four decoder layers, three decode steps.  Layer k reads (h, c) from rows 2k, 2k+1 of the state buffer and writes
+    them back there (aten_ops_executor.cpp:2238-2270; miopen_ops_executor.cpp:196-217); layers 0 and 1 put their output
+    into the first H columns of the attention concatenation buffer (:2272-2287).  Checked against LibTorch CPU run
+    layer by layer with explicit states."""
+    H, steps = 256, 3
+    g = torch.Generator().manual_seed(31)
+    layer_params = [oracle.lstm_inputs(40 + k, H, H, 1, False, 1)[0] for k in range(4)]
+    state = (0.2 * torch.randn(8, 1, H, generator=g)).half()
+    xs = torch.randn(steps, 4, 1, 1, H, generator=g).half()           # an independent input per step and layer
+    ex = E.StreamExecutor([], model_type="GNMT", device=0)
+    state_d, att_d = state.to(DEV), torch.zeros(1, 1, 2 * H, dtype=torch.float16, device=DEV)
+    att_d[..., H:] = 7.0                                                # the other half belongs to another producer
+    ex.update_blob(100, DataType.TENSOR, state_d)
+    ex.update_blob(101, DataType.TENSOR, att_d)
+    layers = []
+    for k in range(4):
+        layers.append(E.AtenLSTM1Layer(LayerType.ATENLSTM1, k, [10 + k, 20 + k], [30 + k, 40 + k, 50 + k], has_biases=1,
+                                       num_layers=1, dropout=0.0, train=0, bidirectional=0, batch_first=0,
+                                       param_vector=[p.to(DEV) for p in layer_params[k]], match_custom_opt=True,
+                                       custom_opt_number=k, custom_cat_mem_id=100, output_cat_mem_id=101 if k < 2 else -1))
+    ref_state = state.clone()
+    for t in range(steps):
+        for k in range(4):
+            flat = ex.find_blob(100)[1].view(-1)
+            h0 = flat[2 * k * H:(2 * k + 1) * H].view(1, 1, H)           # the decoder slices its state out of the buffer
+            c0 = flat[(2 * k + 1) * H:(2 * k + 2) * H].view(1, 1, H)
+            ex.update_blob(10 + k, DataType.TENSOR, xs[t, k].to(DEV))
+            ex.update_blob(20 + k, DataType.LIST, [h0, c0])
+            E.execute_aten_lstm1(layers[k], ex)
+            wy, wh, wc = oracle.torch_lstm(xs[t, k], ref_state[2 * k:2 * k + 1], ref_state[2 * k + 1:2 * k + 2], layer_params[k],
+                                           True, 1, False)
+            ref_state[2 * k], ref_state[2 * k + 1] = wh[0], wc[0]
+            y = ex.find_blob(30 + k)[1]
+            assert maxabs(y, wy) <= TOL_LSTM
+            if k < 2:
+                assert y.data_ptr() == att_d.data_ptr() and maxabs(att_d[..., :H], wy) <= TOL_LSTM
+                assert bool((att_d[..., H:] == 7.0).all())
+            assert ex.find_blob(40 + k)[1].data_ptr() == state_d.data_ptr() + 2 * k * H * 2
+    assert maxabs(state_d, ref_state) <= TOL_LSTM
