@@ -131,6 +131,13 @@ class AtenAddLayer(NNLayer):            # ir/include/layers/aten_add_layer.h
 
 
 @dataclass
+class AtenBmmLayer(NNLayer):            # ir/include/layers/aten_bmm_layer.h
+    # GNMT: the blob ids of the three concatenation buffers whose second half receives the attention context.  The
+    # reference finds them by walking the graph from this layer (aten_ops_executor.cpp:680-705).
+    cat_mem_ids: List[int] = field(default_factory=list)
+
+
+@dataclass
 class MultiStreamLayer(NNLayer):        # ir/include/layers/multi_stream_layer.h
     layers: List[NNLayer] = field(default_factory=list)
 
@@ -478,7 +485,22 @@ def execute_aten_add(layer, executor):
 
 def execute_aten_bmm(layer, executor):
     ids = layer.in_stensor_ids
-    out = ops.aten_bmm(_tensor(executor, ids[0], "bmm self"), _tensor(executor, ids[1], "bmm other"))
+    a, b = _tensor(executor, ids[0], "bmm self"), _tensor(executor, ids[1], "bmm other")
+    outs = None
+    cat_ids = getattr(layer, "cat_mem_ids", [])
+    if executor.model_type == "GNMT" and cat_ids:
+        # y goes to elements [n, 2n) of every concatenation buffer: one launch with several destinations replaces the
+        # reference's kernel plus two device copies (aten_ops_executor.cpp:694-737).
+        n = b.size(-1)
+        outs = []
+        for cid in cat_ids:
+            cat = _tensor(executor, cid, "bmm concatenation buffer")
+            if not cat.is_contiguous() or cat.numel() < 2 * n:
+                raise NNRuntimeException(f"blob {cid} cannot take the attention context at offset {n}")
+            outs.append(cat.view(-1)[n:2 * n])
+    out = ops.aten_bmm(a, b, outs=outs)
+    if outs:
+        out = out.view(1, 1, -1)
     executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, out)
 
 

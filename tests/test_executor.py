@@ -424,3 +424,20 @@ def test_gnmt_decoder_steps_write_into_the_state_and_attention_buffers(ops):
                 assert bool((att_d[..., H:] == 7.0).all())
             assert ex.find_blob(40 + k)[1].data_ptr() == state_d.data_ptr() + 2 * k * H * 2
     assert maxabs(state_d, ref_state) <= TOL_LSTM
+
+
+@pytest.mark.gpu
+def test_gnmt_attention_context_lands_in_three_concatenation_buffers(ops):
+    """aten_ops_executor.cpp:680-737: y[1,1,1024] = p[1,1,50] . enc[1,50,1024] at offset 1024 of three buffers."""
+    g = torch.Generator().manual_seed(8)
+    p_att, enc = torch.rand(1, 1, 50, generator=g).half(), torch.randn(1, 50, 1024, generator=g).half()
+    ex = E.StreamExecutor([], model_type="GNMT", device=0)
+    cats = [torch.full((1, 1, 2048), float(i + 1), dtype=torch.float16, device=DEV) for i in range(3)]
+    _blobs(ex, b0=p_att.to(DEV), b1=enc.to(DEV), b60=cats[0], b61=cats[1], b62=cats[2])
+    E.execute_aten_bmm(E.AtenBmmLayer(LayerType.ATENBMM, 0, [0, 1], [5], cat_mem_ids=[60, 61, 62]), ex)
+    want = oracle.gemv_vm(p_att.numpy().reshape(-1), enc.numpy().reshape(50, 1024), None)
+    out = ex.find_blob(5)[1]
+    assert list(out.shape) == [1, 1, 1024] and out.data_ptr() == cats[0].data_ptr() + 2048
+    for i, c in enumerate(cats):
+        assert maxabs(c[..., 1024:], want) <= 4e-3 and bool((c[..., :1024] == float(i + 1)).all())
+    assert torch.equal(cats[0][..., 1024:], cats[1][..., 1024:]) and torch.equal(cats[0][..., 1024:], cats[2][..., 1024:])
