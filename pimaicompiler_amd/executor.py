@@ -128,6 +128,10 @@ class AtenLSTM2Layer(NNLayer):          # ir/include/layers/aten_lstm2_layer.h
 @dataclass
 class AtenAddLayer(NNLayer):            # ir/include/layers/aten_add_layer.h
     alpha: int = INT64_MIN
+    # GNMT: blob id of the concatenation buffer whose first n elements receive the sum of the outputs of decoder layers
+    # 2 and 1 (the reference derives both the condition and the id from the neighbouring layers,
+    # aten_ops_executor.cpp:129-148); -1: none.
+    cat_mem_id: int = -1
 
 
 @dataclass
@@ -472,12 +476,24 @@ def execute_aten_add(layer, executor):
     a, b = executor.find_blob(ids[0])[1], executor.find_blob(ids[1])[1]
     alpha = layer.alpha
     if is_default_int64(alpha):
-        alpha = int(executor.find_blob(ids[2])[1]) if len(ids) == 3 and executor.check_valid_blob_id(ids[2]) else 1
+        # As written in the reference (aten_ops_executor.cpp:57-70): with three inputs it asks whether blob id 2 (the
+        # input *index*, not in_stensor_id[2]) is valid before reading the third input.
+        alpha = int(executor.find_blob(ids[2])[1]) if len(ids) == 3 and executor.check_valid_blob_id(2) else 1
     if isinstance(a, int) and isinstance(b, int):
         executor.update_blob(layer.out_stensor_ids[0], DataType.INT64, a + b * alpha)
         return
-    if isinstance(b, torch.Tensor):
-        out = ops.aten_add(a, b, alpha=alpha)
+    if not isinstance(a, torch.Tensor):
+        raise NNRuntimeException("Unsupported input type for aten::add")
+    if isinstance(b, torch.Tensor) and a.dtype == torch.float16 and ops.custom_add_applies(a, b):
+        # The custom kernel writes the sum over `self` (C = A, aten_ops_executor.cpp:121-123), or, for the GNMT
+        # residual add, into the head of a concatenation buffer; alpha is ignored by the kernel (custom_ops.h:415-433).
+        dst = a if a.is_contiguous() else a.contiguous()
+        if executor.model_type == "GNMT" and layer.cat_mem_id >= 0:
+            cat = _tensor(executor, layer.cat_mem_id, "add concatenation buffer")
+            if not cat.is_contiguous() or cat.numel() < a.numel():
+                raise NNRuntimeException(f"blob {layer.cat_mem_id} cannot take the sum")
+            dst = cat.view(-1)[:a.numel()].view(a.shape)
+        out = ops.aten_add(a, b, alpha=alpha, out=dst)
     else:
         out = torch.add(a, b, alpha=alpha)
     executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, out)

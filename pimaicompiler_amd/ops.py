@@ -368,6 +368,18 @@ def aten_add(self_tensor, other_tensor, alpha=1, out=None, stream=None):
     return out
 
 
+def custom_add_applies(self_tensor, other_tensor):
+    """True where executeAtenAdd takes its custom kernel and this path can: fp16 GPU tensors that pass
+    customAddDimensionsCheck, equal in size or `other` one row of `self`."""
+    if not (isinstance(other_tensor, torch.Tensor) and self_tensor.dtype == torch.float16 and
+            other_tensor.dtype == torch.float16 and self_tensor.is_cuda and other_tensor.is_cuda and
+            self_tensor.dim() >= 1 and _custom_add_dims_ok(self_tensor, other_tensor)):
+        return False
+    if self_tensor.dim() == other_tensor.dim():
+        return other_tensor.numel() == self_tensor.numel()
+    return other_tensor.numel() == self_tensor.size(-1)
+
+
 def _custom_add_dims_ok(t1, t2):
     """customAddDimensionsCheck (aten_ops_executor.cpp:87-109) on the larger-rank operand first."""
     s1, s2 = (t1.shape, t2.shape) if t1.dim() >= t2.dim() else (t2.shape, t1.shape)

@@ -195,6 +195,16 @@ def test_integer_add_stays_on_the_host(ex):
     assert ex.find_blob(2) == (DataType.INT64, 11)
 
 
+def test_add_reads_alpha_only_if_blob_id_two_exists(ex):
+    """aten_ops_executor.cpp:59-66 asks checkValidBlobID(in_id) with the input index (2), not the third input's id."""
+    _blobs(ex, b10=3, b11=4, b12=5)
+    E.execute_aten_add(E.AtenAddLayer(LayerType.ATENADD, 0, [10, 11, 12], [20]), ex)
+    assert ex.find_blob(20) == (DataType.INT64, 7)           # blob 2 does not exist: alpha = 1
+    _blobs(ex, b2=0)
+    E.execute_aten_add(E.AtenAddLayer(LayerType.ATENADD, 0, [10, 11, 12], [20]), ex)
+    assert ex.find_blob(20) == (DataType.INT64, 23)          # blob 2 exists: alpha = blob 12 = 5
+
+
 def test_builder_assigns_fresh_ids_and_orders_lstm_parameters(rec, monkeypatch):
     """model_builder.cpp:18-224: ids start after the largest output id; weights before biases per layer; the
     parameter vector is (w_ih, w_hh, b_ih, b_hh) per layer and direction."""
@@ -352,9 +362,20 @@ def test_add_and_bmm_layers(ops):
     q, keys = (0.1 * torch.randn(1, 1, 40, generator=g)).half(), torch.randn(1, 40, 1024, generator=g).half()
     ex = E.StreamExecutor([], device=0)
     _blobs(ex, b0=a.to(DEV), b1=b.to(DEV), b2=q.to(DEV), b3=keys.to(DEV), b4=1)
+    a_d = a.to(DEV)
+    _blobs(ex, b0=a_d)
     E.execute_aten_add(E.AtenAddLayer(LayerType.ATENADD, 0, [0, 1, 4], [5]), ex)
     E.execute_aten_bmm(E.NNLayer(LayerType.ATENBMM, 0, [2, 3], [6]), ex)
     assert np.array_equal(ex.find_blob(5)[1].cpu().numpy(), oracle.add(a.numpy(), b.numpy()).reshape(1, 1, 1024))
+    assert ex.find_blob(5)[1].data_ptr() == a_d.data_ptr()      # the custom add writes over `self` (C = A in the reference)
+    # GNMT residual add: the sum goes to the head of a concatenation buffer, `self` stays as it was
+    exg = E.StreamExecutor([], model_type="GNMT", device=0)
+    cat = torch.full((1, 1, 2048), 3.0, dtype=torch.float16, device=DEV)
+    a2 = a.to(DEV)
+    _blobs(exg, b0=a2, b1=b.to(DEV), b70=cat)
+    E.execute_aten_add(E.AtenAddLayer(LayerType.ATENADD, 0, [0, 1], [5], cat_mem_id=70), exg)
+    assert np.array_equal(cat[..., :1024].cpu().numpy(), oracle.add(a.numpy(), b.numpy()).reshape(1, 1, 1024))
+    assert bool((cat[..., 1024:] == 3.0).all()) and torch.equal(a2.cpu(), a) and exg.find_blob(5)[1].data_ptr() == cat.data_ptr()
     want = oracle.gemv_vm(q.numpy().reshape(-1), keys.numpy().reshape(40, 1024), None)
     assert list(ex.find_blob(6)[1].shape) == [1, 1, 1024] and maxabs(ex.find_blob(6)[1], want) <= TOL_GEMV
 
