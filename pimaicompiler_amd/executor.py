@@ -466,7 +466,10 @@ def execute_aten_lstm2(layer, executor):
     has_biases, num_layers, dropout, train, bidirectional, _ = _lstm_flags(layer, executor, 3, False)
     y, hy, cy = ops.aten_lstm2(data, batch_sizes, tuple(hx), layer.param_vector, bool(has_biases), num_layers, dropout,
                                bool(train), bool(bidirectional))
-    for i, v in zip(layer.out_stensor_ids[:3], (y, hy, cy)):
+    out_ids = _unique_in_order(layer.out_stensor_ids)
+    if len(out_ids) != 3:
+        raise NNRuntimeException("lstm needs three output ids")
+    for i, v in zip(out_ids, (y, hy, cy)):
         executor.update_blob(i, DataType.TENSOR, v)
 
 
