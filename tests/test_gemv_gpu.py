@@ -165,6 +165,36 @@ def test_gemv_full_size_properties(ops, n, k):
     assert abs(float(y1.double().sum()) - want) <= GEMV_TOL * n ** 0.5
 
 
+@pytest.mark.parametrize("n,k", [(4096, 4096), (32000, 1024), (1024, 1024), (520, 4104)])
+def test_gemv_vm_order_full_size_properties(ops, n, k):
+    """The VM order splits K over blocks; its cross-block sum has a fixed order, so repeated launches agree to the bit."""
+    from pimaicompiler_amd import _lib as L
+    g = torch.Generator().manual_seed(n * 3 + k)
+    A = (0.02 * torch.randn(k, n, generator=g)).half().to(DEV)
+    b = (0.01 * torch.randn(n, generator=g)).half().to(DEV)
+    x = (2 * torch.rand(k, generator=g) - 1).half().to(DEV)
+    rc, y0 = raw_gemv(ops, A, x, b, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+    assert rc == 0
+    for _ in range(10):
+        rc, y = raw_gemv(ops, A, x, b, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+        assert rc == 0 and torch.equal(y, y0)
+    want = (x.cpu().double() @ A.cpu().double() + b.cpu().double()).numpy()
+    assert maxabs(y0, want) <= GEMV_TOL
+    # zero input: y == bias exactly; one-hot input: y == A[j, :] + b with one rounding, exactly
+    rc, y = raw_gemv(ops, A, torch.zeros_like(x), b, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+    assert torch.equal(y, b)
+    for j in (0, k // 3 + 1, k - 1):
+        e = torch.zeros_like(x)
+        e[j] = 1.0
+        rc, y = raw_gemv(ops, A, e, b, k, n, 0, L.PIMHIP_ACT_RELU, L.PIMHIP_I_X_W)
+        assert torch.equal(y, torch.relu((A[j].float() + b.float()).half()))
+    # several destinations receive the same bits
+    outs = [torch.empty(n, dtype=torch.float16, device=DEV) for _ in range(3)]
+    ops.aten_bmm(x.reshape(1, 1, k), A.reshape(1, k, n), outs=outs)
+    rc, ynb = raw_gemv(ops, A, x, None, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+    assert all(torch.equal(o, ynb) for o in outs)
+
+
 def test_moe_ffn_decode_step_matches_libtorch(ops, golden):
     import importlib.util, os
     spec = importlib.util.spec_from_file_location("make_golden", os.path.join(os.path.dirname(__file__), "golden", "make_golden.py"))
