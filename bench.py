@@ -245,6 +245,18 @@ def main():
         us = timed_us(vm_launch, 50)
         vm_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
     other["gemv_vm_order"] = vm_times
+    # MoE FFN decode step (router 768 -> 8, then one expert 768 -> 3072 ReLU -> 768): three dependent launches on
+    # resident (warm) weights, the expert fixed so that no host round trip for the argmax is inside the figure
+    wr, w1, w2 = (0.02 * torch.randn(8, 768, device=dev)).half(), (0.02 * torch.randn(3072, 768, device=dev)).half(), \
+        (0.02 * torch.randn(768, 3072, device=dev)).half()
+    tok, logits = torch.randn(768, device=dev).half(), torch.empty(8, dtype=torch.float16, device=dev)
+    hid, yo = torch.empty(3072, dtype=torch.float16, device=dev), torch.empty(768, dtype=torch.float16, device=dev)
+
+    def moe_step():
+        lib.pimhip_execute_gemv(logits.data_ptr(), tok.data_ptr(), wr.data_ptr(), None, 768, 8, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+        lib.pimhip_execute_gemv(hid.data_ptr(), tok.data_ptr(), w1.data_ptr(), None, 768, 3072, 0, L.PIMHIP_ACT_RELU, L.PIMHIP_W_X_I, sh)
+        lib.pimhip_execute_gemv(yo.data_ptr(), hid.data_ptr(), w2.data_ptr(), None, 3072, 768, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+    other["moe_ffn_step_three_gemvs_us"] = round(timed_us(moe_step, 200), 3)
     # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
     big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
     big_c = torch.empty_like(big_a)
