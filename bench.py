@@ -46,7 +46,14 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="first run three out-of-place fp32 adds over 256 MiB (read 256 MiB, write 256 MiB each): "
                          "a kernel of known traffic that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--sections", default="sweep,lstm,other",
+                    help="comma list of what to run: sweep (the timed steps, always run), lstm (LSTM and input projection "
+                         "figures), other (the other kernels of the path); counter runs use --sections sweep")
     args = ap.parse_args()
+    sections = set(args.sections.split(","))
+
+    def progress(msg):
+        print(f"[bench] {msg}", file=sys.stderr, flush=True)
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)", file=sys.stderr)
         return 2
@@ -151,11 +158,12 @@ def main():
                     frac=round(achieved / HBM_PEAK_GBS, 4), traffic=DOMINANT_KERNEL_TRAFFIC_BYTES,
                     kernel="gemv_mv_f16_kernel<2,4,4,4>", bytes_per_launch=int(dom_bytes), us_per_launch=round(dom_us, 3))
 
+    progress("sweep timed")
     # ---- LSTM: RNNT-style 2 layers, I=240, H=1024, T=200 (400 layer-steps per call) ------------------------------
     from oracle import oracle  # seeded inputs only; the oracle's arithmetic is not called here
     params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
-    lstm = {}
-    for mode, name in ((2, "persistent"), (1, "per_step_launches")):
+    lstm = {"persistent": None, "per_step_launches": None}
+    for mode, name in ((2, "persistent"), (1, "per_step_launches")) if "lstm" in sections else ():
         plan = P.LstmPlan([p.to(dev) for p in params], True, 2, False, 200)
         plan.set_mode(mode)
         xd, hd, cd = x.reshape(200, 240).to(dev), h0.to(dev), c0.to(dev)
@@ -170,19 +178,22 @@ def main():
         torch.cuda.synchronize()
         plan.status()
         lstm[name] = e0.elapsed_time(e1) * 1e3 / reps / 400
-    # input projection of layer 1 (T=200, I=1024, 4H=4096): the MFMA kernel
-    xp_x = torch.randn(200, 1024, device=dev).half()
-    xp_w = (0.03 * torch.randn(4096, 1024, device=dev)).half()
-    for _ in range(5):
-        P.input_projection(xp_x, xp_w)
-    torch.cuda.synchronize()
-    e0.record(stream)
-    for _ in range(50):
-        P.input_projection(xp_x, xp_w)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    xp_us = e0.elapsed_time(e1) * 1e3 / 50
-    xp_tflops = 2 * 200 * 1024 * 4096 / xp_us / 1e6
+    xp_us = xp_tflops = None
+    if "lstm" in sections:
+        # input projection of layer 1 (T=200, I=1024, 4H=4096): the MFMA kernel
+        xp_x = torch.randn(200, 1024, device=dev).half()
+        xp_w = (0.03 * torch.randn(4096, 1024, device=dev)).half()
+        for _ in range(5):
+            P.input_projection(xp_x, xp_w)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(50):
+            P.input_projection(xp_x, xp_w)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        xp_us = e0.elapsed_time(e1) * 1e3 / 50
+        xp_tflops = 2 * 200 * 1024 * 4096 / xp_us / 1e6
+    progress("lstm and input projection timed")
 
     # ---- the other kernels of the path (reported beside the headline figures, not part of `value`) ---------------
     def timed_us(fn, reps, warm=5):
@@ -197,94 +208,96 @@ def main():
         return e0.elapsed_time(e1) * 1e3 / reps
 
     other = {}
-    # GNMT-style stack: four at::lstm calls (L0 bidirectional I=1024, L1 I=2048, L2, L3 I=1024), T=50: 250 layer-steps
-    gn = []
-    seq = torch.randn(50, 1024, device=dev).half()
-    for li, (in_w, bidir) in enumerate([(1024, True), (2048, False), (1024, False), (1024, False)]):
-        prm, _, h0g, c0g = oracle.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
-        gn.append((P.LstmPlan([q.to(dev) for q in prm], True, 1, bidir, 50), h0g.to(dev), c0g.to(dev)))
+    if "other" in sections:
+        # GNMT-style stack: four at::lstm calls (L0 bidirectional I=1024, L1 I=2048, L2, L3 I=1024), T=50: 250 layer-steps
+        gn = []
+        seq = torch.randn(50, 1024, device=dev).half()
+        for li, (in_w, bidir) in enumerate([(1024, True), (2048, False), (1024, False), (1024, False)]):
+            prm, _, h0g, c0g = oracle.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
+            gn.append((P.LstmPlan([q.to(dev) for q in prm], True, 1, bidir, 50), h0g.to(dev), c0g.to(dev)))
 
-    def gnmt_stack():
-        cur = seq
-        for plan_g, hg, cg in gn:
-            cur, _, _ = plan_g.forward(cur, hg, cg)
+        def gnmt_stack():
+            cur = seq
+            for plan_g, hg, cg in gn:
+                cur, _, _ = plan_g.forward(cur, hg, cg)
 
-    other["gnmt_lstm_stack_us_per_layer_step"] = round(timed_us(gnmt_stack, 30) / 250, 3)
-    # one decoder step (seq_len 1, I = H = 1024): the fused step kernel, W_ih and W_hh streamed once (16.8 MB)
-    prm, _, h0d, c0d = oracle.lstm_inputs(4101, 1024, 1024, 1, False, 1)
-    plan_d = P.LstmPlan([q.to(dev) for q in prm], True, 1, False, 1)
-    xd1, h0d, c0d = torch.randn(1, 1024, device=dev).half(), h0d.to(dev).contiguous(), c0d.to(dev).contiguous()
-    yd1, hnd, cnd = torch.empty(1024, dtype=torch.float16, device=dev), torch.empty_like(h0d), torch.empty_like(c0d)
-    # (these small launches are timed through the C ABI on preallocated buffers: the operator layer's Python
-    # bookkeeping costs more than the kernels)
-    us = timed_us(lambda: lib.pimhip_lstm_forward(plan_d._handle, xd1.data_ptr(), h0d.data_ptr(), c0d.data_ptr(), yd1.data_ptr(),
-                                                  hnd.data_ptr(), cnd.data_ptr(), 1, sh), 200)
-    other["lstm_decode_step"] = {"us": round(us, 3), "gbs": round((2 * 4096 * 2048 + 8 * 4096) / us / 1e3, 1)}
-    # the same sweep as ONE grouped launch (executeMultiStream's siblings in one grid), cold
-    def grouped():
-        ws = []
+        other["gnmt_lstm_stack_us_per_layer_step"] = round(timed_us(gnmt_stack, 30) / 250, 3)
+        # one decoder step (seq_len 1, I = H = 1024): the fused step kernel, W_ih and W_hh streamed once (16.8 MB)
+        prm, _, h0d, c0d = oracle.lstm_inputs(4101, 1024, 1024, 1, False, 1)
+        plan_d = P.LstmPlan([q.to(dev) for q in prm], True, 1, False, 1)
+        xd1, h0d, c0d = torch.randn(1, 1024, device=dev).half(), h0d.to(dev).contiguous(), c0d.to(dev).contiguous()
+        yd1, hnd, cnd = torch.empty(1024, dtype=torch.float16, device=dev), torch.empty_like(h0d), torch.empty_like(c0d)
+        # (these small launches are timed through the C ABI on preallocated buffers: the operator layer's Python
+        # bookkeeping costs more than the kernels)
+        us = timed_us(lambda: lib.pimhip_lstm_forward(plan_d._handle, xd1.data_ptr(), h0d.data_ptr(), c0d.data_ptr(), yd1.data_ptr(),
+                                                      hnd.data_ptr(), cnd.data_ptr(), 1, sh), 200)
+        other["lstm_decode_step"] = {"us": round(us, 3), "gbs": round((2 * 4096 * 2048 + 8 * 4096) / us / 1e3, 1)}
+        # the same sweep as ONE grouped launch (executeMultiStream's siblings in one grid), cold
+        def grouped():
+            ws = []
+            for s_ in shapes:
+                ws.append(s_["pool"][s_["it"] % s_["copies"]])
+                s_["it"] += 1
+            P.execute_gemv_group([s_["x"] for s_ in shapes], ws, [s_["b"] for s_ in shapes])
+        us = timed_us(grouped, 100)
+        other["gemv_sweep_grouped_launch"] = {"us": round(us, 2), "gbs": round(step_bytes / us / 1e3, 1)}
+        # the sweep in the other operand order (y = x . A, A [in, out] row-major: the un-swapped addmm / matmul route); the
+        # same cold pools, read as [in, out]
+        vm_times = []
         for s_ in shapes:
-            ws.append(s_["pool"][s_["it"] % s_["copies"]])
-            s_["it"] += 1
-        P.execute_gemv_group([s_["x"] for s_ in shapes], ws, [s_["b"] for s_ in shapes])
-    us = timed_us(grouped, 100)
-    other["gemv_sweep_grouped_launch"] = {"us": round(us, 2), "gbs": round(step_bytes / us / 1e3, 1)}
-    # the sweep in the other operand order (y = x . A, A [in, out] row-major: the un-swapped addmm / matmul route); the
-    # same cold pools, read as [in, out]
-    vm_times = []
-    for s_ in shapes:
-        xv = (2 * torch.rand(s_["k"], generator=g, device=dev) - 1).half()
+            xv = (2 * torch.rand(s_["k"], generator=g, device=dev) - 1).half()
 
-        def vm_launch(s_=s_, xv=xv):
-            w = s_["pool"][s_["it"] % s_["copies"]]
-            s_["it"] += 1
-            rc = lib.pimhip_execute_gemv(s_["y"].data_ptr(), xv.data_ptr(), w.data_ptr(), s_["b"].data_ptr(), s_["k"], s_["n"], 0,
-                                         L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W, sh)
-            if rc != 0:
-                raise RuntimeError(lib.pimhip_last_error().decode())
-        us = timed_us(vm_launch, 50)
-        vm_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
-    other["gemv_vm_order"] = vm_times
-    # MoE FFN decode step (router 768 -> 8, then one expert 768 -> 3072 ReLU -> 768): three dependent launches on
-    # resident (warm) weights, the expert fixed so that no host round trip for the argmax is inside the figure
-    wr, w1, w2 = (0.02 * torch.randn(8, 768, device=dev)).half(), (0.02 * torch.randn(3072, 768, device=dev)).half(), \
-        (0.02 * torch.randn(768, 3072, device=dev)).half()
-    tok, logits = torch.randn(768, device=dev).half(), torch.empty(8, dtype=torch.float16, device=dev)
-    hid, yo = torch.empty(3072, dtype=torch.float16, device=dev), torch.empty(768, dtype=torch.float16, device=dev)
-
-    def moe_step():
-        lib.pimhip_execute_gemv(logits.data_ptr(), tok.data_ptr(), wr.data_ptr(), None, 768, 8, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
-        lib.pimhip_execute_gemv(hid.data_ptr(), tok.data_ptr(), w1.data_ptr(), None, 768, 3072, 0, L.PIMHIP_ACT_RELU, L.PIMHIP_W_X_I, sh)
-        lib.pimhip_execute_gemv(yo.data_ptr(), hid.data_ptr(), w2.data_ptr(), None, 3072, 768, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
-    other["moe_ffn_step_three_gemvs_us"] = round(timed_us(moe_step, 200), 3)
-    # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
-    big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
-    big_c = torch.empty_like(big_a)
-    us = timed_us(lambda: P.aten_add(big_a, big_b, out=big_c), 50)
-    other["add_32Mi"] = {"us": round(us, 2), "gbs": round(6 * (32 << 20) / us / 1e3, 1)}
-    sa, sb = big_a[:1].reshape(1, 1, 1024), big_b[:1].reshape(1, 1, 1024)
-    other["add_1024_us"] = round(timed_us(lambda: lib.pimhip_execute_add(sa.data_ptr(), sa.data_ptr(), sb.data_ptr(), 1, 1024, 0, sh), 200), 3)
-    del big_a, big_b, big_c
-    # attention context: y[1, 1024] = p[1, 50] . enc[50, 1024], stored to three buffers
-    pa, enc = torch.rand(1, 1, 50, device=dev).half(), torch.randn(1, 50, 1024, device=dev).half()
-    dsts = [torch.empty(1024, dtype=torch.float16, device=dev) for _ in range(3)]
-    import ctypes
-    dst_arr = (ctypes.c_void_p * 3)(*[d_.data_ptr() for d_ in dsts])
-    other["bmm_50x1024_three_destinations_us"] = round(
-        timed_us(lambda: lib.pimhip_execute_bmm(dst_arr, 3, pa.data_ptr(), enc.data_ptr(), 50, 1024, sh), 200), 3)
-    # the reference's own HIP GEMV (custom_ops.h addmv_kernel_Axy, compiled from its tree) on the same cold weights
-    ref = oracle.ref_lib()
-    if ref is not None:
-        ref_times = []
-        for s_ in shapes:
-            def ref_launch(s_=s_):
+            def vm_launch(s_=s_, xv=xv):
                 w = s_["pool"][s_["it"] % s_["copies"]]
                 s_["it"] += 1
-                ref.ref_addmv_Axy(sh, s_["b"].data_ptr(), w.data_ptr(), s_["x"].data_ptr(), s_["y"].data_ptr(), s_["n"], s_["k"], 0)
-            us = timed_us(ref_launch, 30)
-            ref_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
-        other["reference_hip_gemv_kernel"] = ref_times
+                rc = lib.pimhip_execute_gemv(s_["y"].data_ptr(), xv.data_ptr(), w.data_ptr(), s_["b"].data_ptr(), s_["k"], s_["n"], 0,
+                                             L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W, sh)
+                if rc != 0:
+                    raise RuntimeError(lib.pimhip_last_error().decode())
+            us = timed_us(vm_launch, 50)
+            vm_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
+        other["gemv_vm_order"] = vm_times
+        # MoE FFN decode step (router 768 -> 8, then one expert 768 -> 3072 ReLU -> 768): three dependent launches on
+        # resident (warm) weights, the expert fixed so that no host round trip for the argmax is inside the figure
+        wr, w1, w2 = (0.02 * torch.randn(8, 768, device=dev)).half(), (0.02 * torch.randn(3072, 768, device=dev)).half(), \
+            (0.02 * torch.randn(768, 3072, device=dev)).half()
+        tok, logits = torch.randn(768, device=dev).half(), torch.empty(8, dtype=torch.float16, device=dev)
+        hid, yo = torch.empty(3072, dtype=torch.float16, device=dev), torch.empty(768, dtype=torch.float16, device=dev)
 
+        def moe_step():
+            lib.pimhip_execute_gemv(logits.data_ptr(), tok.data_ptr(), wr.data_ptr(), None, 768, 8, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+            lib.pimhip_execute_gemv(hid.data_ptr(), tok.data_ptr(), w1.data_ptr(), None, 768, 3072, 0, L.PIMHIP_ACT_RELU, L.PIMHIP_W_X_I, sh)
+            lib.pimhip_execute_gemv(yo.data_ptr(), hid.data_ptr(), w2.data_ptr(), None, 3072, 768, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+        other["moe_ffn_step_three_gemvs_us"] = round(timed_us(moe_step, 200), 3)
+        # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
+        big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
+        big_c = torch.empty_like(big_a)
+        us = timed_us(lambda: P.aten_add(big_a, big_b, out=big_c), 50)
+        other["add_32Mi"] = {"us": round(us, 2), "gbs": round(6 * (32 << 20) / us / 1e3, 1)}
+        sa, sb = big_a[:1].reshape(1, 1, 1024), big_b[:1].reshape(1, 1, 1024)
+        other["add_1024_us"] = round(timed_us(lambda: lib.pimhip_execute_add(sa.data_ptr(), sa.data_ptr(), sb.data_ptr(), 1, 1024, 0, sh), 200), 3)
+        del big_a, big_b, big_c
+        # attention context: y[1, 1024] = p[1, 50] . enc[50, 1024], stored to three buffers
+        pa, enc = torch.rand(1, 1, 50, device=dev).half(), torch.randn(1, 50, 1024, device=dev).half()
+        dsts = [torch.empty(1024, dtype=torch.float16, device=dev) for _ in range(3)]
+        import ctypes
+        dst_arr = (ctypes.c_void_p * 3)(*[d_.data_ptr() for d_ in dsts])
+        other["bmm_50x1024_three_destinations_us"] = round(
+            timed_us(lambda: lib.pimhip_execute_bmm(dst_arr, 3, pa.data_ptr(), enc.data_ptr(), 50, 1024, sh), 200), 3)
+        # the reference's own HIP GEMV (custom_ops.h addmv_kernel_Axy, compiled from its tree) on the same cold weights
+        ref = oracle.ref_lib()
+        if ref is not None:
+            ref_times = []
+            for s_ in shapes:
+                def ref_launch(s_=s_):
+                    w = s_["pool"][s_["it"] % s_["copies"]]
+                    s_["it"] += 1
+                    ref.ref_addmv_Axy(sh, s_["b"].data_ptr(), w.data_ptr(), s_["x"].data_ptr(), s_["y"].data_ptr(), s_["n"], s_["k"], 0)
+                us = timed_us(ref_launch, 30)
+                ref_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
+            other["reference_hip_gemv_kernel"] = ref_times
+
+    progress("other kernels timed")
     # ---- CPU baseline: LibTorch CPU at::addmm in fp16 on the same sweep, bounded sample ---------------------------
     cpu = None
     if not args.no_cpu_baseline:
@@ -336,11 +349,12 @@ def main():
                    "bytes_per_step": step_bytes},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "gemv_per_shape": per_shape,
-        "lstm_us_per_layer_step": round(lstm["persistent"], 3),
-        "lstm_us_per_layer_step_per_step_launches": round(lstm["per_step_launches"], 3),
+        "lstm_us_per_layer_step": None if lstm["persistent"] is None else round(lstm["persistent"], 3),
+        "lstm_us_per_layer_step_per_step_launches": None if lstm["per_step_launches"] is None else round(lstm["per_step_launches"], 3),
         "lstm_config": "2 layers unidirectional, I=240, H=1024, T=200, batch 1 (400 layer-steps per call, input projection included)",
-        "input_projection": {"shape": "T=200, I=1024, 4H=4096", "us": round(xp_us, 2), "tflops": round(xp_tflops, 2),
-                             "mfma_utilisation": round(xp_tflops / MFMA_FP16_PEAK_TFLOPS, 5)},
+        "input_projection": None if xp_us is None else {
+            "shape": "T=200, I=1024, 4H=4096", "us": round(xp_us, 2), "tflops": round(xp_tflops, 2),
+            "mfma_utilisation": round(xp_tflops / MFMA_FP16_PEAK_TFLOPS, 5)},
         "other_kernels": other,
         "wall_ms_timed_region": round(wall_ms, 2),
         "roofline": roofline,

@@ -409,6 +409,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
         for (int k = 0; k < NC; ++k) a[k] = wave_sum_mod4(a[k]);
 
         half_t h_new[NC];
+        bool h_is_number[NC];
         float c_out[NC];
         const bool is_g = my_gate == 2;
 #pragma unroll
@@ -432,6 +433,8 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             const float g_g = dpp_mov_f32<0xAA>(act);
             const float g_o = dpp_mov_f32<0xFF>(act);
             const float c_new = g_f * c_reg[k] + g_i * g_g;
+            // h is NaN exactly when c_new or the output gate is; known here, before the tanh, off the critical path
+            h_is_number[k] = (c_new == c_new) && (g_o == g_o);
             const half_t h = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
             h_new[k] = active ? h : (half_t)0.0f;
             c_reg[k] = active ? c_new : c_reg[k];
@@ -445,10 +448,10 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             const unsigned int flag = (((p.g_base + (unsigned int)tau) >> 1) & 1u) << 14;
 #pragma unroll
             for (int k = 0; k < NC; ++k) {
-                unsigned int hbits = unit_ok ? (unsigned int)__builtin_bit_cast(unsigned short, h_new[k]) : 0u;
                 // A NaN (from non-finite inputs or weights) has bit 14 set and cannot travel with the flag: y, hn and
-                // cn below still receive it, the recurrence continues from 0 for this unit instead of waiting forever.
-                if ((hbits & 0x7c00u) == 0x7c00u) hbits = 0u;
+                // cn below still receive it, the exchange carries 0 for this unit instead of making every reader wait
+                // for a flag that never matches.
+                const unsigned int hbits = (unit_ok && h_is_number[k]) ? (unsigned int)__builtin_bit_cast(unsigned short, h_new[k]) : 0u;
                 pub[k][wave] = (unsigned short)(hbits | flag);
             }
             if (unit_ok) {
