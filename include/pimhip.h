@@ -95,7 +95,12 @@ int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* other_shape4
  *   order == PIMHIP_I_X_W: weight is [in_w, out_w] row-major with row pitch ld_weight (elements)
  * out[out_w] = act(sum_k weight * in[k] + bias[out_w]); bias may be NULL.  fp32 accumulation, one
  * rounding to fp16 at the store.  As in the reference's VM/MV branches there is no alpha/beta
- * (aten_ops.cpp:627-628).  ld_weight == 0 selects the dense pitch. */
+ * (aten_ops.cpp:627-628).  ld_weight == 0 selects the dense pitch.
+ * The I_X_W order splits the reduction over blocks for all but small weights; the blocks exchange partial sums through
+ * a per-stream workspace the library allocates on the first such call on a stream (the call synchronises that stream
+ * then, and again whenever a later call needs a larger workspace).  Calls that share a stream must not overlap.  Every
+ * wait inside the kernel is bounded; should one ever give up, the next I_X_W call on that stream returns
+ * PIMHIP_ERR_TIMEOUT (the earlier result is undefined), re-initialises the workspace and launches nothing. */
 int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
                         int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
 

@@ -179,11 +179,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_generic_kernel(const h
 // A block owns CW = 8 * LPR adjacent outputs and a slice [k_begin, k_end) of the reduction.  LPR lanes (8 columns,
 // one 16-byte load each) cover the block's part of one weight row, so a wavefront reads 64 / LPR rows per load
 // instruction and the block's wavefronts interleave over the rows of the slice, U loads in flight per lane.
-// gridDim.y slices cover K.  With one slice the block finishes the outputs itself; with several, each block writes
-// its CW partial sums (fp32) to `partial[slice][N]` and takes a ticket from `tickets[blockIdx.x]`; the block that
-// draws the last ticket adds the slices with all its lanes, in an order that depends on the slice index only (so the
-// result does not depend on which block finishes last), applies the epilogue and re-arms the ticket counter for
-// the next launch.
+// gridDim.y slices cover K.  With one slice the block finishes the outputs itself.  With several, the blocks of all
+// slices but the last store their CW partial sums (fp32) as 32-byte records in `partial[slice][N]` and exit; the blocks
+// of the LAST slice add the records to their own sums, in an order that depends on the slice index only (so the result
+// is the same in every run), and apply the epilogue.
+//
+// A record that has not arrived yet holds kVmEmpty in every word (the bit pattern 0xffffffff: a NaN that no sum of
+// products of fp16 values can be, since arithmetic yields the canonical NaN or the widened payload of an fp16 NaN), so
+// the reducing block polls each record until none of its words is kVmEmpty, adds it and writes kVmEmpty back for the
+// next launch.  Records travel with device-scope (sc1) stores and loads; there is no fence (a device-scope fence writes
+// back and invalidates the XCD's whole L2, once per block) and no ticket counter (store, acknowledgement, atomic,
+// loads would be three trips through the memory side after the last block's arithmetic; polling is one).  Blocks are
+// dispatched in order of their linear id, so the reducing blocks start last; the producers never wait for anything, so
+// they finish whatever else occupies the GPU.  A wait still is bounded: after `spin_limit` polls the lane sets *status
+// (host-visible) and goes on with what it has; the host then reports the failure and re-initialises the records.
 // ---------------------------------------------------------------------------------------------
 // Destinations of a VM product: the same result is stored to `count` buffers (the GNMT attention context goes
 // straight into three concatenation buffers, runtime/source/executor/op_executor/aten_ops_executor.cpp:694-737).
@@ -193,27 +202,22 @@ struct GemvOuts {
     int count;
 };
 
-// 32 contiguous bytes written / read at device scope (partial sums cross CUs and XCDs).  The loads of one call are
-// issued together and waited for once.
+// 32 contiguous bytes written at device scope (partial sums cross CUs and XCDs).
 __device__ __forceinline__ void store32_device_scope(float* p, const float (&v)[8])
 {
     const float4_t lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\tglobal_store_dwordx4 %0, %2, off offset:16 sc1" : : "v"(p), "v"(lo), "v"(hi) : "memory");
 }
-template <int B>
-__device__ __forceinline__ void load32_device_scope(const float* const (&p)[B], float4_t (&lo)[B], float4_t (&hi)[B])
+// One 32-byte record of partial sums read at device scope (both halves issued together, one wait).
+__device__ __forceinline__ void load32_device_scope_one(const float* p, float4_t& lo, float4_t& hi)
 {
-    static_assert(B == 4, "four slices per batch");
-    asm volatile(
-        "global_load_dwordx4 %0, %8, off sc1\n\tglobal_load_dwordx4 %1, %8, off offset:16 sc1\n\t"
-        "global_load_dwordx4 %2, %9, off sc1\n\tglobal_load_dwordx4 %3, %9, off offset:16 sc1\n\t"
-        "global_load_dwordx4 %4, %10, off sc1\n\tglobal_load_dwordx4 %5, %10, off offset:16 sc1\n\t"
-        "global_load_dwordx4 %6, %11, off sc1\n\tglobal_load_dwordx4 %7, %11, off offset:16 sc1\n\t"
-        "s_waitcnt vmcnt(0)"
-        : "=&v"(lo[0]), "=&v"(hi[0]), "=&v"(lo[1]), "=&v"(hi[1]), "=&v"(lo[2]), "=&v"(hi[2]), "=&v"(lo[3]), "=&v"(hi[3])
-        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3])
-        : "memory");
+    asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(lo), "=&v"(hi)
+                 : "v"(p)
+                 : "memory");
 }
+
+static constexpr unsigned int kVmEmpty = 0xffffffffu;
 
 template <int WAVES, int U, int LPR>
 __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* __restrict__ x,
@@ -221,14 +225,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
                                                                  const half_t* __restrict__ bias,
                                                                  GemvOuts outs, int K, int N, long lda,
                                                                  int relu, int k_per_slice, float* partial,
-                                                                 unsigned int* tickets)
+                                                                 unsigned int* status, unsigned int spin_limit)
 {
     static_assert(LPR == 16 || LPR == 32 || LPR == 64, "lanes per weight row");
     constexpr int RPW = 64 / LPR;          // rows per wavefront and load instruction
     constexpr int GROUPS = WAVES * RPW;    // row groups per block = LDS rows of the reduction
     constexpr int STEP = GROUPS;           // rows between consecutive loads of one lane
     __shared__ float red[GROUPS][8][LPR];
-    __shared__ unsigned int s_ticket;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -302,46 +305,46 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
         return;
     }
 
-    // The partial sums travel with device-scope stores and loads (write-through / read-through the XCD's L2), so no
-    // fence is needed, and none is wanted: a device-scope fence writes back and invalidates the whole L2, once per
-    // block.  The stores are complete (acknowledged) before the block's ticket is drawn; the last block's loads are
-    // issued after it has seen the last ticket.
-    if (finisher) {
-        store32_device_scope(partial + (long)blockIdx.y * N + col0, acc);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const int last = nslices - 1;
+    if ((int)blockIdx.y != last) {
+        if (finisher) store32_device_scope(partial + (long)blockIdx.y * N + col0, acc);
+        return;
     }
-    __syncthreads();
-    if (tid == 0) s_ticket = __hip_atomic_fetch_add(tickets + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (s_ticket != (unsigned int)(nslices - 1)) return;
-
-    // Row group g of the block adds slices g, g + GROUPS, ... (four loads of 32 bytes in flight), then the groups are
-    // added in group order as above.
+    float own[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    for (int j = 0; j < 8; ++j) {
+        own[j] = acc[j];  // meaningful in the finisher lanes
+        acc[j] = 0.0f;
+    }
+    // Row group g adds the records of slices g, g + GROUPS, ... < last in that order.
     if (col_ok) {
-        const float* base = partial + col0;
-        int sl = grp;
-        for (; sl + 3 * GROUPS < nslices; sl += 4 * GROUPS) {
-            const float* const ptr[4] = {base + (long)sl * N, base + (long)(sl + GROUPS) * N, base + (long)(sl + 2 * GROUPS) * N,
-                                         base + (long)(sl + 3 * GROUPS) * N};
-            float4_t lo[4], hi[4];
-            load32_device_scope<4>(ptr, lo, hi);
+        for (int sl = grp; sl < last; sl += GROUPS) {
+            float* rec = partial + (long)sl * N + col0;
+            float4_t lo, hi;
+            unsigned int spins = 0;
+            while (true) {
+                load32_device_scope_one(rec, lo, hi);
+                bool ok = true;
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    acc[j] += lo[b][j];
-                    acc[4 + j] += hi[b][j];
+                for (int j = 0; j < 4; ++j)
+                    ok = ok && __builtin_bit_cast(unsigned int, lo[j]) != kVmEmpty && __builtin_bit_cast(unsigned int, hi[j]) != kVmEmpty;
+                if (ok) break;
+                if (++spins > spin_limit) {
+                    __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    break;
                 }
             }
-        }
-        for (; sl < nslices; sl += GROUPS) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-                acc[j] += __hip_atomic_load(base + (long)sl * N + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int j = 0; j < 4; ++j) {
+                acc[j] += lo[j];
+                acc[4 + j] += hi[j];
+            }
+            const float e = __builtin_bit_cast(float, kVmEmpty);
+            const float empty[8] = {e, e, e, e, e, e, e, e};
+            store32_device_scope(rec, empty);
         }
     }
+    __syncthreads();  // the first lanes have read `red` above before it is written again
 #pragma unroll
     for (int j = 0; j < 8; ++j) red[grp][j][cg] = acc[j];
     __syncthreads();
@@ -352,10 +355,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
             v[j] = red[0][j][cg];
 #pragma unroll
             for (int g = 1; g < GROUPS; ++g) v[j] += red[g][j][cg];
+            v[j] += own[j];
         }
         epilogue_store(v);
     }
-    if (tid == 0) __hip_atomic_store(tickets + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // VM order, any N / leading dimension / alignment: one lane per output column, 2-byte loads.

@@ -45,10 +45,10 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 // ---- per-device state --------------------------------------------------------------------------
 struct SplitWorkspace {
-    float* partial = nullptr;        // [slices][N] fp32 partial sums of the VM kernel
+    float* partial = nullptr;            // [slices][N] fp32 records of the VM kernel; every word kVmEmpty between launches
     size_t partial_elems = 0;
-    unsigned int* tickets = nullptr; // one arrival counter per column block, zero between launches
-    size_t ticket_count = 0;
+    unsigned int* status = nullptr;      // pinned host word the kernel sets when a wait for a record gives up
+    unsigned int* status_dev = nullptr;  // the same word as the device addresses it
 };
 
 struct DeviceState {
@@ -72,28 +72,31 @@ int current_device_state(DeviceState** out)
     return PIMHIP_OK;
 }
 
-int get_split_workspace(DeviceState* st, hipStream_t stream, size_t partial_elems, size_t ticket_count,
-                        SplitWorkspace** out)
+int get_split_workspace(DeviceState* st, hipStream_t stream, size_t partial_elems, SplitWorkspace** out)
 {
     std::lock_guard<std::mutex> lock(g_mutex);
     SplitWorkspace& ws = st->workspaces[stream];
-    if (ws.partial_elems < partial_elems) {
+    if (!ws.status) {
+        PIMHIP_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&ws.status), sizeof(unsigned int), hipHostMallocMapped));
+        *ws.status = 0u;
+        PIMHIP_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&ws.status_dev), ws.status, 0));
+    }
+    const bool gave_up = *ws.status != 0u;
+    if (ws.partial_elems < partial_elems || gave_up) {
         // Work already queued on this stream may still use the old buffer.
         PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
-        if (ws.partial) PIMHIP_HIP_CHECK(hipFree(ws.partial));
-        ws.partial = nullptr;
-        ws.partial_elems = 0;
-        PIMHIP_HIP_CHECK(hipMalloc(&ws.partial, partial_elems * sizeof(float)));
-        ws.partial_elems = partial_elems;
-    }
-    if (ws.ticket_count < ticket_count) {
-        PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
-        if (ws.tickets) PIMHIP_HIP_CHECK(hipFree(ws.tickets));
-        ws.tickets = nullptr;
-        ws.ticket_count = 0;
-        PIMHIP_HIP_CHECK(hipMalloc(&ws.tickets, ticket_count * sizeof(unsigned int)));
-        PIMHIP_HIP_CHECK(hipMemsetAsync(ws.tickets, 0, ticket_count * sizeof(unsigned int), stream));
-        ws.ticket_count = ticket_count;
+        if (ws.partial_elems < partial_elems) {
+            if (ws.partial) PIMHIP_HIP_CHECK(hipFree(ws.partial));
+            ws.partial = nullptr;
+            ws.partial_elems = 0;
+            PIMHIP_HIP_CHECK(hipMalloc(&ws.partial, partial_elems * sizeof(float)));
+            ws.partial_elems = partial_elems;
+        }
+        PIMHIP_HIP_CHECK(hipMemsetAsync(ws.partial, 0xff, ws.partial_elems * sizeof(float), stream));  // every word kVmEmpty
+        *ws.status = 0u;
+        if (gave_up)
+            return fail(PIMHIP_ERR_TIMEOUT, "an earlier GEMV on this stream gave up waiting for partial sums; its result is undefined "
+                                            "(the workspace has been re-initialised, this call was not launched)");
     }
     *out = &ws;
     return PIMHIP_OK;
@@ -134,6 +137,10 @@ int gemv_mv(const half_t* W, const half_t* x, const half_t* bias, half_t* y, int
     return PIMHIP_OK;
 }
 
+// Polls of one record before a reducing lane of the VM kernel gives up (seconds; a record normally arrives within
+// microseconds of its producer's last load).
+constexpr unsigned int kVmSpinLimit = 1u << 22;
+
 int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bias, const GemvOuts& outs, int64_t K,
             int64_t N, int64_t lda, int relu, hipStream_t s)
 {
@@ -145,7 +152,7 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
         return PIMHIP_OK;
     }
     // Measured on MI355X: 128-column blocks (16 lanes per weight row, 4 rows per wavefront and load) with 8 loads in
-    // flight per lane are fastest for every shape tried; a cross-block reduction costs about 3 us, so K is sliced
+    // flight per lane are fastest for every shape tried; a cross-block reduction costs 1 to 2 us, so K is sliced
     // only as far as needed for roughly one block per CU (64 blocks for a weight of a few MB), and not at all for
     // weights of up to 256 KB.
     constexpr int WAVES = 4, U = 8, LPR = 16;
@@ -167,16 +174,16 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     if (slices < 1) slices = 1;
     SplitWorkspace* ws = nullptr;
     float* partial = nullptr;
-    unsigned int* tickets = nullptr;
+    unsigned int* status = nullptr;
     if (slices > 1) {
-        int rc = get_split_workspace(st, s, (size_t)slices * (size_t)N, (size_t)col_blocks, &ws);
+        int rc = get_split_workspace(st, s, (size_t)slices * (size_t)N, &ws);
         if (rc != PIMHIP_OK) return rc;
         partial = ws->partial;
-        tickets = ws->tickets;
+        status = ws->status_dev;
     }
     dim3 grid(col_blocks, slices);
     gemv_vm_f16_kernel<WAVES, U, LPR><<<grid, WAVES * 64, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu,
-                                                                    k_per_slice, partial, tickets);
+                                                                    k_per_slice, partial, status, kVmSpinLimit);
     return PIMHIP_OK;
 }
 
@@ -508,7 +515,7 @@ extern "C" int pimhip_deinitialize(void)
         hipDeviceSynchronize();
         for (auto& w : kv.second.workspaces) {
             if (w.second.partial) hipFree(w.second.partial);
-            if (w.second.tickets) hipFree(w.second.tickets);
+            if (w.second.status) hipHostFree(w.second.status);
         }
         kv.second.workspaces.clear();
         kv.second.initialized = false;
