@@ -209,7 +209,8 @@ struct LstmSeqChain {
 struct LstmSeqArgs {
     LstmSeqChain chain[kSeqMaxChains];
     unsigned int* hx;          // [2][NB][kSeqEntryWords]; zero when g_base == 2
-    unsigned int* abort_flag;  // set to 1 when a wait gives up
+    unsigned int* abort_flag;  // set to 1 when a wait gives up; polled by the other waiting lanes
+    unsigned int* abort_host;  // host-visible word set at the same time (what the host reads afterwards)
     long y_stride;             // elements between consecutive time steps of y
     int H;
     int T;
@@ -345,6 +346,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
                     }
                     if (spins >= p.spin_limit) {
                         __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                         gave_up = true;
                     }
                 }

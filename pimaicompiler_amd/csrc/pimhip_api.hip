@@ -468,7 +468,8 @@ struct PimHipLstmPlan {
     float* c_state = nullptr;         // [num_dirs][H] fp32, per-step kernel's cell state
     unsigned int* hx = nullptr;       // [kSeqMaxChains][2][NB][kSeqEntryWords] exchange entries of the sequence kernel
     unsigned int* abort_flag = nullptr;
-    unsigned int* abort_host = nullptr;  // pinned copy read by pimhip_lstm_plan_status
+    unsigned int* abort_host = nullptr;      // pinned host word the kernel sets with the flag; read by pimhip_lstm_plan_status
+    unsigned int* abort_host_dev = nullptr;  // the same word as the device addresses it
     int seq_blocks = 0;
     bool reset_exchange = false;     // the next forward starts from a cleared exchange buffer (layout change)
     bool seq_units8_ok = false;      // a single chain may run with 8 hidden units per block (half as many blocks)
@@ -598,8 +599,9 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
     PLAN_HIP_CHECK(hipMalloc(&plan->c_state, sizeof(float) * (size_t)D * H));
     PLAN_HIP_CHECK(hipMalloc(&plan->abort_flag, sizeof(unsigned int)));
     PLAN_HIP_CHECK(hipMemsetAsync(plan->abort_flag, 0, sizeof(unsigned int), s));
-    PLAN_HIP_CHECK(hipHostMalloc(&plan->abort_host, sizeof(unsigned int), hipHostMallocDefault));
+    PLAN_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&plan->abort_host), sizeof(unsigned int), hipHostMallocMapped));
     *plan->abort_host = 0;
+    PLAN_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&plan->abort_host_dev), plan->abort_host, 0));
 
     // Persistent sequence kernel: one block per 4 hidden units (one unit per wavefront, weights in registers),
     // all blocks resident at once.
@@ -757,6 +759,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             }
             a.hx = plan->hx + plan->hx_region_words * (size_t)(nc - 1);
             a.abort_flag = plan->abort_flag;
+            a.abort_host = plan->abort_host_dev;
             a.y_stride = y_stride;
             a.H = (int)H;
             a.T = (int)T;
@@ -819,7 +822,5 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             layer_in = layer_out;
         }
     }
-    if (use_seq)
-        PIMHIP_HIP_CHECK(hipMemcpyAsync(plan->abort_host, plan->abort_flag, sizeof(unsigned int), hipMemcpyDeviceToHost, s));
     return PIMHIP_OK;
 }
