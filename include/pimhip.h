@@ -152,7 +152,9 @@ int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan);
  *   h0, c0 [num_layers*num_directions, hidden_size]
  *   y  [seq_len, num_directions*hidden_size]
  *   hn, cn [num_layers*num_directions, hidden_size], ordered (l0 fwd, l0 bwd, l1 fwd, ...)
- * y, hn, cn may not alias x, h0, c0.  Calls sharing one plan must be ordered on one stream. */
+ * y, hn, cn may not alias x, h0, c0.  Calls sharing one plan must be ordered on one stream.  Sequences of two or more
+ * steps run in a kernel that needs all its blocks resident at once: a call on another stream than the device's
+ * previous such call is ordered after it (an event wait), so that two of them never share the GPU. */
 int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn,
                         void* cn, int64_t seq_len, void* stream);
 

@@ -55,6 +55,12 @@ struct DeviceState {
     bool initialized = false;
     int num_cus = 0;
     std::map<hipStream_t, SplitWorkspace> workspaces;  // one per stream: sibling GEMVs on different streams must not share
+    // The persistent LSTM kernel needs all its blocks resident at once.  Two of them issued on different streams could
+    // each get part of the GPU and wait for the rest forever, so a launch on another stream than the previous one is
+    // ordered after it with an event (nothing is added while one stream is used).
+    bool seq_launched = false;
+    hipStream_t seq_stream = nullptr;
+    hipEvent_t seq_event = nullptr;
 };
 
 std::mutex g_mutex;
@@ -519,6 +525,7 @@ extern "C" int pimhip_deinitialize(void)
             if (w.second.status) hipHostFree(w.second.status);
         }
         kv.second.workspaces.clear();
+        if (kv.second.seq_event) hipEventDestroy(kv.second.seq_event);
         kv.second.initialized = false;
     }
     g_devices.clear();
@@ -671,6 +678,26 @@ extern "C" int pimhip_lstm_plan_status(PimHipLstmPlan* plan)
     return PIMHIP_OK;
 }
 
+namespace
+{
+int order_after_previous_sequence_launch(DeviceState* st, hipStream_t s)
+{
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (st->seq_launched && st->seq_stream != s) {
+        if (!st->seq_event) PIMHIP_HIP_CHECK(hipEventCreateWithFlags(&st->seq_event, hipEventDisableTiming));
+        // The event marks everything queued on the other stream so far, the earlier sequence kernel included.  That
+        // stream may have been destroyed since: then there is nothing left to wait for.
+        if (hipEventRecord(st->seq_event, st->seq_stream) == hipSuccess)
+            PIMHIP_HIP_CHECK(hipStreamWaitEvent(s, st->seq_event, 0));
+        else
+            (void)hipGetLastError();
+    }
+    st->seq_launched = true;
+    st->seq_stream = s;
+    return PIMHIP_OK;
+}
+}  // namespace
+
 extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y,
                                    void* hn, void* cn, int64_t seq_len, void* stream)
 {
@@ -725,6 +752,8 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     const half_t* layer_in = (const half_t*)x;
     const long y_stride = (long)D * H;
     if (use_seq) {
+        rc = order_after_previous_sequence_launch(st, s);
+        if (rc != PIMHIP_OK) return rc;
         // Layers are taken in groups that one persistent launch advances together: the two directions of a
         // bidirectional layer, or up to kSeqMaxChains consecutive layers of a unidirectional stack as a wavefront.
         int l = 0;

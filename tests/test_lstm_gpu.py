@@ -238,6 +238,30 @@ def test_switching_the_block_shape_on_one_plan_restarts_the_exchange(ops):
         assert torch.equal(first.setdefault(mode, y), y)
 
 
+def test_sequence_kernels_issued_on_two_streams_do_not_starve_each_other(ops):
+    """Each persistent launch needs the whole GPU's worth of resident blocks; launches on different streams are ordered
+    one after the other by the library.  (Bounded all the same: a short spin limit turns a mistake into a time-out.)"""
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    cases = []
+    for i, st in enumerate(streams):
+        params, x, h0, c0 = oracle.lstm_inputs(200 + i, 64, 1024, 2, False, 40)
+        plan = ops.LstmPlan([p.to(DEV) for p in params], True, 2, False, 40)
+        plan.set_mode(2)
+        plan.set_spin_limit(1 << 16)
+        cases.append((plan, st, x.reshape(40, 64).to(DEV), h0.to(DEV), c0.to(DEV), oracle.torch_lstm(x, h0, c0, params, True, 2, False)))
+    torch.cuda.synchronize()
+    outs = []
+    for _ in range(4):                       # alternate the streams without synchronising in between
+        for plan, st, x, h0, c0, _want in cases:
+            outs.append(plan.forward(x, h0, c0, stream=st))
+    torch.cuda.synchronize()
+    for plan, *_ in cases:
+        plan.status()
+    for k, (y, hn, cn) in enumerate(outs):
+        want = cases[k % 2][5]
+        assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
+
+
 # ---- the bounded wait ---------------------------------------------------------------------------------------------
 def test_persistent_kernel_wait_gives_up_and_reports(ops):
     """Forced from the host: with a spin limit of 0 every wait gives up at its first unsuccessful poll, the kernel
