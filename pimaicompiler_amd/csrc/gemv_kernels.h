@@ -361,20 +361,44 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
     }
 }
 
-// VM order, any N / leading dimension / alignment: one lane per output column, 2-byte loads.
-__global__ __launch_bounds__(256) void gemv_vm_f16_generic_kernel(const half_t* __restrict__ x,
-                                                                  const half_t* __restrict__ A,
-                                                                  const half_t* __restrict__ bias,
-                                                                  GemvOuts outs, int K, int N, long lda,
-                                                                  int relu)
+// VM order, any N / leading dimension / alignment: 2-byte loads.  A block of 16 wavefronts owns 64 adjacent output
+// columns (one per lane); wavefront g takes the rows g, g + 16, ... and the sixteen partial sums meet in LDS.
+static constexpr int kVmGenericWaves = 16;
+__global__ __launch_bounds__(64 * kVmGenericWaves) void gemv_vm_f16_generic_kernel(const half_t* __restrict__ x,
+                                                                                   const half_t* __restrict__ A,
+                                                                                   const half_t* __restrict__ bias,
+                                                                                   GemvOuts outs, int K, int N, long lda,
+                                                                                   int relu)
 {
-    const long col = (long)blockIdx.x * 256 + threadIdx.x;
-    if (col >= N) return;
+    __shared__ float red[kVmGenericWaves][64];
+    const int lane = threadIdx.x & 63;
+    const int g = threadIdx.x >> 6;
+    const long col = (long)blockIdx.x * 64 + lane;
     float acc = 0.0f;
-    for (int k = 0; k < K; ++k) acc = fmaf((float)A[(long)k * lda + col], (float)x[k], acc);
-    if (bias) acc += (float)bias[col];
-    if (relu) acc = fmaxf(acc, 0.0f);
-    for (int o = 0; o < outs.count; ++o) outs.y[o][col] = (half_t)acc;
+    if (col < N) {
+        int k = g;
+        for (; k + 3 * kVmGenericWaves < K; k += 4 * kVmGenericWaves) {
+            half_t a[4], xv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                a[u] = A[(long)(k + u * kVmGenericWaves) * lda + col];
+                xv[u] = x[k + u * kVmGenericWaves];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc = fmaf((float)a[u], (float)xv[u], acc);
+        }
+        for (; k < K; k += kVmGenericWaves) acc = fmaf((float)A[(long)k * lda + col], (float)x[k], acc);
+    }
+    red[g][lane] = acc;
+    __syncthreads();
+    if (g == 0 && col < N) {
+        float v = red[0][lane];
+#pragma unroll
+        for (int w = 1; w < kVmGenericWaves; ++w) v += red[w][lane];
+        if (bias) v += (float)bias[col];
+        if (relu) v = fmaxf(v, 0.0f);
+        for (int o = 0; o < outs.count; ++o) outs.y[o][col] = (half_t)v;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -153,8 +153,8 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     bool vec_ok = (N % 8 == 0) && (lda % 8 == 0) && aligned16(A);
     for (int o = 0; o < outs.count; ++o) vec_ok = vec_ok && aligned16(outs.y[o]);
     if (!vec_ok) {
-        const int grid = (int)((N + 255) / 256);
-        gemv_vm_f16_generic_kernel<<<grid, 256, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu);
+        const int grid = (int)((N + 63) / 64);
+        gemv_vm_f16_generic_kernel<<<grid, 64 * kVmGenericWaves, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu);
         return PIMHIP_OK;
     }
     // Measured on MI355X: 128-column blocks (16 lanes per weight row, 4 rows per wavefront and load) with 8 loads in
