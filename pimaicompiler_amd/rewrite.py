@@ -14,7 +14,11 @@ pass_manager.cpp:36-82):
 what the reference leaves to run time: every  T -> addmm/matmul(Wconst, .) -> T  sandwich becomes ONE fused
 `gemv` op on the weight's own row-major bytes (bias and ReLU in the epilogue), so the two transposes and the
 `.contiguous()` copies of customAtenAddmm (runtime/source/executor/op_executor/aten_ops.cpp:630-632, 663-665)
-disappear.  `execute` runs a graph through the operator layer (pimaicompiler_amd.ops) on the GPU.
+disappear.  `multi_stream_execution` restates the middle-end pass of the same name
+(compiler/source/middlend/optimizer/stream_execution/multi_stream_execution.cpp:20-290): sibling products that feed
+one join and hang off one common start are collected into a single `multi_stream` op, which runs as ONE grouped launch
+here where the reference gives each sibling its own stream.  `execute` runs a graph through the operator layer
+(pimaicompiler_amd.ops) on the GPU.
 
 remove_cat_for_addmm is restated for any split point; the reference hard-codes the RNNT joint shapes
 ([1,1024] + [1,320] against a [512,1344] weight, compiler/include/frontend/optimizer/remove_cat_for_addmm.h:77-79).
@@ -169,6 +173,81 @@ def lower_to_hot_path(g: Graph):
     return g
 
 
+# ---- sibling products into one op ------------------------------------------------------------------------------------
+_STREAM_TYPES = ("aten::addmm", "aten::matmul", "pimhip::gemv")
+
+
+def _producers(g: Graph, op: Op):
+    """Distinct non-constant ops that produce the inputs of `op`, in input order."""
+    out = []
+    for t in op.inputs:
+        p = None if g.is_constant(t) else g.producer(t)
+        if p is not None and p.type != "prim::Constant" and all(p is not q for q in out):
+            out.append(p)
+    return out
+
+
+def _backward(g: Graph, root: Op, max_level: int, stop=None):
+    """Breadth-first list of `root` and its non-constant ancestors, at most `max_level` levels up, not beyond `stop`."""
+    seen, frontier = [root], [root]
+    for _ in range(max_level):
+        nxt = []
+        for op in frontier:
+            if op is stop:
+                continue
+            for p in _producers(g, op):
+                if all(p is not q for q in seen):
+                    seen.append(p)
+                    nxt.append(p)
+        frontier = nxt
+    return seen
+
+
+def multi_stream_execution(g: Graph, max_search_level: int = 10):
+    """A join (an op with several non-constant producers) whose branches each contain a product, all hanging off one
+    common start op: the products become one `multi_stream` op placed after the branches' preparation ops
+    (multi_stream_execution.cpp: fitCondition :20-72, backwardToCheckAndFindStartLayer :96-228, process :230-290)."""
+    for join in list(g.ops):
+        if all(join is not o for o in g.ops):
+            continue
+        branches = _producers(g, join)
+        if len(branches) < 2:
+            continue
+        members = []
+        for b in branches:
+            found = next((o for o in _backward(g, b, max_search_level) if o.type in _STREAM_TYPES), None)
+            if found is None or any(found is m for m in members):
+                members = []
+                break
+            members.append(found)
+        if len(members) < 2:
+            continue
+        # no product may feed another one
+        if any(any(a is x for x in _backward(g, m, max_search_level)[1:]) for m in members for a in members if a is not m):
+            continue
+        ancestors = [_backward(g, m, max_search_level)[1:] for m in members]
+        start = next((a for a in ancestors[0] if a.type not in _STREAM_TYPES and all(any(a is x for x in anc) for anc in ancestors[1:])), None)
+        if start is None:
+            continue
+        prep = []
+        for m in members:
+            for a in _backward(g, m, max_search_level, stop=start)[1:]:
+                if a is not start and all(a is not q for q in prep):
+                    prep.append(a)
+        pos_start = g.ops.index(start)
+        if any(g.ops.index(a) < pos_start for a in prep):
+            continue                     # a branch takes something from before the start: leave the order alone
+        prep.sort(key=g.ops.index)
+        for a in prep + members:
+            g.ops.remove(a)
+        at = g.ops.index(start) + 1
+        g.ops[at:at] = prep
+        group = Op("multi_stream", [t for m in members for t in m.inputs], [t for m in members for t in m.outputs],
+                   {"layers": members})
+        g.ops.insert(at + len(prep), group)
+    return g
+
+
 # ---- execution through the operator layer ----------------------------------------------------------------------------
 def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0"):
     """Runs the op list with pimaicompiler_amd.ops; returns the graph outputs.  Constants are moved to `device`."""
@@ -186,6 +265,27 @@ def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0"):
             r = ops.custom_aten_matmul(a[0], a[1])
         elif op.type == "pimhip::gemv":
             r = ops.aten_linear(a[0], a[1], a[2] if op.attrs["has_bias"] else None, act_type=op.attrs["act_type"])
+        elif op.type == "multi_stream":
+            subs = op.attrs["layers"]
+            if all(m.type == "pimhip::gemv" for m in subs):
+                xs = [env[m.inputs[0]] for m in subs]
+                outs = ops.execute_gemv_group(xs, [env[m.inputs[1]] for m in subs],
+                                              [env[m.inputs[2]] if m.attrs["has_bias"] else None for m in subs],
+                                              [m.attrs["act_type"] for m in subs])
+                for m, x, o in zip(subs, xs, outs):
+                    env[m.outputs[0]] = o.view(list(x.shape[:-1]) + [o.numel()])
+            else:
+                for m in subs:
+                    am = [env[i] for i in m.inputs]
+                    env[m.outputs[0]] = (ops.custom_aten_addmm(m.attrs.get("act_type", "none"), am[0], am[1], am[2])
+                                         if m.type == "aten::addmm" else ops.custom_aten_matmul(am[0], am[1]))
+            continue
+        elif op.type == "aten::contiguous":
+            r = a[0].contiguous()
+        elif op.type == "aten::slice":
+            r = a[0].narrow(op.attrs["dim"], op.attrs["start"], op.attrs["end"] - op.attrs["start"])
+        elif op.type == "aten::add":
+            r = ops.aten_add(a[0], a[1])
         elif op.type == "aten::transpose":
             r = a[0].transpose(op.attrs["dim0"], op.attrs["dim1"])
         elif op.type == "aten::relu":

@@ -105,3 +105,96 @@ def test_rewritten_graphs_compute_what_eager_libtorch_computes(ops):
         assert list(y.shape) == [1, 512], stage
         # two roundings (the split product is rounded to fp16 in between): 2 x 2e-3
         assert float((y.float().cpu() - want).abs().max()) <= 4e-3, stage
+
+
+def attention_projection_graph(seed=3, d=512, n=4, constant_weights=True):
+    """The structure the reference's multi-stream pass looks for (multi_stream_execution.h:24-41): one start op, n
+    branches ending in matmul -> add, joined by a ListConstruct.  With constant 2-D weights the branches are
+    slice(x) -> matmul(., W_i) and the front-end passes turn each product into the MV order; otherwise the weights are
+    slices of one stacked tensor, transposed on the way, as in the reference's Switch Transformer graph."""
+    g = torch.Generator().manual_seed(seed)
+    c, join_in = {}, []
+    if constant_weights:
+        ops, inputs = [R.Op("aten::contiguous", [0], [1])], [0]
+        feeds = {0: torch.randn(n, d, generator=g).half()}
+    else:
+        ops, inputs = [R.Op("aten::contiguous", [0], [1])], [0, 5]
+        feeds = {0: (0.03 * torch.randn(n, d, d, generator=g)).half(), 5: torch.randn(1, d, generator=g).half()}
+    for i in range(n):
+        c[200 + i] = (0.1 * torch.randn(1, d, generator=g)).half()
+        if constant_weights:
+            c[100 + i] = (0.03 * torch.randn(d, d, generator=g)).half()
+            ops += [R.Op("aten::slice", [1], [10 + i], {"dim": 0, "start": i, "end": i + 1}),
+                    R.Op("aten::matmul", [10 + i, 100 + i], [20 + i])]
+        else:
+            ops += [R.Op("aten::slice", [1], [10 + i], {"dim": 0, "start": i, "end": i + 1}),
+                    R.Op("aten::transpose", [10 + i], [50 + i], {"dim0": -2, "dim1": -1}),
+                    R.Op("aten::matmul", [5, 50 + i], [20 + i])]
+        ops.append(R.Op("aten::add", [20 + i, 200 + i], [30 + i]))
+        join_in.append(30 + i)
+    ops.append(R.Op("prim::ListConstruct", join_in, [40]))
+    return R.Graph(ops, inputs, [40], c, next_id=300), feeds
+
+
+def test_multi_stream_pass_collects_the_sibling_products():
+    g, _ = attention_projection_graph()
+    R.apply_reference_passes(g)
+    R.lower_to_hot_path(g)
+    assert g.types().count("pimhip::gemv") == 4
+    R.multi_stream_execution(g)
+    # start, the four slices moved up behind it, ONE multi_stream op holding the four products, then the adds and the join
+    assert g.types() == ["aten::contiguous"] + ["aten::slice"] * 4 + ["multi_stream"] + ["aten::add"] * 4 + ["prim::ListConstruct"]
+    ms = g.ops[5]
+    assert [m.type for m in ms.attrs["layers"]] == ["pimhip::gemv"] * 4 and ms.outputs == [20, 21, 22, 23]
+    # the Switch Transformer shape of it: the products keep their type, their slices and transposes move up
+    g, _ = attention_projection_graph(constant_weights=False)
+    R.apply_reference_passes(g)
+    R.lower_to_hot_path(g)
+    R.multi_stream_execution(g)
+    assert g.types() == ["aten::contiguous"] + ["aten::slice", "aten::transpose"] * 4 + ["multi_stream"] + ["aten::add"] * 4 + ["prim::ListConstruct"]
+    assert [m.type for m in g.ops[9].attrs["layers"]] == ["aten::matmul"] * 4
+
+
+def test_multi_stream_pass_leaves_dependent_or_startless_products_alone():
+    # a chain (the second product consumes the first) joined with its own input: nothing to run side by side
+    c = {10: torch.randn(8, 8).half(), 11: torch.randn(8, 8).half()}
+    g = R.Graph([R.Op("aten::relu", [0], [1]), R.Op("aten::matmul", [1, 10], [2]), R.Op("aten::matmul", [2, 11], [3]),
+                 R.Op("prim::ListConstruct", [2, 3], [4])], [0], [4], c, 20)
+    before = g.types()
+    R.multi_stream_execution(g)
+    assert g.types() == before
+    # two products on two different graph inputs: no common start
+    g = R.Graph([R.Op("aten::matmul", [0, 10], [2]), R.Op("aten::matmul", [1, 11], [3]), R.Op("prim::ListConstruct", [2, 3], [4])],
+                [0, 1], [4], c, 20)
+    R.multi_stream_execution(g)
+    assert g.types() == ["aten::matmul", "aten::matmul", "prim::ListConstruct"]
+
+
+@pytest.mark.gpu
+def test_multi_stream_graph_matches_the_original_op_list(ops):
+    # stacked, sliced, transposed weights: x . W_i^T + b_i
+    g, feeds = attention_projection_graph(constant_weights=False)
+    want = [feeds[5].float() @ feeds[0][i].float().t() + g.constants[200 + i].float() for i in range(4)]
+    (plain,) = R.execute(g, feeds, DEV)
+    R.apply_reference_passes(g)
+    R.lower_to_hot_path(g)
+    R.multi_stream_execution(g)
+    assert "multi_stream" in g.types()
+    (outs,) = R.execute(g, feeds, DEV)
+    for o, p0, w in zip(outs, plain, want):
+        assert float((o.float().cpu().reshape(-1) - w.reshape(-1)).abs().max()) <= 4e-3
+        assert torch.equal(o.reshape(-1), p0.reshape(-1))
+    # constant 2-D weights: SwapMatmulInputs puts the constant first without transposing it
+    # (swap_matmul_inputs.cpp:74-78), so the rewritten graph computes (W_i . x^T)^T = x . W_i^T; the grouped launch must
+    # give what the reference's rewritten graph gives op by op
+    g, feeds = attention_projection_graph()
+    R.apply_reference_passes(g)
+    (ref,) = R.execute(g, feeds, DEV)
+    R.lower_to_hot_path(g)
+    R.multi_stream_execution(g)
+    (outs,) = R.execute(g, feeds, DEV)
+    x = feeds[0]
+    for i, (o, r) in enumerate(zip(outs, ref)):
+        w = x[i:i + 1].float() @ g.constants[100 + i].float().t() + g.constants[200 + i].float()
+        assert list(o.shape) == [1, 512] and float((o.float().cpu() - w).abs().max()) <= 4e-3
+        assert float((o.float() - r.float()).abs().max()) <= 2e-3
