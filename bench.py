@@ -257,6 +257,16 @@ def main():
             us = timed_us(vm_launch, 50)
             vm_times.append({"out": s_["n"], "in": s_["k"], "us": round(us, 2), "gbs": round(gemv_bytes(s_["n"], s_["k"]) / us / 1e3, 1)})
         other["gemv_vm_order"] = vm_times
+        # the 1024 x 1024 GEMV of the reference's own unit-test size class (2 MB: launch-bound), cold rotation over 64 copies
+        c1_pool = (0.02 * torch.randn(64, 1024, 1024, device=dev)).half()
+        c1_x, c1_b, c1_y = torch.randn(1024, device=dev).half(), torch.randn(1024, device=dev).half(), torch.empty(1024, dtype=torch.float16, device=dev)
+        c1_it = [0]
+
+        def c1_launch():
+            c1_it[0] += 1
+            lib.pimhip_execute_gemv(c1_y.data_ptr(), c1_x.data_ptr(), c1_pool[c1_it[0] % 64].data_ptr(), c1_b.data_ptr(), 1024, 1024, 0,
+                                    L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+        other["gemv_1024x1024_us"] = round(timed_us(c1_launch, 200), 3)
         # MoE FFN decode step (router 768 -> 8, then one expert 768 -> 3072 ReLU -> 768): three dependent launches on
         # resident (warm) weights, the expert fixed so that no host round trip for the argmax is inside the figure
         wr, w1, w2 = (0.02 * torch.randn(8, 768, device=dev)).half(), (0.02 * torch.randn(3072, 768, device=dev)).half(), \
