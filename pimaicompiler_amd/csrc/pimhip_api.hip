@@ -406,24 +406,43 @@ __global__ void fill_u32_kernel(unsigned int* p, size_t n, unsigned int v)
     if (i < n) p[i] = v;
 }
 
-int launch_input_projection(float* out, const half_t* x, const half_t* w, const float* bias, int64_t T, int64_t K,
-                            int64_t N, hipStream_t s)
+// out_p[T, N] = x[T, K] . w_p[N, K]^T + bias_p for p < count (1, or 2 for the two directions of a bidirectional layer).
+int launch_input_projection(int count, float* const* out, const half_t* x, const half_t* const* w, const float* const* bias,
+                            int64_t T, int64_t K, int64_t N, hipStream_t s)
 {
     if (T <= 0 || N <= 0) return PIMHIP_OK;
-    if (K % 8 != 0 || !aligned16(x) || !aligned16(w))
+    if (K % 8 != 0 || !aligned16(x))
         return fail(PIMHIP_ERR_UNSUPPORTED, "input projection needs in_w %% 8 == 0 (got %lld) and 16-byte aligned x and w", (long long)K);
     if (T > INT32_MAX || K > INT32_MAX || N > INT32_MAX) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "dimension above 2^31-1");
+    XprojProblems pr;
+    memset(&pr, 0, sizeof(pr));
+    for (int p = 0; p < count; ++p) {
+        if (!aligned16(w[p]))
+            return fail(PIMHIP_ERR_UNSUPPORTED, "input projection needs in_w %% 8 == 0 (got %lld) and 16-byte aligned x and w", (long long)K);
+        pr.w[p] = w[p];
+        pr.bias[p] = bias[p];
+        pr.out[p] = out[p];
+    }
     // 64 time steps per block row.  Measured on MI355X for T = 50, 200, 800 and K = 240, 1024, 2048 (N = 4096): 32-column
     // tiles are fastest as soon as there are two row blocks, 16-column tiles with one (more blocks than CUs either way).
     const unsigned row_blocks = (unsigned)((T + kXprojTile - 1) / kXprojTile);
     auto blocks = [&](int cols) { return (unsigned)(((N + cols - 1) / cols + 7) / 8 * 8) * row_blocks; };
-    if (row_blocks >= 2)
-        input_projection_f16_kernel<2><<<blocks(32), 256, 0, s>>>(x, w, bias, out, (int)T, (int)K, (int)N, (long)K, (long)K, (int)row_blocks);
-    else
-        input_projection_f16_kernel<1><<<blocks(16), 256, 0, s>>>(x, w, bias, out, (int)T, (int)K, (int)N, (long)K, (long)K, (int)row_blocks);
+    if (row_blocks >= 2) {
+        pr.blocks_per_problem = (int)blocks(32);
+        input_projection_f16_kernel<2><<<blocks(32) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, (long)K, (int)row_blocks);
+    } else {
+        pr.blocks_per_problem = (int)blocks(16);
+        input_projection_f16_kernel<1><<<blocks(16) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, (long)K, (int)row_blocks);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(PIMHIP_ERR_HIP, "input projection launch failed: %s", hipGetErrorString(e));
     return PIMHIP_OK;
+}
+
+int launch_input_projection(float* out, const half_t* x, const half_t* w, const float* bias, int64_t T, int64_t K,
+                            int64_t N, hipStream_t s)
+{
+    return launch_input_projection(1, &out, x, &w, &bias, T, K, N, s);
 }
 }  // namespace
 
@@ -776,8 +795,15 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                 ch.cn = cnp + (size_t)ci * H;
                 if (D == 2 || k == 0) {
                     float* xp = plan->xproj + (size_t)((D == 2) ? k : 0) * plan->max_seq_len * 4 * H;
-                    rc = launch_input_projection(xp, layer_in, c.w_ih, c.bsum, T, in_w, 4 * H, s);
-                    if (rc != PIMHIP_OK) return rc;
+                    if (k == 0) {
+                        // both directions of a bidirectional layer read the same x: one launch
+                        const PimHipLstmPlan::Cell& c2 = plan->cells[(D == 2) ? ci + 1 : ci];
+                        float* outs2[2] = {xp, xp + (size_t)plan->max_seq_len * 4 * H};
+                        const half_t* ws2[2] = {c.w_ih, c2.w_ih};
+                        const float* bs2[2] = {c.bsum, c2.bsum};
+                        rc = launch_input_projection(D, outs2, layer_in, ws2, bs2, T, in_w, 4 * H, s);
+                        if (rc != PIMHIP_OK) return rc;
+                    }
                     ch.xproj = xp;
                 } else {
                     ch.w_ih = c.w_ih;

@@ -6,7 +6,7 @@
 // receives out rows 4 * (l / 16) .. + 3 of column (l % 16).
 //
 // Grid (1-D): one block of 256 lanes per 16 * NT output columns and 64 time steps, 8 * ceil(column tiles / 8) * row
-// blocks in all.  Requirements checked by the launcher:
+// blocks per projection.  Requirements checked by the launcher:
 // K % 8 == 0, 16-byte aligned x and w, row pitches % 8 == 0.
 #pragma once
 
@@ -27,14 +27,25 @@ static constexpr int kXprojKSplit = 4;   // wavefronts per block = MFMA K steps 
 static constexpr int kXprojSlab = 32 * kXprojKSplit;  // K values per slab (128)
 static constexpr int kXprojPitch = kXprojSlab + 8;    // LDS row pitch in halves (272 bytes)
 
+// Up to two projections of the same x in one launch (the two directions of a bidirectional layer): blocks
+// [p * blocks_per_problem, (p + 1) * blocks_per_problem) work on weight / bias / output set p.
+struct XprojProblems {
+    const half_t* w[2];
+    const float* bias[2];
+    float* out[2];
+    int blocks_per_problem;
+};
+
 // NT: column tiles of 16 per block (2, or 1 when a single row block would leave CUs without work).
 template <int NT>
-__global__ __launch_bounds__(256) void input_projection_f16_kernel(const half_t* __restrict__ x,
-                                                                  const half_t* __restrict__ w,
-                                                                  const float* __restrict__ bias,
-                                                                  float* __restrict__ out, int T, int K, int N, long ldx,
-                                                                  long ldw, int row_blocks)
+__global__ __launch_bounds__(256) void input_projection_f16_kernel(const half_t* __restrict__ x, XprojProblems problems,
+                                                                  int T, int K, int N, long ldx, long ldw, int row_blocks)
 {
+    const int problem = blockIdx.x >= (unsigned)problems.blocks_per_problem ? 1 : 0;
+    const int block = blockIdx.x - problem * problems.blocks_per_problem;
+    const half_t* __restrict__ w = problems.w[problem];
+    const float* __restrict__ bias = problems.bias[problem];
+    float* __restrict__ out = problems.out[problem];
     constexpr int ROWS = kXprojTile + 16 * NT;            // LDS rows per slab: x rows first, then w rows
     constexpr int CHUNKS = ROWS * (kXprojSlab / 8);       // 16-byte pieces per slab
     constexpr int PER_LANE = CHUNKS / 256;                // 5, 6 or 8
@@ -52,8 +63,8 @@ __global__ __launch_bounds__(256) void input_projection_f16_kernel(const half_t*
     // Workgroups go to the eight XCDs round-robin by linear id, and each XCD has its own L2.  All row blocks of a column
     // tile are therefore given ids that are equal modulo 8: the tile's slice of w is then pulled into one L2 once and
     // shared by its row blocks, instead of crossing the fabric once per row block and XCD.
-    const int xcd = blockIdx.x & 7;
-    const int local = blockIdx.x >> 3;
+    const int xcd = block & 7;
+    const int local = block >> 3;
     const int col_tile = (local / row_blocks) * 8 + xcd;
     if (col_tile * (16 * NT) >= N) return;  // whole block, before any barrier
     const int n_base = col_tile * (16 * NT);
