@@ -177,6 +177,17 @@ int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);
 int pimhip_input_projection(void* out, const void* x, const void* w, const void* bias, int64_t seq_len,
                             int64_t in_w, int64_t n_out, void* stream);
 
+/* The same product with the weight re-laid out once in the matrix cores' fragment order, which is what an LSTM plan
+ * does with the w_ih of its batched layers at creation (it takes the place of the MIOpen weight packing,
+ * model_builder.cpp:226-319): pimhip_projection_packed_bytes gives the size of the packed copy,
+ * pimhip_pack_projection_weight fills it from w[n_out, in_w] (row-major, dense), and
+ * pimhip_input_projection_packed computes out[T, n_out] from it; results equal pimhip_input_projection's bit for bit.
+ * They have no counterpart in the reference; they are exported for callers that batch the projection themselves. */
+int pimhip_projection_packed_bytes(int64_t in_w, int64_t n_out, uint64_t* bytes);
+int pimhip_pack_projection_weight(void* packed, const void* w, int64_t in_w, int64_t n_out, void* stream);
+int pimhip_input_projection_packed(void* out, const void* x, const void* packed, const void* bias, int64_t seq_len,
+                                   int64_t in_w, int64_t n_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

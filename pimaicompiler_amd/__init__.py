@@ -22,5 +22,7 @@ from .ops import (  # noqa: F401
     aten_lstm2,
     execute_gemv_group,
     input_projection,
+    input_projection_packed,
+    pack_projection_weight,
     LstmPlan,
 )

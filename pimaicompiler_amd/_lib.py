@@ -43,6 +43,11 @@ SIGNATURES = {
     "pimhip_lstm_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "pimhip_input_projection": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
+    "pimhip_projection_packed_bytes": (ctypes.c_int, [ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_uint64)]),
+    "pimhip_pack_projection_weight": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                                     ctypes.c_void_p]),
+    "pimhip_input_projection_packed": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                      ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
 }
 
 # Status codes and enums of include/pimhip.h.

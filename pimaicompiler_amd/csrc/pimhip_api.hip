@@ -444,6 +444,32 @@ int launch_input_projection(float* out, const half_t* x, const half_t* w, const 
 {
     return launch_input_projection(1, &out, x, &w, &bias, T, K, N, s);
 }
+
+// The same with weights in fragment order (pack_w_fragments_kernel); N, K checked by the caller (plan creation).
+int launch_input_projection_packed(int count, float* const* out, const half_t* x, const half_t* const* wp, const float* const* bias,
+                                   int64_t T, int64_t K, int64_t N, int ksteps, hipStream_t s)
+{
+    if (T <= 0 || N <= 0) return PIMHIP_OK;
+    XprojPackedProblems pr;
+    memset(&pr, 0, sizeof(pr));
+    for (int p = 0; p < count; ++p) {
+        pr.wp[p] = wp[p];
+        pr.bias[p] = bias[p];
+        pr.out[p] = out[p];
+    }
+    const unsigned row_blocks = (unsigned)((T + kXprojTile - 1) / kXprojTile);
+    auto blocks = [&](int cols) { return (unsigned)(((N + cols - 1) / cols + 7) / 8 * 8) * row_blocks; };
+    if (row_blocks >= 2) {
+        pr.blocks_per_problem = (int)blocks(32);
+        input_projection_packed_f16_kernel<2><<<blocks(32) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+    } else {
+        pr.blocks_per_problem = (int)blocks(16);
+        input_projection_packed_f16_kernel<1><<<blocks(16) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(PIMHIP_ERR_HIP, "input projection launch failed: %s", hipGetErrorString(e));
+    return PIMHIP_OK;
+}
 }  // namespace
 
 extern "C" int pimhip_input_projection(void* out, const void* x, const void* w, const void* bias, int64_t seq_len,
@@ -456,6 +482,63 @@ extern "C" int pimhip_input_projection(void* out, const void* x, const void* w, 
     if (seq_len < 0 || in_w < 0 || n_out < 0) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "negative dimension");
     return launch_input_projection((float*)out, (const half_t*)x, (const half_t*)w, (const float*)bias, seq_len, in_w,
                                    n_out, static_cast<hipStream_t>(stream));
+}
+
+namespace
+{
+void packed_geometry(int64_t in_w, int64_t n_out, int* ntiles, int* ksteps)
+{
+    *ksteps = (int)((in_w + kXprojSlab - 1) / kXprojSlab * kXprojSlab / 32);
+    *ntiles = (int)((n_out + 63) / 64 * 4);
+}
+}  // namespace
+
+extern "C" int pimhip_projection_packed_bytes(int64_t in_w, int64_t n_out, uint64_t* bytes)
+{
+    if (!bytes) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "bytes is null");
+    if (in_w < 1 || n_out < 1 || in_w > INT32_MAX || n_out > INT32_MAX) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "in_w=%lld n_out=%lld out of range", (long long)in_w, (long long)n_out);
+    int ntiles = 0, ksteps = 0;
+    packed_geometry(in_w, n_out, &ntiles, &ksteps);
+    *bytes = (uint64_t)ntiles * (uint64_t)ksteps * 64u * 16u;
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_pack_projection_weight(void* packed, const void* w, int64_t in_w, int64_t n_out, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!packed || !w) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "packed and w must be non-null");
+    if (in_w < 1 || n_out < 1 || in_w > INT32_MAX || n_out > INT32_MAX) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "in_w=%lld n_out=%lld out of range", (long long)in_w, (long long)n_out);
+    if (in_w % 8 != 0 || !aligned16(w) || !aligned16(packed))
+        return fail(PIMHIP_ERR_UNSUPPORTED, "packing needs in_w %% 8 == 0 (got %lld) and 16-byte aligned pointers", (long long)in_w);
+    int ntiles = 0, ksteps = 0;
+    packed_geometry(in_w, n_out, &ntiles, &ksteps);
+    const size_t chunks = (size_t)ntiles * ksteps * 64;
+    pack_w_fragments_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        (const half_t*)w, (half_t*)packed, (int)n_out, (int)in_w, (long)in_w, ntiles, ksteps);
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_input_projection_packed(void* out, const void* x, const void* packed, const void* bias, int64_t seq_len,
+                                              int64_t in_w, int64_t n_out, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (seq_len < 0 || in_w < 1 || n_out < 1 || seq_len > INT32_MAX || in_w > INT32_MAX || n_out > INT32_MAX)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "seq_len=%lld in_w=%lld n_out=%lld out of range", (long long)seq_len, (long long)in_w, (long long)n_out);
+    if (seq_len == 0) return PIMHIP_OK;
+    if (!out || !x || !packed) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "out, x and packed must be non-null");
+    if (in_w % 8 != 0 || !aligned16(x) || !aligned16(packed))
+        return fail(PIMHIP_ERR_UNSUPPORTED, "input projection needs in_w %% 8 == 0 (got %lld) and 16-byte aligned x and packed", (long long)in_w);
+    int ntiles = 0, ksteps = 0;
+    packed_geometry(in_w, n_out, &ntiles, &ksteps);
+    float* outs[1] = {(float*)out};
+    const half_t* wps[1] = {(const half_t*)packed};
+    const float* bs[1] = {(const float*)bias};
+    return launch_input_projection_packed(1, outs, (const half_t*)x, wps, bs, seq_len, in_w, n_out, ksteps, static_cast<hipStream_t>(stream));
 }
 
 // ================================================================================================
@@ -483,11 +566,14 @@ struct PimHipLstmPlan {
         const half_t* b_ih = nullptr;
         const half_t* b_hh = nullptr;
         float* bsum = nullptr;  // [4H] fp32, b_ih + b_hh (zeros when has_biases == 0)
+        half_t* w_ih_packed = nullptr;  // w_ih in MFMA fragment order (cells whose projection runs as a batch), else null
+        int ksteps = 0;                 // 32-wide K steps of the packed matrix
         int64_t in_w = 0;
     };
     std::vector<Cell> cells;          // index = layer * num_dirs + dir
 
     float* bsum_all = nullptr;        // backing store of every Cell::bsum
+    std::vector<half_t*> packed;      // every Cell::w_ih_packed allocation
     float* xproj = nullptr;           // [num_dirs][max_seq_len][4H] fp32
     half_t* ybuf[2] = {nullptr, nullptr};  // inter-layer sequences [max_seq_len][num_dirs * H]
     float* c_state = nullptr;         // [num_dirs][H] fp32, per-step kernel's cell state
@@ -510,6 +596,7 @@ int destroy_plan_locked(PimHipLstmPlan* plan)
     hipSetDevice(plan->device);
     hipDeviceSynchronize();
     if (plan->bsum_all) hipFree(plan->bsum_all);
+    for (half_t* q : plan->packed) hipFree(q);
     if (plan->xproj) hipFree(plan->xproj);
     if (plan->ybuf[0]) hipFree(plan->ybuf[0]);
     if (plan->ybuf[1]) hipFree(plan->ybuf[1]);
@@ -614,6 +701,22 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
             if (!aligned16(c.w_ih) || !aligned16(c.w_hh))
                 return cleanup_fail(fail(PIMHIP_ERR_UNSUPPORTED, "weights of layer %d direction %d are not 16-byte aligned", l, d));
             lstm_bias_sum_kernel<<<(unsigned)((4 * H + 255) / 256), 256, 0, s>>>(c.b_ih, c.b_hh, c.bsum, (int)(4 * H));
+        }
+    }
+    PLAN_HIP_CHECK(hipGetLastError());
+    // Cells whose input projection runs as a batch over the sequence (every layer of a bidirectional stack, the first
+    // layer of every wavefront group of a unidirectional one) get a copy of w_ih in MFMA fragment order.
+    for (int l = 0; l < num_layers; ++l) {
+        if (D == 1 && l % plan->max_wavefront != 0) continue;
+        for (int d = 0; d < D; ++d) {
+            PimHipLstmPlan::Cell& c = plan->cells[(size_t)l * D + d];
+            int ntiles = 0;
+            packed_geometry(c.in_w, 4 * H, &ntiles, &c.ksteps);
+            const size_t chunks = (size_t)ntiles * c.ksteps * 64;
+            PLAN_HIP_CHECK(hipMalloc(&c.w_ih_packed, chunks * 16));
+            plan->packed.push_back(c.w_ih_packed);
+            pack_w_fragments_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, s>>>(c.w_ih, c.w_ih_packed, (int)(4 * H), (int)c.in_w,
+                                                                                      (long)c.in_w, ntiles, c.ksteps);
         }
     }
     PLAN_HIP_CHECK(hipGetLastError());
@@ -799,9 +902,14 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                         // both directions of a bidirectional layer read the same x: one launch
                         const PimHipLstmPlan::Cell& c2 = plan->cells[(D == 2) ? ci + 1 : ci];
                         float* outs2[2] = {xp, xp + (size_t)plan->max_seq_len * 4 * H};
-                        const half_t* ws2[2] = {c.w_ih, c2.w_ih};
                         const float* bs2[2] = {c.bsum, c2.bsum};
-                        rc = launch_input_projection(D, outs2, layer_in, ws2, bs2, T, in_w, 4 * H, s);
+                        if (c.w_ih_packed && c2.w_ih_packed) {
+                            const half_t* ws2[2] = {c.w_ih_packed, c2.w_ih_packed};
+                            rc = launch_input_projection_packed(D, outs2, layer_in, ws2, bs2, T, in_w, 4 * H, c.ksteps, s);
+                        } else {
+                            const half_t* ws2[2] = {c.w_ih, c2.w_ih};
+                            rc = launch_input_projection(D, outs2, layer_in, ws2, bs2, T, in_w, 4 * H, s);
+                        }
                         if (rc != PIMHIP_OK) return rc;
                     }
                     ch.xproj = xp;

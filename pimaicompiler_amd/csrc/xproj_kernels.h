@@ -164,6 +164,163 @@ __global__ __launch_bounds__(256) void input_projection_f16_kernel(const half_t*
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same product with w re-laid out once (at plan creation) in MFMA fragment order, so that w never passes through
+// LDS: a wavefront's B fragment of a (16-row tile j, 32-wide K step s) is the 1 KB at ((j * ksteps + s) * 64 + lane) * 8
+// halves, lane = kq * 16 + r16 holding w[16 j + r16][32 s + 8 kq .. + 7]; rows past N and columns past K are zero;
+// ksteps = padded K / 32 with K padded to a multiple of kXprojSlab.  Only x goes through LDS, which halves the LDS
+// traffic per MFMA (the bound of the kernel above).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pack_w_fragments_kernel(const half_t* __restrict__ w, half_t* __restrict__ wp, int N, int K,
+                                                               long ldw, int ntiles, int ksteps)
+{
+    const long chunk = (long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte piece of the packed matrix
+    const long total = (long)ntiles * ksteps * 64;
+    if (chunk >= total) return;
+    const int lane = (int)(chunk & 63);
+    const long frag = chunk >> 6;
+    const int s = (int)(frag % ksteps);
+    const int j = (int)(frag / ksteps);
+    const int row = j * 16 + (lane & 15);
+    const int k = s * 32 + (lane >> 4) * 8;
+    half8_t v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (half_t)0.0f;
+    if (row < N && k < K) v = *reinterpret_cast<const half8_t*>(w + (long)row * ldw + k);  // K % 8 == 0
+    reinterpret_cast<half8_t*>(wp)[chunk] = v;
+}
+
+struct XprojPackedProblems {
+    const half_t* wp[2];
+    const float* bias[2];
+    float* out[2];
+    int blocks_per_problem;
+};
+
+template <int NT>
+__global__ __launch_bounds__(256) void input_projection_packed_f16_kernel(const half_t* __restrict__ x, XprojPackedProblems problems,
+                                                                         int T, int K, int N, long ldx, int ksteps,
+                                                                         int row_blocks)
+{
+    constexpr int CHUNKS = kXprojTile * (kXprojSlab / 8);  // 16-byte pieces of an x slab: 1024
+    constexpr int PER_LANE = CHUNKS / 256;                 // 4
+    constexpr int SLAB_BYTES = kXprojTile * kXprojPitch * 2;
+    constexpr int RED_BYTES = kXprojKSplit * 4 * NT * 64 * 16;
+    constexpr int LDS_BYTES = 2 * SLAB_BYTES > RED_BYTES ? 2 * SLAB_BYTES : RED_BYTES;
+    __shared__ __align__(16) unsigned char lds[LDS_BYTES];
+
+    const int problem = blockIdx.x >= (unsigned)problems.blocks_per_problem ? 1 : 0;
+    const int block = blockIdx.x - problem * problems.blocks_per_problem;
+    const half_t* __restrict__ wp = problems.wp[problem];
+    const float* __restrict__ bias = problems.bias[problem];
+    float* __restrict__ out = problems.out[problem];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int ks = tid >> 6;
+    const int r16 = lane & 15;
+    const int kq = lane >> 4;
+    const int xcd = block & 7;  // column tiles pinned to one XCD, as above
+    const int local = block >> 3;
+    const int col_tile = (local / row_blocks) * 8 + xcd;
+    if (col_tile * (16 * NT) >= N) return;
+    const int n_base = col_tile * (16 * NT);
+    const int t_base = (local % row_blocks) * kXprojTile;
+
+    const half_t* src[PER_LANE];
+    int dst[PER_LANE];
+    const int kcol = (tid & 15) * 8;
+#pragma unroll
+    for (int i = 0; i < PER_LANE; ++i) {
+        const int row = (tid >> 4) + 16 * i;
+        src[i] = x + (long)min(t_base + row, T - 1) * ldx;
+        dst[i] = row * kXprojPitch + kcol;
+    }
+    // This wavefront's B fragments: tile (col_tile * NT + n), K step 4 * slab + ks.
+    const half8_t* wfrag[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) wfrag[n] = reinterpret_cast<const half8_t*>(wp) + ((long)(col_tile * NT + n) * ksteps + ks) * 64 + lane;
+
+    half8_t zero;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) zero[e] = (half_t)0.0f;
+    float4_t acc[4][NT];
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int slabs = ksteps / kXprojKSplit;
+    half8_t stage[PER_LANE];
+    half8_t b_next[NT];
+    auto fetch = [&](int slab) {
+        const int k = slab * kXprojSlab + kcol;
+        const bool ok = k < K;
+        const int kc = ok ? k : 0;
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) {
+            const half8_t v = *reinterpret_cast<const half8_t*>(src[i] + kc);
+            stage[i] = ok ? v : zero;
+        }
+#pragma unroll
+        for (int n = 0; n < NT; ++n) b_next[n] = wfrag[n][(long)slab * kXprojKSplit * 64];
+    };
+    auto deposit = [&](int buf) {
+        half_t* base = reinterpret_cast<half_t*>(lds + buf * SLAB_BYTES);
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) *reinterpret_cast<half8_t*>(base + dst[i]) = stage[i];
+    };
+
+    fetch(0);
+    deposit(0);
+    __syncthreads();
+    for (int s = 0; s < slabs; ++s) {
+        half8_t b[NT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n) b[n] = b_next[n];
+        if (s + 1 < slabs) fetch(s + 1);
+        const half_t* base = reinterpret_cast<const half_t*>(lds + (s & 1) * SLAB_BYTES) + ks * 32 + kq * 8;
+        half8_t a[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) a[m] = *reinterpret_cast<const half8_t*>(base + (m * 16 + r16) * kXprojPitch);
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[m], b[n], acc[m][n], 0, 0, 0);
+        if (s + 1 < slabs) deposit((s + 1) & 1);
+        __syncthreads();
+    }
+
+    float(*red)[4 * NT][64][4] = reinterpret_cast<float(*)[4 * NT][64][4]>(lds);
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) *reinterpret_cast<float4_t*>(&red[ks][m * NT + n][lane][0]) = acc[m][n];
+    __syncthreads();
+    const int m = ks;
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+        float4_t v = *reinterpret_cast<const float4_t*>(&red[0][m * NT + n][lane][0]);
+#pragma unroll
+        for (int q = 1; q < kXprojKSplit; ++q) {
+            const float4_t p = *reinterpret_cast<const float4_t*>(&red[q][m * NT + n][lane][0]);
+            v[0] += p[0];
+            v[1] += p[1];
+            v[2] += p[2];
+            v[3] += p[3];
+        }
+        const int col = n_base + n * 16 + r16;
+        if (col < N) {
+            const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int t = t_base + m * 16 + kq * 4 + i;
+                if (t < T) out[(long)t * N + col] = v[i] + bv;
+            }
+        }
+    }
+}
+
 // bsum[i] = b_ih[i] + b_hh[i] in fp32 (either may be null, meaning zero).
 __global__ void lstm_bias_sum_kernel(const half_t* __restrict__ b_ih, const half_t* __restrict__ b_hh,
                                      float* __restrict__ bsum, int n)

@@ -414,6 +414,38 @@ def input_projection(x, w, bias=None, stream=None):
     return out
 
 
+def pack_projection_weight(w, stream=None):
+    """w[N, K] in the matrix cores' fragment order (one-time); what an LSTM plan does with its batched layers' w_ih."""
+    lib = L.load()
+    _require_half_cuda(w)
+    _ensure_init(w)
+    w = w.contiguous()
+    nbytes = ctypes.c_uint64()
+    _check(lib.pimhip_projection_packed_bytes(w.size(1), w.size(0), ctypes.byref(nbytes)))
+    packed = torch.empty(nbytes.value // 2, dtype=torch.float16, device=w.device)
+    _check(lib.pimhip_pack_projection_weight(packed.data_ptr(), w.data_ptr(), w.size(1), w.size(0), _stream_handle(stream)))
+    return packed
+
+
+def input_projection_packed(x, packed, n_out, bias=None, stream=None):
+    """input_projection with a weight from pack_projection_weight; the same bits, less LDS traffic."""
+    lib = L.load()
+    _require_half_cuda(x, packed)
+    x = x.contiguous()
+    T, K = x.shape
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_cuda or bias.numel() != n_out):
+        raise NNRuntimeException("bias must be an fp32 GPU tensor of N elements")
+    nbytes = ctypes.c_uint64()
+    _check(lib.pimhip_projection_packed_bytes(K, n_out, ctypes.byref(nbytes)))
+    if packed.numel() * 2 != nbytes.value:
+        raise NNRuntimeException("`packed` does not have the size of a packed [n_out, in_w] weight")
+    out = torch.empty((T, n_out), dtype=torch.float32, device=x.device)
+    _check(lib.pimhip_input_projection_packed(out.data_ptr(), x.data_ptr(), packed.data_ptr(),
+                                              bias.contiguous().data_ptr() if bias is not None else None, T, K, n_out,
+                                              _stream_handle(stream)))
+    return out
+
+
 # ---------------------------------------------------------------------------------------------------
 # LSTM
 # ---------------------------------------------------------------------------------------------------

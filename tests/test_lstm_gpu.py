@@ -310,3 +310,7 @@ def test_input_projection_matches_fp32_matmul(ops, T, K, N):
     assert maxabs(out, want) <= 1e-4 * max(1.0, float(want.abs().max()))   # fp32 accumulation of exact fp16 products
     out = ops.input_projection(x.to(DEV), w.to(DEV))
     assert maxabs(out, want - b) <= 1e-4 * max(1.0, float(want.abs().max()))
+    # the weight in fragment order (what a plan keeps for its batched layers): the same bits
+    packed = ops.pack_projection_weight(w.to(DEV))
+    assert torch.equal(ops.input_projection_packed(x.to(DEV), packed, N), out)
+    assert torch.equal(ops.input_projection_packed(x.to(DEV), packed, N, b.to(DEV)), ops.input_projection(x.to(DEV), w.to(DEV), b.to(DEV)))
