@@ -181,7 +181,8 @@ int pimhip_input_projection(void* out, const void* x, const void* w, const void*
  * does with the w_ih of its batched layers at creation (it takes the place of the MIOpen weight packing,
  * model_builder.cpp:226-319): pimhip_projection_packed_bytes gives the size of the packed copy,
  * pimhip_pack_projection_weight fills it from w[n_out, in_w] (row-major, dense), and
- * pimhip_input_projection_packed computes out[T, n_out] from it; results equal pimhip_input_projection's bit for bit.
+ * pimhip_input_projection_packed computes out[T, n_out] from it (the same exact products as pimhip_input_projection,
+ * summed in a fixed order that may differ from its).
  * They have no counterpart in the reference; they are exported for callers that batch the projection themselves. */
 int pimhip_projection_packed_bytes(int64_t in_w, int64_t n_out, uint64_t* bytes);
 int pimhip_pack_projection_weight(void* packed, const void* w, int64_t in_w, int64_t n_out, void* stream);

@@ -459,12 +459,17 @@ int launch_input_projection_packed(int count, float* const* out, const half_t* x
     }
     const unsigned row_blocks = (unsigned)((T + kXprojTile - 1) / kXprojTile);
     auto blocks = [&](int cols) { return (unsigned)(((N + cols - 1) / cols + 7) / 8 * 8) * row_blocks; };
+    // Measured on MI355X (T = 50, 200, 800; K = 240, 1024, 2048; N = 4096): with one row block 16-column tiles and
+    // eight wavefronts splitting K; with more, 32-column tiles, and eight wavefronts only for long rows and few row blocks.
     if (row_blocks >= 2) {
         pr.blocks_per_problem = (int)blocks(32);
-        input_projection_packed_f16_kernel<2><<<blocks(32) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+        if (row_blocks <= 4 && K >= 2048)
+            input_projection_packed_f16_kernel<2, 8><<<blocks(32) * count, 512, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+        else
+            input_projection_packed_f16_kernel<2, 4><<<blocks(32) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
     } else {
         pr.blocks_per_problem = (int)blocks(16);
-        input_projection_packed_f16_kernel<1><<<blocks(16) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+        input_projection_packed_f16_kernel<1, 8><<<blocks(16) * count, 512, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(PIMHIP_ERR_HIP, "input projection launch failed: %s", hipGetErrorString(e));

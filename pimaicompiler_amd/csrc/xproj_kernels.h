@@ -197,15 +197,19 @@ struct XprojPackedProblems {
     int blocks_per_problem;
 };
 
-template <int NT>
-__global__ __launch_bounds__(256) void input_projection_packed_f16_kernel(const half_t* __restrict__ x, XprojPackedProblems problems,
+// KS wavefronts per block, one 32-wide K step of a (32 * KS)-wide slab each.
+template <int NT, int KS = kXprojKSplit>
+__global__ __launch_bounds__(64 * KS) void input_projection_packed_f16_kernel(const half_t* __restrict__ x, XprojPackedProblems problems,
                                                                          int T, int K, int N, long ldx, int ksteps,
                                                                          int row_blocks)
 {
-    constexpr int CHUNKS = kXprojTile * (kXprojSlab / 8);  // 16-byte pieces of an x slab: 1024
-    constexpr int PER_LANE = CHUNKS / 256;                 // 4
-    constexpr int SLAB_BYTES = kXprojTile * kXprojPitch * 2;
-    constexpr int RED_BYTES = kXprojKSplit * 4 * NT * 64 * 16;
+    constexpr int SLAB = 32 * KS;                          // K values per slab
+    constexpr int PITCH = SLAB + 8;                        // LDS row pitch in halves
+    constexpr int CPR = SLAB / 8;                          // 16-byte pieces per x row and slab
+    constexpr int CHUNKS = kXprojTile * CPR;               // 16-byte pieces of an x slab
+    constexpr int PER_LANE = CHUNKS / (64 * KS);           // 4
+    constexpr int SLAB_BYTES = kXprojTile * PITCH * 2;
+    constexpr int RED_BYTES = KS * 4 * NT * 64 * 16;
     constexpr int LDS_BYTES = 2 * SLAB_BYTES > RED_BYTES ? 2 * SLAB_BYTES : RED_BYTES;
     __shared__ __align__(16) unsigned char lds[LDS_BYTES];
 
@@ -229,12 +233,12 @@ __global__ __launch_bounds__(256) void input_projection_packed_f16_kernel(const 
 
     const half_t* src[PER_LANE];
     int dst[PER_LANE];
-    const int kcol = (tid & 15) * 8;
+    const int kcol = (tid % CPR) * 8;
 #pragma unroll
     for (int i = 0; i < PER_LANE; ++i) {
-        const int row = (tid >> 4) + 16 * i;
+        const int row = tid / CPR + (64 * KS / CPR) * i;
         src[i] = x + (long)min(t_base + row, T - 1) * ldx;
-        dst[i] = row * kXprojPitch + kcol;
+        dst[i] = row * PITCH + kcol;
     }
     // This wavefront's B fragments: tile (col_tile * NT + n), K step 4 * slab + ks.
     const half8_t* wfrag[NT];
@@ -250,11 +254,11 @@ __global__ __launch_bounds__(256) void input_projection_packed_f16_kernel(const 
 #pragma unroll
         for (int n = 0; n < NT; ++n) acc[m][n] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const int slabs = ksteps / kXprojKSplit;
+    const int slabs = (ksteps + KS - 1) / KS;
     half8_t stage[PER_LANE];
     half8_t b_next[NT];
     auto fetch = [&](int slab) {
-        const int k = slab * kXprojSlab + kcol;
+        const int k = slab * SLAB + kcol;
         const bool ok = k < K;
         const int kc = ok ? k : 0;
 #pragma unroll
@@ -263,7 +267,7 @@ __global__ __launch_bounds__(256) void input_projection_packed_f16_kernel(const 
             stage[i] = ok ? v : zero;
         }
 #pragma unroll
-        for (int n = 0; n < NT; ++n) b_next[n] = wfrag[n][(long)slab * kXprojKSplit * 64];
+        for (int n = 0; n < NT; ++n) b_next[n] = (slab * KS + ks < ksteps) ? wfrag[n][(long)slab * KS * 64] : zero;
     };
     auto deposit = [&](int buf) {
         half_t* base = reinterpret_cast<half_t*>(lds + buf * SLAB_BYTES);
@@ -282,7 +286,7 @@ __global__ __launch_bounds__(256) void input_projection_packed_f16_kernel(const 
         const half_t* base = reinterpret_cast<const half_t*>(lds + (s & 1) * SLAB_BYTES) + ks * 32 + kq * 8;
         half8_t a[4];
 #pragma unroll
-        for (int m = 0; m < 4; ++m) a[m] = *reinterpret_cast<const half8_t*>(base + (m * 16 + r16) * kXprojPitch);
+        for (int m = 0; m < 4; ++m) a[m] = *reinterpret_cast<const half8_t*>(base + (m * 16 + r16) * PITCH);
 #pragma unroll
         for (int m = 0; m < 4; ++m)
 #pragma unroll
@@ -297,12 +301,13 @@ __global__ __launch_bounds__(256) void input_projection_packed_f16_kernel(const 
 #pragma unroll
         for (int n = 0; n < NT; ++n) *reinterpret_cast<float4_t*>(&red[ks][m * NT + n][lane][0]) = acc[m][n];
     __syncthreads();
+    if (ks >= 4) return;  // four row tiles, finished by the first four wavefronts
     const int m = ks;
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
         float4_t v = *reinterpret_cast<const float4_t*>(&red[0][m * NT + n][lane][0]);
 #pragma unroll
-        for (int q = 1; q < kXprojKSplit; ++q) {
+        for (int q = 1; q < KS; ++q) {
             const float4_t p = *reinterpret_cast<const float4_t*>(&red[q][m * NT + n][lane][0]);
             v[0] += p[0];
             v[1] += p[1];

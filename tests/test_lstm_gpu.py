@@ -310,7 +310,11 @@ def test_input_projection_matches_fp32_matmul(ops, T, K, N):
     assert maxabs(out, want) <= 1e-4 * max(1.0, float(want.abs().max()))   # fp32 accumulation of exact fp16 products
     out = ops.input_projection(x.to(DEV), w.to(DEV))
     assert maxabs(out, want - b) <= 1e-4 * max(1.0, float(want.abs().max()))
-    # the weight in fragment order (what a plan keeps for its batched layers): the same bits
+    # the weight in fragment order (what a plan keeps for its batched layers): the same products, summed in the same
+    # or (with eight wavefronts per block) another fixed order
     packed = ops.pack_projection_weight(w.to(DEV))
-    assert torch.equal(ops.input_projection_packed(x.to(DEV), packed, N), out)
-    assert torch.equal(ops.input_projection_packed(x.to(DEV), packed, N, b.to(DEV)), ops.input_projection(x.to(DEV), w.to(DEV), b.to(DEV)))
+    tol = 1e-5 * max(1.0, float(want.abs().max()))
+    assert maxabs(ops.input_projection_packed(x.to(DEV), packed, N), out.cpu()) <= tol
+    got = ops.input_projection_packed(x.to(DEV), packed, N, b.to(DEV))
+    assert maxabs(got, want) <= 1e-4 * max(1.0, float(want.abs().max()))
+    assert torch.equal(got, ops.input_projection_packed(x.to(DEV), packed, N, b.to(DEV)))
