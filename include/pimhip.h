@@ -137,8 +137,9 @@ typedef struct PimHipLstmPlan PimHipLstmPlan;
  *   params: host array of n_params device pointers in LibTorch order, per layer then per direction
  *           (w_ih [4H, I_l], w_hh [4H, H], then b_ih [4H], b_hh [4H] when has_biases), gate order
  *           (i, f, g, o); I_0 = input_size, I_l = num_directions * H for l > 0.
- * The plan keeps the caller's weight pointers (they must outlive the plan), pre-adds b_ih + b_hh, and
- * owns the internal buffers for up to max_seq_len steps.  Runs on `stream` and synchronises it. */
+ * The plan keeps the caller's weight pointers (they must outlive the plan), pre-adds b_ih + b_hh, copies the w_ih of
+ * the layers whose input projection runs as a batch into the matrix cores' fragment order (one more w_ih of memory
+ * for those layers), and owns the internal buffers for up to max_seq_len steps.  Runs on `stream` and synchronises it. */
 int pimhip_lstm_plan_create(PimHipLstmPlan** plan, const void* const* params, int n_params, int has_biases,
                             int num_layers, int bidirectional, int64_t input_size, int64_t hidden_size,
                             int64_t max_seq_len, void* stream);
