@@ -248,6 +248,16 @@ def multi_stream_execution(g: Graph, max_search_level: int = 10):
     return g
 
 
+def _as_row_major_weight(t):
+    """For a [..1.., in, out] tensor that is a transposed view of a dense row-major [out, in] matrix: that matrix."""
+    if t.dim() < 2 or any(d != 1 for d in t.shape[:-2]) or t.dtype != torch.float16:
+        return None
+    m = t.reshape(t.shape[-2:]) if t.dim() == 2 else t[(0,) * (t.dim() - 2)]
+    if m.stride(0) == 1 and m.stride(1) == m.size(0) and m.size(0) % 8 == 0 and m.data_ptr() % 16 == 0:
+        return m.t()
+    return None
+
+
 # ---- execution through the operator layer ----------------------------------------------------------------------------
 def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0"):
     """Runs the op list with pimaicompiler_amd.ops; returns the graph outputs.  Constants are moved to `device`."""
@@ -274,6 +284,18 @@ def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0"):
                                               [m.attrs["act_type"] for m in subs])
                 for m, x, o in zip(subs, xs, outs):
                     env[m.outputs[0]] = o.view(list(x.shape[:-1]) + [o.numel()])
+            elif all(m.type == "aten::matmul" and _as_row_major_weight(env[m.inputs[1]]) is not None and
+                     env[m.inputs[0]].numel() == env[m.inputs[1]].size(-2) for m in subs):
+                # x . T(W_i) with W_i a dense [out, in] slice (the Switch Transformer wiring): the transposed view is the
+                # MV order on the slice's own bytes, so these siblings also go out as one grouped launch.
+                xs = [env[m.inputs[0]] for m in subs]
+                ws = [_as_row_major_weight(env[m.inputs[1]]) for m in subs]
+                outs = ops.execute_gemv_group(xs, ws)
+                for m, x, o in zip(subs, xs, outs):
+                    other = env[m.inputs[1]]
+                    shape = list(other.shape) if other.dim() > x.dim() else list(x.shape)
+                    shape[-1], shape[-2] = o.numel(), 1
+                    env[m.outputs[0]] = o.view(shape)
             else:
                 for m in subs:
                     am = [env[i] for i in m.inputs]
