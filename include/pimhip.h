@@ -155,7 +155,9 @@ int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan);
  *   hn, cn [num_layers*num_directions, hidden_size], ordered (l0 fwd, l0 bwd, l1 fwd, ...)
  * y, hn, cn may not alias x, h0, c0.  Calls sharing one plan must be ordered on one stream.  Sequences of two or more
  * steps run in a kernel that needs all its blocks resident at once: a call on another stream than the device's
- * previous such call is ordered after it (an event wait), so that two of them never share the GPU. */
+ * previous such call is ordered after it (an event wait), so that two of them never share the GPU.  That kernel's
+ * launch carries a host-side step count and cannot be replayed from a graph: on a capturing stream the call records
+ * the per-step launches instead (mode 0 and 1), or returns PIMHIP_ERR_UNSUPPORTED when mode 2 or 3 forces the kernel. */
 int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn,
                         void* cn, int64_t seq_len, void* stream);
 

@@ -669,8 +669,10 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         return fail(PIMHIP_ERR_INVALID_ARGUMENT, "dimension above 2^31-1");
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    int device = -1;
+    PIMHIP_HIP_CHECK(hipGetDevice(&device));
     PimHipLstmPlan* plan = new PimHipLstmPlan();
-    PIMHIP_HIP_CHECK(hipGetDevice(&plan->device));
+    plan->device = device;
     plan->num_cus = st->num_cus;
     plan->has_biases = has_biases ? 1 : 0;
     plan->num_layers = num_layers;
@@ -859,9 +861,13 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         return PIMHIP_OK;
     }
 
-    if (*plan->abort_host != 0u || plan->reset_exchange) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
+    const bool capturing = capture != hipStreamCaptureStatusNone;
+    if (!capturing && (*plan->abort_host != 0u || plan->reset_exchange)) {
         // The previous forward of this plan timed out (or the entry layout changes): re-arm the flag and bring the
-        // exchange buffer back to its initial state (fill kernels, not memset nodes, so that callers may capture this call).
+        // exchange buffer back to its initial state.  (Left pending on a capturing stream: the launches recorded there
+        // do not use the buffer, and a recorded clear would run again with every replay.)
         fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 1, 0u);
         if (plan->hx) {
             const size_t words = plan->hx_region_words * kSeqMaxChains;
@@ -871,8 +877,18 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         *plan->abort_host = 0u;
         plan->reset_exchange = false;
     }
-    const bool use_seq = (plan->mode >= 2 && T + kSeqMaxChains <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T + kSeqMaxChains <= kSeqMaxT);
+    // A launch of the persistent kernel carries the host's count of super-steps (g_base) as an argument, and the flag
+    // bits in the exchange buffer follow that count: replayed from a graph, the same count would meet a buffer that has
+    // moved on.  On a capturing stream the automatic mode therefore records the per-step launches, and a plan forced to
+    // the persistent kernel refuses.
+    bool use_seq = (plan->mode >= 2 && T + kSeqMaxChains <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T + kSeqMaxChains <= kSeqMaxT);
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
+    if (use_seq && capturing) {
+        if (plan->mode >= 2)
+            return fail(PIMHIP_ERR_UNSUPPORTED, "the persistent sequence kernel cannot be recorded into a graph (mode %d forces it); "
+                                                "use mode 0 or 1 on a capturing stream", plan->mode);
+        use_seq = false;
+    }
     // seq_len == 1: fuse the input projection into the step (one launch per layer and direction).
     const bool fuse_xproj = !use_seq && T == 1;
 

@@ -123,3 +123,42 @@ def test_decoder_step_matches_libtorch_cpu(ops):
     logits = torch.addmm(step.bc.cpu(), r1, step.Wc.cpu().t())
     assert float((step.res[1].cpu().float() - r1.float()).abs().max()) <= 5e-3
     assert float((step.logits.cpu().float() - logits.float()).abs().max()) <= 5e-3
+
+
+def test_sequence_forward_records_per_step_launches_under_capture(ops):
+    """A persistent sequence launch depends on a host-side counter and cannot be replayed: on a capturing stream the
+    automatic mode records the per-step launches instead (bit-equal to mode 1), a plan forced to the persistent kernel
+    refuses, and the plan's exchange buffer is left as the eager launches expect it."""
+    T, I, Hs, layers = 7, 64, 256, 2
+    params, x, h0, c0 = oracle.lstm_inputs(7101, I, Hs, layers, False, T)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, False, T)
+    xd, hd, cd = x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV)
+    plan.set_mode(1)
+    want = [t.clone() for t in plan.forward(xd, hd, cd)]
+    plan.set_mode(0)
+    eager = [t.clone() for t in plan.forward(xd, hd, cd)]      # the persistent kernel, eager
+    torch.cuda.synchronize()
+    out = tuple(torch.zeros_like(t) for t in want)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            plan.forward(xd, hd, cd, out=out)
+            plan.set_mode(2)
+            with pytest.raises(ops.NNRuntimeException, match="graph"):
+                plan.forward(xd, hd, cd, out=out)
+            plan.set_mode(0)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for t in out:
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, w in zip(out, want):
+            assert torch.equal(got, w)
+        again = plan.forward(xd, hd, cd)                        # eager persistent launches between the replays
+        torch.cuda.synchronize()
+        for got, w in zip(again, eager):
+            assert torch.equal(got, w)
