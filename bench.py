@@ -415,7 +415,27 @@ def main():
         for _ in range(3):
             torch.lstm(x, (h0, c0), pc, True, 2, 0.0, False, False, False)
         other["cpu_libtorch_lstm_us_per_layer_step"] = round((time.perf_counter() - t) / 3 / 400 * 1e6, 1)
+        # context columns on the 4096 x 4096 shape: one thread (a per-core figure) and fp32 operands on all threads
+        def cpu_median_s(fn, n=7, limit_s=3.0):
+            fn()
+            ts, t_begin = [], time.perf_counter()
+            while len(ts) < n and (time.perf_counter() - t_begin) < limit_s:
+                t_ = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t_)
+            return sorted(ts)[len(ts) // 2]
+        s0 = shapes[0]
+        W0, x0, b0 = s0["pool"][0].cpu(), s0["x"].cpu().reshape(1, -1), s0["b"].cpu()
+        bytes0 = gemv_bytes(s0["n"], s0["k"])
+        W0f, x0f, b0f = W0.float(), x0.float(), b0.float()
+        fp32_gbs = 2 * bytes0 / cpu_median_s(lambda: torch.addmm(b0f, x0f, W0f.t())) / 1e9
+        torch.set_num_threads(1)
+        try:
+            one_thread_gbs = bytes0 / cpu_median_s(lambda: torch.addmm(b0, x0, W0.t())) / 1e9
+        finally:
+            torch.set_num_threads(threads)
         cpu = dict(value=round(b_total / t_total / 1e9, 2), unit="GB/s", cores=threads, kind="reference",
+                   one_thread_fp16_4096x4096_gbs=round(one_thread_gbs, 2), fp32_operands_4096x4096_gbs=round(fp32_gbs, 2),
                    sample="LibTorch CPU at::addmm(b, x, W^T) in fp16, the op atenAddmm passes through to: median of <= 20 "
                           "runs (<= 4 s) per sweep shape after 2 warm-ups, same weight every run (cache-warm), one pass of the "
                           "same 4-GEMV sweep; " + "; ".join(detail))
