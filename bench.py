@@ -246,6 +246,8 @@ def main():
                 cur, _, _ = plan_g.forward(cur, hg, cg)
 
         other["gnmt_lstm_stack_us_per_layer_step"] = round(timed_us(gnmt_stack, 30) / 250, 3)
+        # the same four calls (eight launches) replayed from a HIP graph
+        other["gnmt_lstm_stack_us_per_layer_step_hip_graph"] = round(graph_timed_us(lambda _s: gnmt_stack(), 1) / 250, 3)
         # one decoder step (seq_len 1, I = H = 1024): the fused step kernel, W_ih and W_hh streamed once (16.8 MB)
         prm, _, h0d, c0d = oracle.lstm_inputs(4101, 1024, 1024, 1, False, 1)
         plan_d = P.LstmPlan([q.to(dev) for q in prm], True, 1, False, 1)

@@ -155,9 +155,10 @@ int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan);
  *   hn, cn [num_layers*num_directions, hidden_size], ordered (l0 fwd, l0 bwd, l1 fwd, ...)
  * y, hn, cn may not alias x, h0, c0.  Calls sharing one plan must be ordered on one stream.  Sequences of two or more
  * steps run in a kernel that needs all its blocks resident at once: a call on another stream than the device's
- * previous such call is ordered after it (an event wait), so that two of them never share the GPU.  That kernel's
- * launch carries a host-side step count and cannot be replayed from a graph: on a capturing stream the call records
- * the per-step launches instead (mode 0 and 1), or returns PIMHIP_ERR_UNSUPPORTED when mode 2 or 3 forces the kernel. */
+ * previous such call is ordered after it (an event wait), so that two of them never share the GPU.  On a capturing
+ * stream that wait is left out (a graph cannot wait for another stream's event): order replays of such a graph against
+ * the device's other sequence calls yourself.  The call records kernels only; the one case a graph must not hold, the
+ * re-initialisation of the plan's buffers after a time-out or a change of mode, returns PIMHIP_ERR_UNSUPPORTED there. */
 int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn,
                         void* cn, int64_t seq_len, void* stream);
 
@@ -172,7 +173,8 @@ int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limi
 
 /* Selects how pimhip_lstm_forward runs the recurrence: 0 = automatic, 1 = one fused launch per step,
  * 2 = persistent sequence kernel (fails with PIMHIP_ERR_UNSUPPORTED if the shape does not fit), 3 = as 2 but with
- * four hidden units per block in every launch (2 runs a single unidirectional layer with eight). */
+ * four hidden units per block in every launch (2 runs a single unidirectional layer with eight).  A call with
+ * seq_len 1 runs the fused step launch in every mode. */
 int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);
 
 /* The dense input projection of one LSTM layer over all time steps, the only MFMA kernel of the path:

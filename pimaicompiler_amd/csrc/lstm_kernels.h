@@ -144,7 +144,7 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 //
 // Exchange buffer: hx[2][NB] entries of 64 bytes (entries of different blocks do not share a 64-byte segment,
 // which measurably shortens the exchange); chain k of block b uses the 8-byte word k of the entry, one fp16 per
-// wavefront.  |h| <= 1, so bit 14 of its fp16 pattern is always 0 (a NaN is published as 0) and carries the flag: with g = g_base + tau
+// wavefront.  |h| <= 1, so bit 14 of its fp16 pattern is always 0 (a NaN is published as 0) and carries the flag: with g = *g_counter + tau
 // counting super-steps over all launches of a plan, super-step g publishes into parity g & 1 with flag bit
 // (g >> 1) & 1, i.e. the bit flips every time a slot is rewritten.  A slot can only hold what was published two
 // super-steps earlier or the current values (publishing g + 2 needs the words of g + 1 from all blocks, which
@@ -208,13 +208,13 @@ struct LstmSeqChain {
 
 struct LstmSeqArgs {
     LstmSeqChain chain[kSeqMaxChains];
-    unsigned int* hx;          // [2][NB][kSeqEntryWords]; zero when g_base == 2
+    unsigned int* hx;          // [2][NB][kSeqEntryWords]; zero when *g_counter == 2
     unsigned int* abort_flag;  // set to 1 when a wait gives up; polled by the other waiting lanes
     unsigned int* abort_host;  // host-visible word set at the same time (what the host reads afterwards)
     long y_stride;             // elements between consecutive time steps of y
     int H;
     int T;
-    unsigned int g_base;       // super-steps this buffer has seen so far, plus 2
+    unsigned int* g_counter;   // device word: super-steps this buffer has seen so far, plus 2; advanced by the kernel
     unsigned int spin_limit;
 };
 
@@ -256,6 +256,11 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
     const int j = blockIdx.x * UNITS + wave;  // this wavefront's hidden unit
     const bool unit_ok = j < H;
     const int n_super = WAVEFRONT ? T + NC - 1 : T;
+    // The count of super-steps lives in device memory and is advanced by the kernel itself (last statement), so that a
+    // launch carries no host-side state and replays from a graph like any other.  Device-scope load: the previous
+    // launch stored it from another XCD.  The value is first needed when super-step 0 publishes.
+    const unsigned int g_base = __builtin_amdgcn_readfirstlane(
+        __hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 
     // ---- weights into registers: per chain the four gate rows of unit j, columns 16 * lane .. + 15 ----
     // Accumulator slot v holds gate {i, g, f, o}[v]: the transpose-sum below then leaves gate k in lane k.
@@ -325,7 +330,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
 #pragma unroll
             for (int k = 0; k < NW; ++k) words[k] = 0ull;
             if (tau > 0) {
-                const unsigned int gp = p.g_base + (unsigned int)tau - 1u;  // the super-step whose values are awaited
+                const unsigned int gp = g_base + (unsigned int)tau - 1u;  // the super-step whose values are awaited
                 const unsigned long long want = ((gp >> 1) & 1u) ? 0x4000400040004000ull : 0ull;
                 const unsigned long long* src =
                     reinterpret_cast<const unsigned long long*>(p.hx + ((long)(gp & 1u) * nb + tid) * kSeqEntryWords);
@@ -447,7 +452,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
         // The block's values are gathered in LDS and published by ONE lane with ONE store per 16 bytes: the time
         // until every block has seen a super-step grows by about 0.3 us with every further store per block.
         if (lane == 0) {
-            const unsigned int flag = (((p.g_base + (unsigned int)tau) >> 1) & 1u) << 14;
+            const unsigned int flag = (((g_base + (unsigned int)tau) >> 1) & 1u) << 14;
 #pragma unroll
             for (int k = 0; k < NC; ++k) {
                 // A NaN (from non-finite inputs or weights) has bit 14 set and cannot travel with the flag: y, hn and
@@ -472,7 +477,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
         }
         __syncthreads();
         if (tid == 0) {
-            const unsigned int g = p.g_base + (unsigned int)tau;
+            const unsigned int g = g_base + (unsigned int)tau;
             unsigned long long* dst = reinterpret_cast<unsigned long long*>(p.hx + ((long)(g & 1u) * nb + blockIdx.x) * kSeqEntryWords);
             const unsigned long long* src = reinterpret_cast<const unsigned long long*>(&pub[0][0]);
 #pragma unroll
@@ -487,6 +492,11 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
         super_step(tau + 1, xp_odd);
     }
     if (tau < n_super) super_step(tau, xp_even);
+    // Block 0 has finished its last super-step, for which (n_super >= 2, the launcher's condition) it needed what every
+    // block published one super-step earlier: every block has read the counter by now.  The next launch reads it after
+    // this one has ended.
+    if (blockIdx.x == 0 && tid == 0)
+        __hip_atomic_store(p.g_counter, g_base + (unsigned int)n_super, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace pimhip

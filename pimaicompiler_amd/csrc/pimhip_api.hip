@@ -561,7 +561,7 @@ struct PimHipLstmPlan {
     int mode = 0;
     bool seq_kernel_ok = false;      // shape fits the persistent sequence kernel
     unsigned int spin_limit = 1u << 22;
-    unsigned int g_count[kSeqMaxChains + 1] = {2, 2, 2, 2, 2};  // per chain count: super-steps its buffer region has seen, plus 2
+    unsigned int* g_counters = nullptr;  // device, [kSeqMaxChains + 1]: per chain count, super-steps its region of hx has seen, plus 2
     size_t hx_region_words = 0;      // 32-bit words of one region of hx (one region per chain count)
     int max_wavefront = kSeqMaxChains;  // layers of a unidirectional stack advanced by one persistent launch
 
@@ -607,6 +607,7 @@ int destroy_plan_locked(PimHipLstmPlan* plan)
     if (plan->ybuf[1]) hipFree(plan->ybuf[1]);
     if (plan->c_state) hipFree(plan->c_state);
     if (plan->hx) hipFree(plan->hx);
+    if (plan->g_counters) hipFree(plan->g_counters);
     if (plan->abort_flag) hipFree(plan->abort_flag);
     if (plan->abort_host) hipHostFree(plan->abort_host);
     if (prev >= 0) hipSetDevice(prev);
@@ -760,6 +761,9 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         const size_t words = plan->hx_region_words * kSeqMaxChains;
         PLAN_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned int)));
         PLAN_HIP_CHECK(hipMemsetAsync(plan->hx, 0, words * sizeof(unsigned int), s));
+        PLAN_HIP_CHECK(hipMalloc(&plan->g_counters, (kSeqMaxChains + 1) * sizeof(unsigned int)));
+        fill_u32_kernel<<<1, 64, 0, s>>>(plan->g_counters, kSeqMaxChains + 1, 2u);
+        PLAN_HIP_CHECK(hipGetLastError());
     }
     PLAN_HIP_CHECK(hipStreamSynchronize(s));
 #undef PLAN_HIP_CHECK
@@ -864,30 +868,27 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
     const bool capturing = capture != hipStreamCaptureStatusNone;
-    if (!capturing && (*plan->abort_host != 0u || plan->reset_exchange)) {
-        // The previous forward of this plan timed out (or the entry layout changes): re-arm the flag and bring the
-        // exchange buffer back to its initial state.  (Left pending on a capturing stream: the launches recorded there
-        // do not use the buffer, and a recorded clear would run again with every replay.)
-        fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 1, 0u);
-        if (plan->hx) {
-            const size_t words = plan->hx_region_words * kSeqMaxChains;
-            fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->hx, words, 0u);
-        }
-        for (int i = 0; i <= kSeqMaxChains; ++i) plan->g_count[i] = 2;
-        *plan->abort_host = 0u;
-        plan->reset_exchange = false;
-    }
-    // A launch of the persistent kernel carries the host's count of super-steps (g_base) as an argument, and the flag
-    // bits in the exchange buffer follow that count: replayed from a graph, the same count would meet a buffer that has
-    // moved on.  On a capturing stream the automatic mode therefore records the per-step launches, and a plan forced to
-    // the persistent kernel refuses.
-    bool use_seq = (plan->mode >= 2 && T + kSeqMaxChains <= kSeqMaxT) || (plan->mode == 0 && plan->seq_kernel_ok && T >= 2 && T + kSeqMaxChains <= kSeqMaxT);
+    // One step: the fused step kernel in every mode (the persistent kernel's hand-over of its step count to the next
+    // launch needs two super-steps).
+    const bool use_seq = T >= 2 && T + kSeqMaxChains <= kSeqMaxT && (plan->mode >= 2 || (plan->mode == 0 && plan->seq_kernel_ok));
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
-    if (use_seq && capturing) {
-        if (plan->mode >= 2)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "the persistent sequence kernel cannot be recorded into a graph (mode %d forces it); "
-                                                "use mode 0 or 1 on a capturing stream", plan->mode);
-        use_seq = false;
+    if (*plan->abort_host != 0u) {
+        // The previous sequence kernel of this plan timed out (pimhip_lstm_plan_status has had its chance to report it).
+        *plan->abort_host = 0u;
+        plan->reset_exchange = true;
+    }
+    if (use_seq && plan->reset_exchange) {
+        // After a time-out or a change of the entry layout: re-arm the flag and bring the exchange buffer and its step
+        // counters back to their initial state.
+        if (capturing)
+            return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's exchange buffer has to be re-initialised (after a time-out or a change of "
+                                                "mode), which a graph must not record: run one forward outside the capture first");
+        fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 1, 0u);
+        const size_t words = plan->hx_region_words * kSeqMaxChains;
+        fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->hx, words, 0u);
+        fill_u32_kernel<<<1, 64, 0, s>>>(plan->g_counters, kSeqMaxChains + 1, 2u);
+        PIMHIP_HIP_CHECK(hipGetLastError());
+        plan->reset_exchange = false;
     }
     // seq_len == 1: fuse the input projection into the step (one launch per layer and direction).
     const bool fuse_xproj = !use_seq && T == 1;
@@ -895,8 +896,12 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     const half_t* layer_in = (const half_t*)x;
     const long y_stride = (long)D * H;
     if (use_seq) {
-        rc = order_after_previous_sequence_launch(st, s);
-        if (rc != PIMHIP_OK) return rc;
+        // (Not on a capturing stream, where an event of another stream cannot be waited for: a caller who replays
+        // graphs orders them against the device's other sequence launches.)
+        if (!capturing) {
+            rc = order_after_previous_sequence_launch(st, s);
+            if (rc != PIMHIP_OK) return rc;
+        }
         // Layers are taken in groups that one persistent launch advances together: the two directions of a
         // bidirectional layer, or up to kSeqMaxChains consecutive layers of a unidirectional stack as a wavefront.
         int l = 0;
@@ -947,9 +952,8 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             a.y_stride = y_stride;
             a.H = (int)H;
             a.T = (int)T;
-            a.g_base = plan->g_count[nc];
+            a.g_counter = plan->g_counters + nc;
             a.spin_limit = plan->spin_limit;
-            plan->g_count[nc] += (unsigned int)((D == 2) ? T : T + nc - 1);
             const dim3 grid(plan->seq_blocks), block(256);
             if (D == 2) {
                 lstm_seq_f16_kernel<2, false><<<grid, block, 0, s>>>(a);

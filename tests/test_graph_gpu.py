@@ -125,40 +125,59 @@ def test_decoder_step_matches_libtorch_cpu(ops):
     assert float((step.logits.cpu().float() - logits.float()).abs().max()) <= 5e-3
 
 
-def test_sequence_forward_records_per_step_launches_under_capture(ops):
-    """A persistent sequence launch depends on a host-side counter and cannot be replayed: on a capturing stream the
-    automatic mode records the per-step launches instead (bit-equal to mode 1), a plan forced to the persistent kernel
-    refuses, and the plan's exchange buffer is left as the eager launches expect it."""
-    T, I, Hs, layers = 7, 64, 256, 2
-    params, x, h0, c0 = oracle.lstm_inputs(7101, I, Hs, layers, False, T)
-    plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, False, T)
-    xd, hd, cd = x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV)
-    plan.set_mode(1)
-    want = [t.clone() for t in plan.forward(xd, hd, cd)]
-    plan.set_mode(0)
-    eager = [t.clone() for t in plan.forward(xd, hd, cd)]      # the persistent kernel, eager
-    torch.cuda.synchronize()
-    out = tuple(torch.zeros_like(t) for t in want)
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
+def test_sequence_forward_replays_from_a_graph(ops):
+    """The persistent sequence kernel keeps its step count in device memory, so a recorded launch replays: every replay
+    equals the eager launch bit for bit, with eager launches of the same plan between the replays.  The one thing a
+    graph must not record, the re-initialisation of the exchange buffer after a change of mode, is refused."""
+    T, I, Hs = 7, 64, 256
+    for layers, bidir in ((2, False), (1, True), (1, False)):
+        params, x, h0, c0 = oracle.lstm_inputs(7101 + layers + 2 * bidir, I, Hs, layers, bidir, T)
+        plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, bidir, T)
+        xd, hd, cd = x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV)
+        x2 = (0.5 * xd + 0.25).contiguous()
+        eager = {k: [t.clone() for t in plan.forward(v, hd, cd)] for k, v in (("a", xd), ("b", x2))}
+        torch.cuda.synchronize()
+        plan.status()
+        x_static = xd.clone()
+        out = tuple(torch.zeros_like(t) for t in eager["a"])
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            plan.forward(x_static, hd, cd, out=out)                 # warm-up on the capture stream
+            with torch.cuda.graph(graph, stream=side):
+                plan.forward(x_static, hd, cd, out=out)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for rep in range(4):
+            key, src = (("a", xd), ("b", x2))[rep & 1]
+            x_static.copy_(src)
+            for t in out:
+                t.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            plan.status()
+            for got, w in zip(out, eager[key]):
+                assert torch.equal(got, w)
+            if rep != 2:                                              # an odd number of eager launches in between as well
+                again = plan.forward(x2, hd, cd)
+                torch.cuda.synchronize()
+                for got, w in zip(again, eager["b"]):
+                    assert torch.equal(got, w)
+    # a pending re-initialisation (mode 3 lays the single chain's entries out differently) is not recorded
+    plan.set_mode(3)
+    graph2 = torch.cuda.CUDAGraph()
+    scratch_out = torch.empty_like(hd)
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        with torch.cuda.graph(graph, stream=side):
-            plan.forward(xd, hd, cd, out=out)
-            plan.set_mode(2)
-            with pytest.raises(ops.NNRuntimeException, match="graph"):
-                plan.forward(xd, hd, cd, out=out)
-            plan.set_mode(0)
+        with torch.cuda.graph(graph2, stream=side):
+            with pytest.raises(ops.NNRuntimeException, match="outside the capture"):
+                plan.forward(x_static, hd, cd, out=out)
+            ops.aten_add(hd, cd, out=scratch_out)                    # something to record
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    for rep in range(3):
-        for t in out:
-            t.fill_(float("nan"))
-        graph.replay()
-        torch.cuda.synchronize()
-        for got, w in zip(out, want):
-            assert torch.equal(got, w)
-        again = plan.forward(xd, hd, cd)                        # eager persistent launches between the replays
-        torch.cuda.synchronize()
-        for got, w in zip(again, eager):
-            assert torch.equal(got, w)
+    got = plan.forward(xd, hd, cd)
+    torch.cuda.synchronize()
+    plan.status()
+    for g_, w in zip(got, eager["a"]):
+        assert float((g_.float() - w.float()).abs().max()) <= 2e-3
