@@ -142,13 +142,21 @@ struct GemvGroupArgs {
     int count;
 };
 
-template <int R, int U, int WAVES, int KS>
-__global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_group_kernel(GemvGroupArgs g)
+// Each problem runs with the block shape a launch of its own would use for its row length (long rows: the four
+// wavefronts of a block split the reduction of two rows; shorter rows: two wavefronts per pair of rows).
+static constexpr int kGemvGroupThreads = 256;
+static constexpr int kGemvGroupLongRow = 4096;
+__host__ __device__ inline int gemv_group_rows_per_block(int K) { return K >= kGemvGroupLongRow ? 2 : 4; }
+
+__global__ __launch_bounds__(kGemvGroupThreads) void gemv_mv_f16_group_kernel(GemvGroupArgs g)
 {
     int i = 0;
     while (i + 1 < g.count && (int)blockIdx.x >= g.block_begin[i + 1]) ++i;
-    gemv_mv_f16_body<R, U, WAVES, KS>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i],
-                                      (int)blockIdx.x - g.block_begin[i]);
+    const int block = (int)blockIdx.x - g.block_begin[i];
+    if (g.K[i] >= kGemvGroupLongRow)
+        gemv_mv_f16_body<2, 4, 4, 4>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i], block);
+    else
+        gemv_mv_f16_body<2, 2, 4, 2>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i], block);
 }
 
 // MV order, any K / leading dimension / alignment: one wavefront per row, 2-byte loads.

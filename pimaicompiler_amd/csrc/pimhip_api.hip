@@ -360,8 +360,6 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
     if (count == 0) return PIMHIP_OK;
     if (!outs || !ins || !weights || !in_ws || !out_ws) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "null array argument");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int R = 2, U = 2, WAVES = 4, KS = 2;
-    constexpr int rows_per_block = (WAVES / KS) * R;
     int done = 0;
     while (done < count) {
         GemvGroupArgs g;
@@ -384,11 +382,12 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
             g.K[n] = (int)in_ws[i];
             g.relu[n] = a == PIMHIP_ACT_RELU;
             g.block_begin[n] = blocks;
+            const int rows_per_block = gemv_group_rows_per_block((int)in_ws[i]);
             blocks += ((int)out_ws[i] + rows_per_block - 1) / rows_per_block;
         }
         g.block_begin[n] = blocks;
         g.count = n;
-        gemv_mv_f16_group_kernel<R, U, WAVES, KS><<<blocks, WAVES * 64, 0, s>>>(g);
+        gemv_mv_f16_group_kernel<<<blocks, kGemvGroupThreads, 0, s>>>(g);
         PIMHIP_HIP_CHECK(hipGetLastError());
         done += n;
     }
