@@ -299,6 +299,22 @@ def main():
         # device's (64 launches replayed from a HIP graph), the second what a Python caller sees
         other["gemv_1024x1024_us"] = round(graph_timed_us(c1_launch, 64), 3)
         other["gemv_1024x1024_issued_from_python_us"] = round(timed_us(c1_launch, 200), 3)
+        # the same GEMV through the C++ operator with the reference's signature (customAtenAddmm: shape logic, output
+        # allocation, launch), 200 calls in a row from C++: the host's cost per call, and the rate the GPU sees
+        try:
+            from pimaicompiler_amd import _aten_ops_pimhip as cpp_ops
+            cpp_ops.initialize(0)
+            c1_w_t, c1_x2 = c1_pool[0].t(), c1_x.view(1, 1024)
+            cpp_ops.customAtenAddmmHostMicroseconds("none", c1_b, c1_x2, c1_w_t, 20)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            host_us = cpp_ops.customAtenAddmmHostMicroseconds("none", c1_b, c1_x2, c1_w_t, 200)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            other["cpp_custom_aten_addmm_1024x1024"] = {"host_us_per_call": round(host_us, 3),
+                                                        "us_per_call_on_the_stream": round(e0.elapsed_time(e1) * 1e3 / 200, 3)}
+        except ImportError:
+            pass
         # MoE FFN decode step (router 768 -> 8, then one expert 768 -> 3072 ReLU -> 768): three dependent launches on
         # resident (warm) weights, the expert fixed so that no host round trip for the argmax is inside the figure
         wr, w1, w2 = (0.02 * torch.randn(8, 768, device=dev)).half(), (0.02 * torch.randn(3072, 768, device=dev)).half(), \

@@ -2,6 +2,8 @@
 // maintainer of the reference would link.
 #include <torch/extension.h>
 
+#include <chrono>
+
 #include "aten_ops_pimhip.h"
 
 namespace ops = nn_compiler::runtime::op_executor;
@@ -15,6 +17,14 @@ PYBIND11_MODULE(_aten_ops_pimhip, m)
         torch::jit::IValue out;
         ops::customAtenAddmm(act, self, mat1, mat2, beta, alpha, out, nullptr);
         return out.toTensor();
+    });
+    // `iters` calls in a row from C++: what one call costs the host thread (wall time of the loop / iters, in us).
+    m.def("customAtenAddmmHostMicroseconds", [](const std::string& act, at::Tensor self, at::Tensor mat1, at::Tensor mat2, int iters) {
+        torch::jit::IValue out;
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < iters; ++i) ops::customAtenAddmm(act, self, mat1, mat2, 1, 1, out, nullptr);
+        const auto t1 = std::chrono::steady_clock::now();
+        return std::chrono::duration<double, std::micro>(t1 - t0).count() / (iters > 0 ? iters : 1);
     });
     m.def("customAtenMatmul", [](at::Tensor self, at::Tensor other) {
         torch::jit::IValue out;
