@@ -82,12 +82,20 @@ int get_split_workspace(DeviceState* st, hipStream_t stream, size_t partial_elem
 {
     std::lock_guard<std::mutex> lock(g_mutex);
     SplitWorkspace& ws = st->workspaces[stream];
+    const bool gave_up = ws.status && *ws.status != 0u;
+    if (!ws.status || ws.partial_elems < partial_elems || gave_up) {
+        // Allocation, synchronisation and the memset below are not for a graph: ask before touching anything.
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        PIMHIP_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
+        if (capture != hipStreamCaptureStatusNone)
+            return fail(PIMHIP_ERR_UNSUPPORTED, "this I_X_W product needs its stream's workspace (re)allocated, which a graph must not "
+                                                "record: run it once on this stream before the capture");
+    }
     if (!ws.status) {
         PIMHIP_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&ws.status), sizeof(unsigned int), hipHostMallocMapped));
         *ws.status = 0u;
         PIMHIP_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&ws.status_dev), ws.status, 0));
     }
-    const bool gave_up = *ws.status != 0u;
     if (ws.partial_elems < partial_elems || gave_up) {
         // Work already queued on this stream may still use the old buffer.
         PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));

@@ -182,3 +182,46 @@ def test_sequence_forward_replays_from_a_graph(ops):
     plan.status()
     for g_, w in zip(got, eager["a"]):
         assert float((g_.float() - w.float()).abs().max()) <= 2e-3
+
+
+def test_sliced_vm_product_replays_from_a_graph(ops):
+    """An I_X_W product whose reduction is sliced over blocks uses a per-stream workspace: its first use on a stream
+    allocates (refused while capturing, with a message that says what to do), later uses record one kernel and replay."""
+    from pimaicompiler_amd import _lib as L
+    lib = L.load()
+    g = torch.Generator().manual_seed(11)
+    K = N = 2048
+    A = (0.02 * torch.randn(K, N, generator=g)).half().to(DEV)
+    xs = [torch.randn(K, generator=g).half().to(DEV) for _ in range(2)]
+    x, y = xs[0].clone(), torch.empty(N, dtype=torch.float16, device=DEV)
+
+    def launch():
+        return lib.pimhip_execute_gemv(y.data_ptr(), x.data_ptr(), A.data_ptr(), None, K, N, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W,
+                                       torch.cuda.current_stream().cuda_stream)
+    eager = []
+    for xv in xs:
+        x.copy_(xv)
+        assert launch() == 0
+        torch.cuda.synchronize()
+        eager.append(y.clone())
+        assert float((y.float() - (xv.float() @ A.float())).abs().max()) <= 2e-3
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    refused = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(refused, stream=side):
+            assert launch() == L.PIMHIP_ERR_UNSUPPORTED
+            assert b"before the capture" in lib.pimhip_last_error()
+            y.add_(0)                                       # something to record
+        assert launch() == 0                                # the warm-up the message asks for
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            assert launch() == 0
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        x.copy_(xs[rep & 1])
+        y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager[rep & 1])
