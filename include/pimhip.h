@@ -172,7 +172,7 @@ int pimhip_lstm_plan_status(PimHipLstmPlan* plan);
 int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limit);
 
 /* Selects how pimhip_lstm_forward runs the recurrence: 0 = automatic, 1 = one fused launch per step,
- * 2 = persistent sequence kernel (fails with PIMHIP_ERR_UNSUPPORTED if the shape does not fit), 3 = as 2 but with
+ * 2 = persistent sequence kernel (hidden_size up to 2048; fails with PIMHIP_ERR_UNSUPPORTED otherwise), 3 = as 2 but with
  * four hidden units per block in every launch (2 runs a single unidirectional layer with eight).  A call with
  * seq_len 1 runs the fused step launch in every mode. */
 int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);

@@ -128,7 +128,8 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 //
 // Grid: NB = ceil(H / UNITS) blocks of UNITS wavefronts (H <= 1024, H % 8 == 0; UNITS = 4, or 8 for a single chain,
 // whose entry then still is one 16-byte store and load and whose exchange among half as many blocks is about 0.4 us
-// shorter), all resident at once.  The text below is written for UNITS = 4.  Block b owns
+// shorter), all resident at once.  Hidden sizes up to 2048 run with COLS = 32 columns of a weight row per lane and eight
+// units per block (256 blocks at most), for one layer or the two directions of one (a second layer's W_ih would spill).  The text below is written for UNITS = 4.  Block b owns
 // hidden units 4b .. 4b+3 of every chain, one unit per wavefront: wavefront w keeps, per chain, the four W_hh
 // gate rows of unit 4b+w (and the four W_ih rows for wavefront chains k > 0) in registers for the whole
 // launch (lane l holds columns 16l .. 16l+15 of each row) and the cell states in registers.
@@ -162,6 +163,7 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 // ---------------------------------------------------------------------------------------------
 static constexpr int kSeqUnits = 4;        // hidden units per block, one per wavefront
 static constexpr int kSeqMaxH = 1024;      // 64 lanes x 16 columns
+static constexpr int kSeqMaxHWide = 2048;  // 64 lanes x 32 columns (eight units per block; one layer, or the two directions of one)
 static constexpr int kSeqEntryWords = 16;  // 32-bit words between the entries of consecutive blocks (64 bytes)
 static constexpr int kSeqMaxT = 1 << 30;    // super-steps per launch (the counters are 32-bit)
 static constexpr int kSeqMaxChains = 4;
@@ -237,14 +239,18 @@ __device__ __forceinline__ void store16_device_scope(void* p, unsigned long long
     asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
 }
 
-template <int NC, bool WAVEFRONT, int UNITS = kSeqUnits>
+template <int NC, bool WAVEFRONT, int UNITS = kSeqUnits, int COLS = 16>
 __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
 {
     static_assert(UNITS == 4 || UNITS == 8, "one or two 8-byte words per chain and block");
+    static_assert(COLS == 16 || COLS == 32, "columns of a weight row per lane");
+    constexpr int MAXH = 64 * COLS;  // widest hidden state this instantiation takes
+    constexpr int CH = COLS / 8;     // 16-byte pieces of a weight row per lane
+    static_assert(MAXH <= 64 * UNITS * UNITS, "lane t of a block fetches the entry of block t");
     constexpr int WPC = UNITS / 4;  // 8-byte words per chain in an entry
     constexpr int NW = NC * WPC;    // 8-byte words of an entry that are in use
     static_assert(NC >= 1 && NC <= kSeqMaxChains && 2 * NW <= kSeqEntryWords, "an entry is 64 bytes");
-    __shared__ __align__(16) half_t hbuf[2][NC][kSeqMaxH];   // published h per chain, double buffered by parity
+    __shared__ __align__(16) half_t hbuf[2][NC][MAXH];       // published h per chain, double buffered by parity
     __shared__ __align__(16) unsigned short pub[NC][UNITS];  // this block's next entry: chain k, wavefront w
 
     const int tid = threadIdx.x;
@@ -264,8 +270,8 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
 
     // ---- weights into registers: per chain the four gate rows of unit j, columns 16 * lane .. + 15 ----
     // Accumulator slot v holds gate {i, g, f, o}[v]: the transpose-sum below then leaves gate k in lane k.
-    half8_t w_hh[NC][4][2];
-    half8_t w_ih[WAVEFRONT ? NC : 1][4][2];  // entry 0 unused
+    half8_t w_hh[NC][4][CH];
+    half8_t w_ih[WAVEFRONT ? NC : 1][4][CH];  // entry 0 unused
     {
         const int gate_of_slot[4] = {0, 2, 1, 3};
         half8_t zero;
@@ -276,8 +282,8 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
 #pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const int col = lane * 16 + c * 8;
+                for (int c = 0; c < CH; ++c) {
+                    const int col = lane * COLS + c * 8;
                     const bool ok = unit_ok && col < H;  // H % 8 == 0: a chunk is entirely inside or outside the row
                     const long off = ((long)gate_of_slot[v] * H + j) * H + col;
                     w_hh[k][v][c] = ok ? *reinterpret_cast<const half8_t*>(p.chain[k].w_hh + off) : zero;
@@ -286,7 +292,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             }
         }
         // Columns at and past H stay zero in all h buffers for the whole kernel.
-        for (int i = tid; i < 2 * NC * kSeqMaxH / 8; i += 64 * UNITS) reinterpret_cast<half8_t*>(&hbuf[0][0][0])[i] = zero;
+        for (int i = tid; i < 2 * NC * MAXH / 8; i += 64 * UNITS) reinterpret_cast<half8_t*>(&hbuf[0][0][0])[i] = zero;
     }
     __syncthreads();
 
@@ -322,7 +328,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
     bool gave_up = false;
 
     auto super_step = [&](const int tau, float (&xp_slot)[NC]) __attribute__((always_inline)) {
-        half_t(*hb)[kSeqMaxH] = hbuf[tau & 1];
+        half_t(*hb)[MAXH] = hbuf[tau & 1];
 
         // ---- 1. what block `tid` published at super-step tau - 1 (or the initial state) into LDS ----
         if (has_entry) {
@@ -388,17 +394,26 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
         float acc[NC][4];
 #pragma unroll
         for (int k = 0; k < NC; ++k) {
-            const half8_t ha = *reinterpret_cast<const half8_t*>(&hb[k][lane * 16]);
-            const half8_t hc = *reinterpret_cast<const half8_t*>(&hb[k][lane * 16 + 8]);
+            half8_t hv[CH];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_hh[k][v][1], hc, dot8(w_hh[k][v][0], ha, 0.0f));
+            for (int c = 0; c < CH; ++c) hv[c] = *reinterpret_cast<const half8_t*>(&hb[k][lane * COLS + c * 8]);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                acc[k][v] = 0.0f;
+#pragma unroll
+                for (int c = 0; c < CH; ++c) acc[k][v] = dot8(w_hh[k][v][c], hv[c], acc[k][v]);
+            }
             if (WAVEFRONT && k > 0) {
                 // Input of layer k at its time step: h of layer k - 1 at the same time step, published one
                 // super-step ago, which is what chain k - 1's buffer holds now.
-                const half8_t xa = *reinterpret_cast<const half8_t*>(&hb[k - 1][lane * 16]);
-                const half8_t xc = *reinterpret_cast<const half8_t*>(&hb[k - 1][lane * 16 + 8]);
+                half8_t xv[CH];
 #pragma unroll
-                for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_ih[k][v][1], xc, dot8(w_ih[k][v][0], xa, acc[k][v]));
+                for (int c = 0; c < CH; ++c) xv[c] = *reinterpret_cast<const half8_t*>(&hb[k - 1][lane * COLS + c * 8]);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) acc[k][v] = dot8(w_ih[k][v][c], xv[c], acc[k][v]);
+                }
             }
         }
 

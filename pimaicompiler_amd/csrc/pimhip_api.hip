@@ -596,6 +596,7 @@ struct PimHipLstmPlan {
     int seq_blocks = 0;
     bool reset_exchange = false;     // the next forward starts from a cleared exchange buffer (layout change)
     bool seq_units8_ok = false;      // a single chain may run with 8 hidden units per block (half as many blocks)
+    bool seq_wide = false;           // 1024 < H <= 2048: 32 columns per lane, eight units per block, one layer per launch
 };
 
 namespace
@@ -701,6 +702,8 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         if (e_ != hipSuccess) return cleanup_fail(fail(PIMHIP_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_))); \
     } while (0)
 
+    plan->seq_wide = H > kSeqMaxH && H <= kSeqMaxHWide;
+    if (plan->seq_wide) plan->max_wavefront = 1;  // W_hh and W_ih of a second layer would not fit a wavefront's registers
     PLAN_HIP_CHECK(hipMalloc(&plan->bsum_all, sizeof(float) * 4 * H * plan->cells.size()));
     for (int l = 0; l < num_layers; ++l) {
         for (int d = 0; d < D; ++d) {
@@ -755,8 +758,12 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         int per_cu = 0;
         PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_seq_f16_kernel<kSeqMaxChains, true>, 256, 0));
         plan->seq_kernel_ok = (int64_t)per_cu * plan->num_cus >= plan->seq_blocks;
+    } else if (plan->seq_wide) {
+        int per_cu = 0;
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_seq_f16_kernel<2, false, 8, 32>, 512, 0));
+        plan->seq_kernel_ok = (int64_t)per_cu * plan->num_cus >= (plan->seq_blocks + 1) / 2;
     }
-    if (plan->seq_kernel_ok) {
+    if (plan->seq_kernel_ok && !plan->seq_wide) {
         int per_cu8 = 0;
         PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu8, lstm_seq_f16_kernel<1, true, 8>, 512, 0));
         plan->seq_units8_ok = (int64_t)per_cu8 * plan->num_cus >= (plan->seq_blocks + 1) / 2;
@@ -962,7 +969,13 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             a.g_counter = plan->g_counters + nc;
             a.spin_limit = plan->spin_limit;
             const dim3 grid(plan->seq_blocks), block(256);
-            if (D == 2) {
+            if (plan->seq_wide) {
+                const dim3 grid8((unsigned)((H + 7) / 8)), block8(512);
+                if (D == 2)
+                    lstm_seq_f16_kernel<2, false, 8, 32><<<grid8, block8, 0, s>>>(a);
+                else
+                    lstm_seq_f16_kernel<1, true, 8, 32><<<grid8, block8, 0, s>>>(a);  // max_wavefront == 1
+            } else if (D == 2) {
                 lstm_seq_f16_kernel<2, false><<<grid, block, 0, s>>>(a);
             } else {
                 switch (nc) {

@@ -56,14 +56,17 @@ CASES = [  # I, H, L, bidirectional, T, biases
     (8, 1024, 1, False, 3, True), (40, 1032, 1, False, 3, True), (16, 2048, 1, True, 2, False),
     (16, 64, 4, False, 7, True), (16, 64, 5, False, 6, True), (24, 136, 7, False, 3, False), (16, 64, 4, False, 1, True),
     (16, 64, 2, False, 2, True), (32, 1024, 4, False, 5, True),
+    # 1024 < H <= 2048: the persistent kernel with 32 columns per lane, one layer (or two directions) per launch
+    (32, 2048, 1, False, 5, True), (16, 1536, 2, False, 4, True), (24, 2048, 2, True, 3, True), (8, 1040, 3, False, 6, False),
+    (8, 2056, 1, False, 3, True),
 ]
 
 
 @pytest.mark.parametrize("mode", [0] + MODES)
 @pytest.mark.parametrize("I,H,L,bidir,T,has_b", CASES)
 def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
-    if mode >= 2 and H > 1024:
-        pytest.skip("the persistent kernel takes hidden sizes up to 1024; larger ones run step by step")
+    if mode >= 2 and H > 2048:
+        pytest.skip("the persistent kernel takes hidden sizes up to 2048; larger ones run step by step")
     params, x, h0, c0 = oracle.lstm_inputs(900 + I + H + T, I, H, L, bidir, T, has_b)
     g = torch.Generator().manual_seed(T)
     h0 = (0.3 * torch.randn(h0.shape, generator=g)).half()
@@ -76,7 +79,7 @@ def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
 
 
 def test_persistent_kernel_refuses_what_it_cannot_hold(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(1, 16, 2048, 1, False, 2)
+    params, x, h0, c0 = oracle.lstm_inputs(1, 16, 2056, 1, False, 2)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 2)
     with pytest.raises(ops.NNRuntimeException):
         plan.set_mode(2)
