@@ -153,9 +153,10 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 // each 8-byte word on its own.  A block gathers its values in LDS and publishes them with ONE store (8 bytes for
 // one chain, 16 for two); a waiting lane reads a block's entry with ONE load of the same size.  The round trip of
 // that pair through the memory side is the cost of a super-step: measured at 256 blocks, every further load per
-// poll and every further store per block adds about 0.3 us.  The buffer is zero when g = 2, the first value
-// the host uses; every launch writes every fp16 of every entry in every super-step, so the sequence of flag bits
-// per slot stays alternating across launches.  After a time-out the host clears the buffer and restarts at g = 2.
+// poll and every further store per block adds about 0.3 us.  The buffer is zero when g = 2, the value
+// the host initialises the counter with; every launch writes every fp16 of every entry in every super-step, so the
+// sequence of flag bits per slot stays alternating across launches.  After a time-out the host clears the buffer and
+// sets the counter back to 2.
 //
 // Every wait is bounded: after `spin_limit` polls a lane raises *abort_flag and stops waiting; lanes poll
 // the flag every 256 spins and stop waiting once it is set.  The kernel then runs to the end with
