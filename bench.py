@@ -435,14 +435,7 @@ def main():
             t_total += med
             b_total += gemv_bytes(s["n"], s["k"])
             detail.append(f"{s['n']}x{s['k']}: {med * 1e3:.2f} ms")
-        # LibTorch CPU at::lstm on the LSTM configuration (fp16, as the reference's atenLstm1 calls it)
-        pc = [q for q in params]
-        torch.lstm(x, (h0, c0), pc, True, 2, 0.0, False, False, False)
-        t = time.perf_counter()
-        for _ in range(3):
-            torch.lstm(x, (h0, c0), pc, True, 2, 0.0, False, False, False)
-        other["cpu_libtorch_lstm_us_per_layer_step"] = round((time.perf_counter() - t) / 3 / 400 * 1e6, 1)
-        # context columns on the 4096 x 4096 shape: one thread (a per-core figure) and fp32 operands on all threads
+
         def cpu_median_s(fn, n=7, limit_s=3.0):
             fn()
             ts, t_begin = [], time.perf_counter()
@@ -451,6 +444,11 @@ def main():
                 fn()
                 ts.append(time.perf_counter() - t_)
             return sorted(ts)[len(ts) // 2]
+        # LibTorch CPU at::lstm on the LSTM configuration (fp16, as the reference's atenLstm1 calls it)
+        pc = [q for q in params]
+        other["cpu_libtorch_lstm_us_per_layer_step"] = round(
+            cpu_median_s(lambda: torch.lstm(x, (h0, c0), pc, True, 2, 0.0, False, False, False), n=5, limit_s=5.0) / 400 * 1e6, 1)
+        # context columns on the 4096 x 4096 shape: one thread (a per-core figure) and fp32 operands on all threads
         s0 = shapes[0]
         W0, x0, b0 = s0["pool"][0].cpu(), s0["x"].cpu().reshape(1, -1), s0["b"].cpu()
         bytes0 = gemv_bytes(s0["n"], s0["k"])
