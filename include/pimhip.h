@@ -104,6 +104,18 @@ int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* other_shape4
 int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
                         int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  Same arguments, result and bits as pimhip_execute_gemv,
+ * but the partial sums of a sliced I_X_W product go through a 256 KiB array that is part of the library's
+ * image on every GPU it runs on, instead of a per-stream workspace: the call allocates, frees and synchronises
+ * nothing and records kernels only.  A product that needs more than 65536 partial sums
+ * ((slices - 1) * out_w; none that pimhip_execute_gemv slices on a 256-CU part does) is refused with
+ * PIMHIP_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that may overlap there (different streams,
+ * or replays of graphs holding such calls) race and must be ordered by the caller.  After a wait that gave up, the next
+ * call returns PIMHIP_ERR_TIMEOUT, refills the array (it synchronises the stream then) and launches nothing. */
+int pimhip_execute_gemv_static(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
+                               int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
+
 /* Replaces the VV branch of customAtenMatmul (aten_ops.cpp:841-882): out[0] = sum_k a[k] * b[k]. */
 int pimhip_execute_dot(void* out, const void* a, const void* b, int64_t in_w, void* stream);
 

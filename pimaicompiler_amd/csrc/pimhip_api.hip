@@ -43,6 +43,18 @@ int fail(int status, const char* fmt, ...)
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+__global__ void fill_u32_kernel(unsigned int* p, size_t n, unsigned int v)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// Partial-sum records of pimhip_execute_gemv_static, the entry point that allocates nothing: 256 KiB that every GPU
+// the library runs on holds until the process ends.  In host code this name is only a stand-in for the symbol: the
+// address a kernel can use is looked up once per device (pimhip_initialize) and kept in DeviceState::static_partial.
+constexpr size_t kStaticScratchFloats = 64 * 1024;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
 // ---- per-device state --------------------------------------------------------------------------
 struct SplitWorkspace {
     float* partial = nullptr;            // [slices][N] fp32 records of the VM kernel; every word kVmEmpty between launches
@@ -61,6 +73,11 @@ struct DeviceState {
     bool seq_launched = false;
     hipStream_t seq_stream = nullptr;
     hipEvent_t seq_event = nullptr;
+    // pimhip_execute_gemv_static: this device's copy of `scratch` (every word kVmEmpty between launches) and the pinned
+    // host word its kernel sets when a wait gives up, both set up by pimhip_initialize.
+    float* static_partial = nullptr;
+    unsigned int* static_status = nullptr;
+    unsigned int* static_status_dev = nullptr;
 };
 
 std::mutex g_mutex;
@@ -155,8 +172,38 @@ int gemv_mv(const half_t* W, const half_t* x, const half_t* bias, half_t* y, int
 // microseconds of its producer's last load).
 constexpr unsigned int kVmSpinLimit = 1u << 22;
 
+// The records of the static scratch array instead of the stream's workspace: nothing is allocated, freed or
+// synchronised (pimhip_execute_gemv_static).
+int get_static_workspace(DeviceState* st, hipStream_t stream, size_t partial_elems, float** partial, unsigned int** status)
+{
+    if (!st->static_partial || !st->static_status)
+        return fail(PIMHIP_ERR_NOT_INITIALIZED, "the static scratch buffer of this device has not been set up");
+    if (partial_elems > kStaticScratchFloats)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "this I_X_W product needs %zu partial sums, the static scratch buffer holds %zu: "
+                                            "use pimhip_execute_gemv", partial_elems, kStaticScratchFloats);
+    if (*st->static_status != 0u) {
+        // An earlier launch gave up a wait and may have left records behind: bring every word back to kVmEmpty with
+        // a fill kernel on this stream (a caller may be recording a graph, which must hold no memset), launch nothing
+        // else.  The word is cleared first: the launch that set it has ended, or the caller's calls overlap.
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        PIMHIP_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
+        if (capture != hipStreamCaptureStatusNone)
+            return fail(PIMHIP_ERR_UNSUPPORTED, "an earlier static GEMV gave up a wait; its recovery is not for a graph");
+        PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
+        *st->static_status = 0u;
+        fill_u32_kernel<<<(unsigned)(kStaticScratchFloats / 256), 256, 0, stream>>>(reinterpret_cast<unsigned int*>(st->static_partial),
+                                                                                   kStaticScratchFloats, kVmEmpty);
+        PIMHIP_HIP_CHECK(hipGetLastError());
+        return fail(PIMHIP_ERR_TIMEOUT, "an earlier static GEMV gave up waiting for partial sums; its result is undefined "
+                                        "(the scratch buffer has been re-initialised, this call was not launched)");
+    }
+    *partial = st->static_partial;
+    *status = st->static_status_dev;
+    return PIMHIP_OK;
+}
+
 int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bias, const GemvOuts& outs, int64_t K,
-            int64_t N, int64_t lda, int relu, hipStream_t s)
+            int64_t N, int64_t lda, int relu, hipStream_t s, bool static_ws = false)
 {
     bool vec_ok = (N % 8 == 0) && (lda % 8 == 0) && aligned16(A);
     for (int o = 0; o < outs.count; ++o) vec_ok = vec_ok && aligned16(outs.y[o]);
@@ -186,14 +233,23 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     if (k_per_slice < GROUPS) k_per_slice = GROUPS;  // K == 0: one empty slice, y = act(bias)
     slices = (int)((K + k_per_slice - 1) / k_per_slice);
     if (slices < 1) slices = 1;
-    SplitWorkspace* ws = nullptr;
     float* partial = nullptr;
     unsigned int* status = nullptr;
     if (slices > 1) {
-        int rc = get_split_workspace(st, s, (size_t)slices * (size_t)N, &ws);
+        // Records of all slices but the last: partial[slice][N].
+        const size_t partial_elems = (size_t)(slices - 1) * (size_t)N;
+        int rc;
+        if (static_ws) {
+            rc = get_static_workspace(st, s, partial_elems, &partial, &status);
+        } else {
+            SplitWorkspace* ws = nullptr;
+            rc = get_split_workspace(st, s, partial_elems, &ws);
+            if (rc == PIMHIP_OK) {
+                partial = ws->partial;
+                status = ws->status_dev;
+            }
+        }
         if (rc != PIMHIP_OK) return rc;
-        partial = ws->partial;
-        status = ws->status_dev;
     }
     dim3 grid(col_blocks, slices);
     gemv_vm_f16_kernel<WAVES, U, LPR><<<grid, WAVES * 64, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu,
@@ -225,8 +281,23 @@ extern "C" int pimhip_initialize(int device)
     PIMHIP_HIP_CHECK(hipSetDevice(device));
     std::lock_guard<std::mutex> lock(g_mutex);
     DeviceState& st = g_devices[device];
-    st.initialized = true;
+    if (st.initialized) return PIMHIP_OK;
     st.num_cus = prop.multiProcessorCount;
+    // The static scratch array of pimhip_execute_gemv_static: every GPU holds its own copy at its own address, so the
+    // address is looked up with this device current, and the copy starts with every record empty.
+    void* scratch_ptr = nullptr;
+    PIMHIP_HIP_CHECK(hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)));
+    st.static_partial = static_cast<float*>(scratch_ptr);
+    fill_u32_kernel<<<(unsigned)(kStaticScratchFloats / 256), 256, 0, nullptr>>>(reinterpret_cast<unsigned int*>(st.static_partial),
+                                                                                kStaticScratchFloats, kVmEmpty);
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    if (!st.static_status) {
+        PIMHIP_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&st.static_status), sizeof(unsigned int), hipHostMallocMapped));
+        PIMHIP_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&st.static_status_dev), st.static_status, 0));
+    }
+    *st.static_status = 0u;
+    PIMHIP_HIP_CHECK(hipStreamSynchronize(nullptr));
+    st.initialized = true;
     return PIMHIP_OK;
 }
 
@@ -262,8 +333,10 @@ extern "C" int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* o
 // ================================================================================================
 // GEMV family
 // ================================================================================================
-extern "C" int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
-                                   int64_t out_w, int64_t ld_weight, int act, int order, void* stream)
+namespace
+{
+int execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w, int64_t out_w,
+                 int64_t ld_weight, int act, int order, void* stream, bool static_ws)
 {
     DeviceState* st = nullptr;
     int rc = current_device_state(&st);
@@ -287,11 +360,24 @@ extern "C" int pimhip_execute_gemv(void* out, const void* in, const void* weight
         memset(&outs, 0, sizeof(outs));
         outs.y[0] = (half_t*)out;
         outs.count = 1;
-        rc = gemv_vm(st, (const half_t*)in, (const half_t*)weight, (const half_t*)bias, outs, in_w, out_w, ld_weight, relu, s);
+        rc = gemv_vm(st, (const half_t*)in, (const half_t*)weight, (const half_t*)bias, outs, in_w, out_w, ld_weight, relu, s, static_ws);
     }
     if (rc != PIMHIP_OK) return rc;
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
+}
+}  // namespace
+
+extern "C" int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
+                                   int64_t out_w, int64_t ld_weight, int act, int order, void* stream)
+{
+    return execute_gemv(out, in, weight, bias, in_w, out_w, ld_weight, act, order, stream, false);
+}
+
+extern "C" int pimhip_execute_gemv_static(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
+                                          int64_t out_w, int64_t ld_weight, int act, int order, void* stream)
+{
+    return execute_gemv(out, in, weight, bias, in_w, out_w, ld_weight, act, order, stream, true);
 }
 
 extern "C" int pimhip_execute_bmm(void* const* outs, int n_outs, const void* x, const void* A, int64_t k, int64_t n,
@@ -407,12 +493,6 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
 // ================================================================================================
 namespace
 {
-__global__ void fill_u32_kernel(unsigned int* p, size_t n, unsigned int v)
-{
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = v;
-}
-
 // out_p[T, N] = x[T, K] . w_p[N, K]^T + bias_p for p < count (1, or 2 for the two directions of a bidirectional layer).
 int launch_input_projection(int count, float* const* out, const half_t* x, const half_t* const* w, const float* const* bias,
                             int64_t T, int64_t K, int64_t N, hipStream_t s)
@@ -645,6 +725,7 @@ extern "C" int pimhip_deinitialize(void)
             if (w.second.status) hipHostFree(w.second.status);
         }
         kv.second.workspaces.clear();
+        if (kv.second.static_status) hipHostFree(kv.second.static_status);
         if (kv.second.seq_event) hipEventDestroy(kv.second.seq_event);
         kv.second.initialized = false;
     }
