@@ -53,12 +53,13 @@ typedef enum PimHipGemmOrder {
     PIMHIP_W_X_I = 1  /* y[out,1] = A[out,in] . x[in,1]   ("MV") */
 } PimHipGemmOrder;
 
-/* Shape classes of a matrix product.  Mirrors GEMM_TYPE (runtime/include/executor/utils/utils.h:30-36). */
+/* Shape classes of a matrix product.  Same enumerators in the same order, hence the same integers, as GEMM_TYPE
+ * {UNKNOW, VV, MV, VM, MM} (runtime/include/executor/utils/utils.h:30-36). */
 typedef enum PimHipGemmType {
     PIMHIP_GEMM_UNKNOWN = 0,
-    PIMHIP_GEMM_VV = 1,
-    PIMHIP_GEMM_VM = 2,
-    PIMHIP_GEMM_MV = 3,
+    PIMHIP_GEMM_VV = 1, /* vector . vector */
+    PIMHIP_GEMM_MV = 2, /* matrix . vector */
+    PIMHIP_GEMM_VM = 3, /* vector . matrix */
     PIMHIP_GEMM_MM = 4
 } PimHipGemmType;
 

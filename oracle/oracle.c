@@ -193,7 +193,8 @@ int oracle_gemm_broadcast(int64_t* shape1, int* rank1, int64_t* shape2, int* ran
     return 0;
 }
 
-/* GEMM_TYPE values as in pimhip.h: VV 1, VM 2, MV 3, MM 4. utils.cpp:373-396. */
+/* Returns the integer of GEMM_TYPE {UNKNOW, VV, MV, VM, MM} (runtime/include/executor/utils/utils.h:30-36): VV 1, MV 2,
+ * VM 3, MM 4.  utils.cpp:373-396. */
 int oracle_get_gemm_type(const int64_t* self_shape, const int64_t* other_shape)
 {
     if (self_shape[0] == 1 && self_shape[1] == 1 && other_shape[0] == 1 && other_shape[1] == 1) {
@@ -203,8 +204,8 @@ int oracle_get_gemm_type(const int64_t* self_shape, const int64_t* other_shape)
         if (other_shape[2] != 1) other_is_vector++;
         if (other_shape[3] != 1) other_is_vector++;
         if (self_is_vector == 1 && other_is_vector == 1) return 1;
-        if (self_is_vector == 1 && other_is_vector == 2) return 2;
-        if (self_is_vector == 2 && other_is_vector == 1) return 3;
+        if (self_is_vector == 1 && other_is_vector == 2) return 3; /* VM */
+        if (self_is_vector == 2 && other_is_vector == 1) return 2; /* MV */
         return 4;
     }
     return 4;

@@ -88,7 +88,7 @@ def gemm_broadcast(shape1, shape2):
 
 
 def get_gemm_type(self_shape, other_shape):
-    """1 VV, 2 VM, 3 MV, 4 MM."""
+    """GEMM_TYPE as the reference numbers it: 1 VV, 2 MV, 3 VM, 4 MM."""
     return lib().oracle_get_gemm_type((ctypes.c_int64 * 4)(*self_shape), (ctypes.c_int64 * 4)(*other_shape))
 
 

@@ -64,7 +64,7 @@ PIMHIP_ACT_NONE = 0
 PIMHIP_ACT_RELU = 1
 PIMHIP_I_X_W = 0
 PIMHIP_W_X_I = 1
-GEMM_UNKNOWN, GEMM_VV, GEMM_VM, GEMM_MV, GEMM_MM = 0, 1, 2, 3, 4
+GEMM_UNKNOWN, GEMM_VV, GEMM_MV, GEMM_VM, GEMM_MM = 0, 1, 2, 3, 4
 
 _lib = None
 

@@ -43,6 +43,7 @@ def build_pimhip(verbose=True):
 
 
 ATEN_LIB_PATH = os.path.join(PKG_DIR, "_aten_ops_pimhip.so")
+ROCM_HOME = os.environ.get("ROCM_HOME") or os.environ.get("ROCM_PATH") or "/opt/rocm"
 
 
 def build_aten_ops(verbose=True):
@@ -57,9 +58,11 @@ def build_aten_ops(verbose=True):
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-DTORCH_EXTENSION_NAME=_aten_ops_pimhip",
            "-DTORCH_API_INCLUDE_EXTENSION_H"]
+    # c10/hip/HIPStream.h (torch's current stream) pulls in the HIP runtime API headers; host compiler only.
+    cmd += ["-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-I{ROCM_HOME}/include"]
     cmd += [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}"]
     cmd += [os.path.join(cpp, "aten_ops_pimhip.cpp"), os.path.join(cpp, "aten_ops_pybind.cpp"), "-o", ATEN_LIB_PATH]
-    cmd += [f"-L{p}" for p in ce.library_paths()] + ["-lc10", "-ltorch", "-ltorch_cpu", "-ltorch_python"]
+    cmd += [f"-L{p}" for p in ce.library_paths()] + ["-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_python"]
     cmd += [f"-L{PKG_DIR}", "-lpimhip", "-Wl,-rpath,$ORIGIN"] + [f"-Wl,-rpath,{p}" for p in ce.library_paths()]
     if verbose:
         print(" ".join(cmd), flush=True)

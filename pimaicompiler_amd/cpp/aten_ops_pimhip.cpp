@@ -3,6 +3,8 @@
 // the HIP kernels behind the C ABI.  at::Tensor is used for device memory only.
 #include "aten_ops_pimhip.h"
 
+#include <c10/hip/HIPStream.h>
+
 #include <map>
 #include <memory>
 #include <mutex>
@@ -64,6 +66,11 @@ void check(int rc)
     if (rc != PIMHIP_OK) throw NNRuntimeException(std::string("pimhip: ") + pimhip_last_error());
 }
 
+// The stream a call runs on: the caller's, or torch's current stream of the current device when none is given (the
+// null stream unless the caller has made another one current), which is the stream the at::Tensor outputs allocated
+// here belong to.
+void* streamOrCurrent(void* stream) { return stream ? stream : static_cast<void*>(c10::hip::getCurrentHIPStream().stream()); }
+
 void requireHalfOnGpu(const at::Tensor& t, const char* what)
 {
     if (!t.defined()) return;
@@ -96,7 +103,7 @@ at::Tensor gemv(const at::Tensor& x, const at::Tensor& weight2d, const at::Tenso
     if (bc.defined() && bc.numel() != out_w) throw NNRuntimeException("bias length does not match the GEMV output");
     at::Tensor out = at::empty({out_w}, w.options());
     check(pimhip_execute_gemv(out.data_ptr(), xc.data_ptr(), w.data_ptr(), bc.defined() ? bc.data_ptr() : nullptr, in_w,
-                              out_w, ld, act, order, stream));
+                              out_w, ld, act, order, streamOrCurrent(stream)));
     return out;
 }
 
@@ -137,7 +144,7 @@ std::shared_ptr<PlanHolder> planFor(at::TensorList params, bool has_biases, int6
     int64_t cap = seq_len > 16 ? seq_len : 16;
     if (it != g_plans.end() && 2 * it->second->max_seq_len > cap) cap = 2 * it->second->max_seq_len;
     check(pimhip_lstm_plan_create(&holder->plan, ptrs.data(), (int)ptrs.size(), has_biases ? 1 : 0, (int)num_layers,
-                                  bidirectional ? 1 : 0, input_size, hidden, cap, nullptr));
+                                  bidirectional ? 1 : 0, input_size, hidden, cap, streamOrCurrent(nullptr)));
     holder->max_seq_len = cap;
     g_plans[key] = holder;
     return holder;
@@ -162,7 +169,7 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> lstmForward(const at::Tensor& x2d
     at::Tensor hn = at::empty({num_layers * D, 1, H}, x.options());
     at::Tensor cn = at::empty({num_layers * D, 1, H}, x.options());
     check(pimhip_lstm_forward(holder->plan, T > 0 ? x.data_ptr() : nullptr, h0.data_ptr(), c0.data_ptr(),
-                              T > 0 ? y.data_ptr() : nullptr, hn.data_ptr(), cn.data_ptr(), T, nullptr));
+                              T > 0 ? y.data_ptr() : nullptr, hn.data_ptr(), cn.data_ptr(), T, streamOrCurrent(nullptr)));
     return std::make_tuple(y, hn, cn);
 }
 }  // namespace
@@ -296,7 +303,7 @@ void customAtenMatmul(at::Tensor& self_tensor, at::Tensor& other_tensor, torch::
         at::Tensor output = at::empty(output_shape, a.options());
         if (output.numel() != 1 || a.numel() < in_w || b.numel() < in_w)
             throw NNRuntimeException("VV operands do not form a single dot product");
-        check(pimhip_execute_dot(output.data_ptr(), a.data_ptr(), b.data_ptr(), in_w, stream));
+        check(pimhip_execute_dot(output.data_ptr(), a.data_ptr(), b.data_ptr(), in_w, streamOrCurrent(stream)));
         output_iv = torch::jit::IValue(output);
     } else {
         // aten_ops.cpp:883-931: LibTorch passthrough.
@@ -304,10 +311,12 @@ void customAtenMatmul(at::Tensor& self_tensor, at::Tensor& other_tensor, torch::
     }
 }
 
-at::Tensor atenLinear(const at::Tensor& input, const at::Tensor& weight, const at::Tensor& bias)
+at::Tensor atenLinear(const at::Tensor& input, const at::Tensor& weight, const c10::optional<at::Tensor>& bias_opt)
 {
-    // aten_ops.cpp:304-307.  One input row: the MV product on W's own row-major bytes.
-    if (input.numel() != weight.size(1)) return at::linear(input, weight, bias);
+    // aten_ops.cpp:304-307 (declared with the optional bias at aten_ops.h:231).  One input row: the MV product on W's
+    // own row-major bytes, on torch's current stream; anything else is LibTorch's.
+    if (weight.dim() != 2 || input.numel() != weight.size(1)) return at::linear(input, weight, bias_opt);
+    const at::Tensor bias = bias_opt.has_value() ? *bias_opt : at::Tensor();
     requireHalfOnGpu(input, "input");
     requireHalfOnGpu(weight, "weight");
     requireHalfOnGpu(bias, "bias");
@@ -316,8 +325,6 @@ at::Tensor atenLinear(const at::Tensor& input, const at::Tensor& weight, const a
     shape.back() = weight.size(0);
     return y.view(shape);
 }
-
-at::Tensor atenLinear(const at::Tensor& input, const at::Tensor& weight) { return atenLinear(input, weight, at::Tensor()); }
 
 std::tuple<at::Tensor, at::Tensor, at::Tensor> atenLstm1(const at::Tensor& input, at::TensorList hx,
                                                          at::TensorList params, bool has_biases, int64_t num_layers,

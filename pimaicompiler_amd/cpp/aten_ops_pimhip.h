@@ -19,8 +19,14 @@ namespace runtime
 {
 namespace utils
 {
-// runtime/include/executor/utils/utils.h:30-36
-enum class GEMM_TYPE { UNKNOW = 0, VV, VM, MV, MM };
+// runtime/include/executor/utils/utils.h:30-36: a plain enum, enumerators in this order (MV = 2, VM = 3).
+enum GEMM_TYPE {
+    UNKNOW,
+    VV,  // Vector * Vector
+    MV,  // Matrix * Vector
+    VM,  // Vector * Matrix
+    MM   // Matrix * Matrix
+};
 
 // runtime/include/executor/utils/utils.h:166-176
 class NNRuntimeException : public std::runtime_error
@@ -46,8 +52,7 @@ void customAtenAddmm(std::string act_type, at::Tensor& self_tensor, at::Tensor& 
 void customAtenMatmul(at::Tensor& self_tensor, at::Tensor& other_tensor, torch::jit::IValue& output_iv,
                       void* stream = nullptr);
 
-at::Tensor atenLinear(const at::Tensor& input, const at::Tensor& weight, const at::Tensor& bias);
-at::Tensor atenLinear(const at::Tensor& input, const at::Tensor& weight);
+at::Tensor atenLinear(const at::Tensor& input, const at::Tensor& weight, const c10::optional<at::Tensor>& bias = {});
 
 std::tuple<at::Tensor, at::Tensor, at::Tensor> atenLstm1(const at::Tensor& input, at::TensorList hx,
                                                          at::TensorList params, bool has_biases, int64_t num_layers,

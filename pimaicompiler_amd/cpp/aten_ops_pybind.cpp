@@ -32,7 +32,7 @@ PYBIND11_MODULE(_aten_ops_pimhip, m)
         return out.toTensor();
     });
     m.def("atenLinear", [](const at::Tensor& x, const at::Tensor& w, const c10::optional<at::Tensor>& b) {
-        return b.has_value() ? ops::atenLinear(x, w, *b) : ops::atenLinear(x, w);
+        return ops::atenLinear(x, w, b);
     });
     m.def("atenLstm1", [](const at::Tensor& input, std::vector<at::Tensor> hx, std::vector<at::Tensor> params, bool has_biases,
                           int64_t num_layers, double dropout, bool train, bool bidirectional, bool batch_first) {

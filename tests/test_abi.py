@@ -39,7 +39,7 @@ def test_enums_match_header():
     for name, value in [("PIMHIP_OK", 0), ("PIMHIP_ERR_INVALID_ARGUMENT", 1), ("PIMHIP_ERR_UNSUPPORTED", 2),
                         ("PIMHIP_ERR_HIP", 3), ("PIMHIP_ERR_NOT_INITIALIZED", 4), ("PIMHIP_ERR_TIMEOUT", 5),
                         ("PIMHIP_ACT_RELU", 1), ("PIMHIP_I_X_W", 0), ("PIMHIP_W_X_I", 1), ("PIMHIP_GEMM_VV", 1),
-                        ("PIMHIP_GEMM_VM", 2), ("PIMHIP_GEMM_MV", 3), ("PIMHIP_GEMM_MM", 4)]:
+                        ("PIMHIP_GEMM_MV", 2), ("PIMHIP_GEMM_VM", 3), ("PIMHIP_GEMM_MM", 4)]:
         assert re.search(rf"\b{name}\s*=\s*{value}\b", text), name
         assert getattr(L, name, getattr(L, name.replace("PIMHIP_", ""), value)) == value
 
@@ -116,3 +116,31 @@ def test_dispatch_classes_of_known_call_sites(mat1, mat2, kind):
     out = ctypes.c_int(-1)
     L.load().pimhip_get_gemm_type((ctypes.c_int64 * 4)(*a), (ctypes.c_int64 * 4)(*b), ctypes.byref(out))
     assert out.value == kind
+
+
+# ---- the product's shape logic against sources that do not restate it --------------------------------------------
+def _abi_broadcast(s1, s2):
+    rc, o1, o2 = _product_broadcast(s1, s2)
+    if rc == L.PIMHIP_OK:
+        return "ok", o1, o2
+    if rc == L.PIMHIP_ERR_UNSUPPORTED:
+        return "short", o1, o2
+    return "abort", None, None
+
+
+def _abi_type(o1, o2):
+    from shape_cases import TYPE_NAMES
+    out = ctypes.c_int(-1)
+    assert L.load().pimhip_get_gemm_type((ctypes.c_int64 * 4)(*o1), (ctypes.c_int64 * 4)(*o2), ctypes.byref(out)) == 0
+    return TYPE_NAMES[out.value]
+
+
+def test_product_shape_logic_matches_the_hand_traced_table():
+    from shape_cases import check_hand_traced
+    check_hand_traced(_abi_broadcast, _abi_type, undefined_may_refuse=True)
+
+
+def test_product_shape_logic_agrees_with_the_meaning_of_the_product():
+    from shape_cases import check_matmul_semantics
+    n_checked, n_as_product, exceptions = check_matmul_semantics(_abi_broadcast, _abi_type)
+    assert n_checked > 600 and n_as_product > 550

@@ -47,6 +47,32 @@ def test_cpp_shape_logic_matches_oracle(cpp):
     assert checked > 1000
 
 
+def test_cpp_shape_logic_matches_the_hand_traced_table(cpp):
+    """utils::gemmBroadcast / getGemmType of the C++ layer on tests/golden/shape_logic_cases.json; getGemmType returns the
+    reference's own integers (GEMM_TYPE is a plain enum there: VV 1, MV 2, VM 3, MM 4)."""
+    from shape_cases import TYPE_NAMES, check_hand_traced
+
+    def broadcast(s1, s2):
+        try:
+            o1, o2 = cpp.gemmBroadcast(list(s1), list(s2))
+        except Exception as e:
+            # the C++ layer throws where the reference would go on with a rank other than 4, abort, or read out of range
+            return ("short" if "stay at ranks" in str(e) else "abort"), None, None
+        return "ok", o1, o2
+
+    n_ok = 0
+    from shape_cases import hand_traced_cases
+    for c in hand_traced_cases():
+        status, o1, o2 = broadcast(c["s1"], c["s2"])
+        if c["status"] == "ok":
+            assert status == "ok" and (o1, o2) == (c["o1"], c["o2"]), c
+            assert TYPE_NAMES[cpp.getGemmType(o1, o2)] == c["type"], c
+            n_ok += 1
+        else:
+            assert status != "ok", c
+    assert n_ok >= 30
+
+
 @pytest.mark.gpu
 def test_cpp_custom_gemv_unit_test(cpp_gpu):
     """custom_op_ut.cpp:20-69 through customAtenMatmul, on seeded inputs scaled so that fp16 rounding of the result
@@ -110,3 +136,36 @@ def test_cpp_lstm_matches_libtorch_cpu(cpp_gpu):
     assert maxabs(y, wy) <= 2e-3 and maxabs(hn, whn) <= 2e-3 and maxabs(cn, wcn) <= 2e-3
     with pytest.raises(Exception):
         cpp_gpu.atenLstm1(x.to(DEV).repeat(1, 2, 1), [h0.to(DEV), c0.to(DEV)], [p.to(DEV) for p in params], True, 1, 0.0, False, True, False)
+
+
+@pytest.mark.gpu
+def test_cpp_ops_run_on_torchs_current_stream(cpp_gpu):
+    """atenLinear / atenLstm1 / customAtenMatmul take no stream argument (or a null one): they must run on the stream
+    that is current in torch, the one their inputs were produced on and their outputs are allocated for.  The side
+    stream is kept busy before the inputs are written; a launch on the null stream would read the inputs too early
+    (torch's side streams do not synchronise with it)."""
+    W, x, b = oracle.gemv_inputs(2101, 1024, 1024)
+    params, xs, h0, c0 = oracle.lstm_inputs(78, 64, 128, 1, False, 9)
+    wy, whn, wcn = oracle.torch_lstm(xs, h0, c0, params, True, 1, False)
+    want = oracle.torch_addmm(b, x, W).reshape(-1)
+    Wd, bd = W.to(DEV), b.to(DEV)
+    pd, h0d, c0d = [p.to(DEV) for p in params], h0.to(DEV), c0.to(DEV)
+    x_src, xs_src = x.to(DEV), xs.to(DEV)
+    xd, xsd = torch.zeros_like(x_src), torch.zeros_like(xs_src)
+    busy = torch.randn(4096, 4096, device=DEV)
+    # warm-up on the default stream: plan creation, workspaces
+    cpp_gpu.atenLstm1(xs_src, [h0d, c0d], pd, True, 1, 0.0, False, False, False)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(30):
+            busy = (busy @ busy) * 1e-3
+        xd.copy_(x_src)
+        xsd.copy_(xs_src)
+        y = cpp_gpu.atenLinear(xd, Wd, bd)
+        ym = cpp_gpu.customAtenMatmul(Wd, xd.t())
+        ys, hn, cn = cpp_gpu.atenLstm1(xsd, [h0d, c0d], pd, True, 1, 0.0, False, False, False)
+    side.synchronize()
+    assert maxabs(y, want) <= 2e-3
+    assert maxabs(ym, want.float() - b.float()) <= 2e-3
+    assert maxabs(ys, wy) <= 5e-3 and maxabs(hn, whn) <= 5e-3 and maxabs(cn, wcn) <= 5e-3

@@ -234,3 +234,31 @@ def test_rnnt_encoder_lstm_on_the_references_feature_file(ops):
     y, hn, cn = ops.aten_lstm1(feat.to(DEV), (h0.to(DEV), c0.to(DEV)), [p.to(DEV) for p in params], True, 2, 0.0, False, False, False)
     assert list(y.shape) == [341, 1, 1024]
     assert maxabs(y, want[0]) <= 5e-3 and maxabs(hn, want[1]) <= 5e-3 and maxabs(cn, want[2]) <= 5e-3
+
+
+def test_matmul_dispatch_on_the_hand_traced_shape_table(ops):
+    """Every case of tests/golden/shape_logic_cases.json that is a valid product and that the reference classifies:
+    custom_aten_matmul takes the branch the table names (VV / VM / MV through the HIP kernels, MM through LibTorch) and
+    in each of them the values are the product's (max abs error <= 2e-3 against the float64 product of the fp16
+    inputs, the GEMV tolerance), with as many elements as torch.matmul yields."""
+    from shape_cases import hand_traced_cases
+    g = torch.Generator().manual_seed(77)
+    taken = set()
+    for c in hand_traced_cases():
+        if c["status"] != "ok":
+            continue
+        a = (torch.rand(*c["s1"], generator=g) - 0.5).half()
+        b = (torch.rand(*c["s2"], generator=g) * 0.05).half()
+        try:
+            want = torch.matmul(a.double(), b.double())
+        except RuntimeError:
+            continue  # the heuristic pads shapes that form no product; nothing to compute
+        s1, s2 = ops.gemm_broadcast(c["s1"], c["s2"])
+        assert (s1, s2) == (c["o1"], c["o2"])
+        assert ops.get_gemm_type(s1, s2).name == c["type"]
+        out = ops.custom_aten_matmul(a.to("cuda:0"), b.to("cuda:0"))
+        assert out.numel() == want.numel(), (c["s1"], c["s2"], list(out.shape))
+        err = float((out.double().cpu().reshape(-1) - want.reshape(-1)).abs().max())
+        assert err <= 2e-3, (c["s1"], c["s2"], err)
+        taken.add(c["type"])
+    assert taken == {"VV", "VM", "MV", "MM"}

@@ -280,3 +280,39 @@ def test_lstm_pack_layout_and_round_trip():
         back = oracle.lstm_unpack_miopen(buf, [p.shape for p in params], has_b, L, D == 2)
         for a, b in zip(params, back):
             assert np.array_equal(a, b)
+
+
+# ---- shape logic -----------------------------------------------------------------------------------------------
+def _oracle_broadcast(s1, s2):
+    rc, o1, o2 = oracle.gemm_broadcast(s1, s2)
+    if rc == 1:
+        return "abort", None, None
+    if rc == 2:
+        return "out_of_range", None, None
+    return ("ok" if len(o1) == 4 and len(o2) == 4 else "short"), o1, o2
+
+
+def _oracle_type(o1, o2):
+    from shape_cases import TYPE_NAMES
+    return TYPE_NAMES[oracle.get_gemm_type(o1, o2)]
+
+
+def test_shape_logic_matches_the_hand_traced_table():
+    """tests/golden/shape_logic_cases.json: traced by hand through utils.cpp:293-396, one or more cases per branch,
+    the reference's unit-test shapes (custom_op_ut.cpp:27-28, 49-50, 76-77, 113-114) among them."""
+    from shape_cases import check_hand_traced, hand_traced_cases
+    check_hand_traced(_oracle_broadcast, _oracle_type)
+    lines = " ".join(c["lines"] for c in hand_traced_cases())
+    for branch in ("299-310", "311-315", "316-317", "320-323", "324-326", "327-329", "331-333", "335-339", "340-341",
+                   "345-346", "347-348", "351-352", "353-354", "356-361", "362-365", "383-384", "385-386", "387-388",
+                   "389-391", "392-394"):
+        assert branch in lines, branch
+
+
+def test_shape_logic_agrees_with_the_meaning_of_the_product():
+    """Independent of the source's structure: class, element counts and padded shapes follow from the real matrix
+    product wherever torch.matmul accepts the pair; the exceptions are the ones the source's lines produce."""
+    from shape_cases import check_matmul_semantics
+    n_checked, n_as_product, exceptions = check_matmul_semantics(_oracle_broadcast, _oracle_type)
+    assert n_checked > 600 and n_as_product > 550
+    assert exceptions["square_behind_rank4_row"] == 12 and exceptions["rank1_rank1"] == 3 and exceptions["rank1_leading_match"] == 12
