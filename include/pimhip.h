@@ -175,8 +175,11 @@ int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan);
 int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn,
                         void* cn, int64_t seq_len, void* stream);
 
-/* After the stream has been synchronised: 0 if every persistent-kernel wait in the last forward of this plan
- * completed, PIMHIP_ERR_TIMEOUT if a bounded wait gave up (the outputs are then undefined). */
+/* After the stream has been synchronised: 0 if every persistent-kernel wait in the forwards of this plan so far
+ * completed, PIMHIP_ERR_TIMEOUT if a bounded wait gave up (the outputs of that forward are undefined).  A time-out is
+ * reported exactly once: by this call, or else by the next pimhip_lstm_forward of the plan, which then returns
+ * PIMHIP_ERR_TIMEOUT after synchronising its stream and launches nothing.  The forward after the report re-initialises
+ * the plan's exchange buffer and runs normally. */
 int pimhip_lstm_plan_status(PimHipLstmPlan* plan);
 
 /* Upper bound on the polls of one wait inside the persistent kernel (default 2^22, roughly seconds).  A wait

@@ -25,4 +25,6 @@ from .ops import (  # noqa: F401
     input_projection_packed,
     pack_projection_weight,
     LstmPlan,
+    prepare_lstm,
+    invalidate_lstm_plans,
 )

@@ -110,15 +110,24 @@ at::Tensor gemv(const at::Tensor& x, const at::Tensor& weight2d, const at::Tenso
 struct PlanHolder {
     PimHipLstmPlan* plan = nullptr;
     int64_t max_seq_len = 0;
-    std::vector<at::Tensor> params;  // keeps the weights alive
+    std::vector<at::Tensor> params;     // what the plan reads: contiguous, kept alive
+    std::vector<at::Tensor> originals;  // the caller's tensors: their addresses cannot be reused while the entry lives
+    std::vector<uint32_t> versions;     // their version counters when the plan was made
+    uint64_t last_use = 0;
     ~PlanHolder()
     {
         if (plan) pimhip_lstm_plan_destroy(plan);
     }
 };
 
+// Plans found again by their weights.  A plan holds values derived from the weights (b_ih + b_hh, w_ih in matrix-core
+// order, contiguous copies): an in-place update of a weight (seen through its version counter) makes the entry stale
+// and the next call builds a new plan; updates torch does not count need pimhipInvalidateLstmPlans.  At most
+// kMaxCachedPlans entries; the least recently used one goes first.
+constexpr size_t kMaxCachedPlans = 64;
 std::mutex g_plan_mutex;
 std::map<std::vector<const void*>, std::shared_ptr<PlanHolder>> g_plans;
+uint64_t g_plan_clock = 0;
 
 std::shared_ptr<PlanHolder> planFor(at::TensorList params, bool has_biases, int64_t num_layers, bool bidirectional,
                                     int64_t seq_len)
@@ -128,11 +137,24 @@ std::shared_ptr<PlanHolder> planFor(at::TensorList params, bool has_biases, int6
     key.push_back(reinterpret_cast<const void*>((uintptr_t)((has_biases ? 1 : 0) | (bidirectional ? 2 : 0) | (num_layers << 2))));
     std::lock_guard<std::mutex> lock(g_plan_mutex);
     auto it = g_plans.find(key);
-    if (it != g_plans.end() && it->second->max_seq_len >= seq_len) return it->second;
+    if (it != g_plans.end()) {
+        bool fresh = it->second->versions.size() == params.size();
+        for (size_t i = 0; fresh && i < params.size(); ++i) fresh = it->second->versions[i] == params[i]._version();
+        if (!fresh) {
+            g_plans.erase(it);
+            it = g_plans.end();
+        }
+    }
+    if (it != g_plans.end() && it->second->max_seq_len >= seq_len) {
+        it->second->last_use = ++g_plan_clock;
+        return it->second;
+    }
     auto holder = std::make_shared<PlanHolder>();
     std::vector<const void*> ptrs;
     for (const at::Tensor& p : params) {
         requireHalfOnGpu(p, "LSTM parameter");
+        holder->originals.push_back(p);
+        holder->versions.push_back(p._version());
         holder->params.push_back(p.contiguous());
         ptrs.push_back(holder->params.back().data_ptr());
     }
@@ -146,7 +168,14 @@ std::shared_ptr<PlanHolder> planFor(at::TensorList params, bool has_biases, int6
     check(pimhip_lstm_plan_create(&holder->plan, ptrs.data(), (int)ptrs.size(), has_biases ? 1 : 0, (int)num_layers,
                                   bidirectional ? 1 : 0, input_size, hidden, cap, streamOrCurrent(nullptr)));
     holder->max_seq_len = cap;
+    holder->last_use = ++g_plan_clock;
     g_plans[key] = holder;
+    while (g_plans.size() > kMaxCachedPlans) {
+        auto oldest = g_plans.begin();
+        for (auto jt = g_plans.begin(); jt != g_plans.end(); ++jt)
+            if (jt->second->last_use < oldest->second->last_use) oldest = jt;
+        g_plans.erase(oldest);  // a forward still holding the shared_ptr keeps its plan until it returns
+    }
     return holder;
 }
 
@@ -175,6 +204,29 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> lstmForward(const at::Tensor& x2d
 }  // namespace
 
 void pimhipRuntimeInitialize(int device) { check(pimhip_initialize(device)); }
+
+int64_t pimhipInvalidateLstmPlans(at::TensorList params)
+{
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    if (params.empty()) {
+        const int64_t n = (int64_t)g_plans.size();
+        g_plans.clear();
+        return n;
+    }
+    int64_t n = 0;
+    for (auto it = g_plans.begin(); it != g_plans.end();) {
+        bool hit = false;
+        for (const at::Tensor& o : it->second->originals)
+            for (const at::Tensor& p : params) hit = hit || o.data_ptr() == p.data_ptr();
+        if (hit) {
+            it = g_plans.erase(it);
+            ++n;
+        } else {
+            ++it;
+        }
+    }
+    return n;
+}
 
 void pimhipRuntimeDeinitialize()
 {

@@ -46,6 +46,12 @@ namespace op_executor
 void pimhipRuntimeInitialize(int device);
 void pimhipRuntimeDeinitialize();
 
+// atenLstm1/2 keep one prepared plan per set of weight tensors (the place of the packed MIOpen buffer the reference's
+// ModelBuilder builds once, runtime/source/builder/model_builder.cpp:226-319).  A plan is rebuilt when torch's
+// version counter of a weight has moved; weights changed behind torch's back need this call, which drops the plans
+// made from any of `params` (all plans for an empty list) and returns how many it dropped.
+int64_t pimhipInvalidateLstmPlans(at::TensorList params);
+
 void customAtenAddmm(std::string act_type, at::Tensor& self_tensor, at::Tensor& mat1_tensor, at::Tensor& mat2_tensor,
                      at::Scalar beta, at::Scalar alpha, torch::jit::IValue& output_iv, void* stream = nullptr);
 

@@ -13,6 +13,7 @@ PYBIND11_MODULE(_aten_ops_pimhip, m)
 {
     m.def("initialize", &ops::pimhipRuntimeInitialize);
     m.def("deinitialize", &ops::pimhipRuntimeDeinitialize);
+    m.def("invalidateLstmPlans", [](std::vector<at::Tensor> params) { return ops::pimhipInvalidateLstmPlans(params); });
     m.def("customAtenAddmm", [](const std::string& act, at::Tensor self, at::Tensor mat1, at::Tensor mat2, double beta, double alpha) {
         torch::jit::IValue out;
         ops::customAtenAddmm(act, self, mat1, mat2, beta, alpha, out, nullptr);

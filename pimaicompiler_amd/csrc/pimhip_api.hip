@@ -902,7 +902,13 @@ extern "C" int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned in
 extern "C" int pimhip_lstm_plan_status(PimHipLstmPlan* plan)
 {
     if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
-    if (*plan->abort_host != 0u) return fail(PIMHIP_ERR_TIMEOUT, "a bounded wait of the persistent LSTM kernel gave up");
+    if (*plan->abort_host != 0u) {
+        // Reported once, here or by the next pimhip_lstm_forward, whichever comes first.  The caller has synchronised
+        // the stream, so the kernel that set the word has ended and nothing sets it again after it is cleared.
+        *plan->abort_host = 0u;
+        plan->reset_exchange = true;
+        return fail(PIMHIP_ERR_TIMEOUT, "a bounded wait of the persistent LSTM kernel gave up: the results of that forward are undefined");
+    }
     return PIMHIP_OK;
 }
 
@@ -968,9 +974,18 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     const bool use_seq = T >= 2 && T + kSeqMaxChains <= kSeqMaxT && (plan->mode >= 2 || (plan->mode == 0 && plan->seq_kernel_ok));
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
     if (*plan->abort_host != 0u) {
-        // The previous sequence kernel of this plan timed out (pimhip_lstm_plan_status has had its chance to report it).
+        // An earlier sequence kernel of this plan gave up a wait and nobody has asked pimhip_lstm_plan_status since:
+        // the error is reported here instead of being dropped, and nothing is launched.  The word is cleared only
+        // after the stream has drained (calls sharing a plan are ordered on one stream), so that kernel cannot set
+        // it again; the next forward starts from a re-initialised exchange buffer.
+        if (capturing)
+            return fail(PIMHIP_ERR_UNSUPPORTED, "an earlier forward of this plan gave up a wait; recovering from that is not for a "
+                                                "graph: call pimhip_lstm_plan_status or one forward outside the capture first");
+        PIMHIP_HIP_CHECK(hipStreamSynchronize(s));
         *plan->abort_host = 0u;
         plan->reset_exchange = true;
+        return fail(PIMHIP_ERR_TIMEOUT, "an earlier forward of this plan gave up a wait of the persistent LSTM kernel: its results "
+                                        "are undefined (this call was not launched; the next one starts from a re-initialised exchange buffer)");
     }
     if (use_seq && plan->reset_exchange) {
         // After a time-out or a change of the entry layout: re-arm the flag and bring the exchange buffer and its step

@@ -15,6 +15,7 @@ LSTM runs in libpimhip.so.  True matrix-matrix products take the same LibTorch p
 (atenAddmm / atenMatmul, aten_ops.cpp:47-51,362).  Errors are raised as NNRuntimeException
 (runtime/include/executor/utils/utils.h:166-176) instead of being ignored.
 """
+import collections
 import contextlib
 import ctypes
 import enum
@@ -556,17 +557,46 @@ def _overlap(a, b):
     return a.numel() > 0 and b.numel() > 0 and a0 < b0 + b.numel() * b.element_size() and b0 < a0 + a.numel() * a.element_size()
 
 
-_plan_cache = {}
+# Plans of aten_lstm1/2 calls, found again by their weights.  An entry keeps the caller's own tensors (so their
+# addresses cannot be reused by other weights while it lives) and their version counters: a plan holds values derived
+# from the weights (b_ih + b_hh, w_ih in matrix-core order, contiguous copies), so an in-place update of a weight makes
+# it stale, and the next call builds a new one.  Updates torch does not count (writes through data_ptr from other
+# libraries) need invalidate_lstm_plans.  At most PLAN_CACHE_MAX plans are kept; the least recently used one goes first.
+PLAN_CACHE_MAX = 64
+_plan_cache = collections.OrderedDict()
 
 
 def _plan_for(params, has_biases, num_layers, bidirectional, seq_len):
     key = (tuple(p.data_ptr() for p in params), bool(has_biases), int(num_layers), bool(bidirectional))
-    plan = _plan_cache.get(key)
+    versions = tuple(p._version for p in params)
+    entry = _plan_cache.get(key)
+    if entry is not None and entry[2] != versions:
+        del _plan_cache[key]
+        entry = None
+    plan = entry[0] if entry is not None else None
     if plan is None or plan.max_seq_len < seq_len:
         cap = max(int(seq_len), 2 * plan.max_seq_len if plan is not None else 0, 16)
         plan = LstmPlan(params, has_biases, num_layers, bidirectional, cap)
-        _plan_cache[key] = plan
+        _plan_cache[key] = (plan, list(params), versions)
+    _plan_cache.move_to_end(key)
+    while len(_plan_cache) > PLAN_CACHE_MAX:
+        _plan_cache.popitem(last=False)
     return plan
+
+
+def invalidate_lstm_plans(params=None):
+    """Drops the cached plans that were built from any of the tensors in `params` (all plans when None): call it after
+    changing LSTM weights in a way torch's version counters do not see.  Returns the number of plans dropped.  A plan
+    still referenced elsewhere (prepare_lstm's return value) lives on; the cache just stops handing it out."""
+    if params is None:
+        n = len(_plan_cache)
+        _plan_cache.clear()
+        return n
+    ptrs = {p.data_ptr() for p in params}
+    stale = [k for k in _plan_cache if ptrs.intersection(k[0])]
+    for k in stale:
+        del _plan_cache[k]
+    return len(stale)
 
 
 def prepare_lstm(params, has_biases, num_layers, bidirectional, max_seq_len=64):

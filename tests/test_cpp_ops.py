@@ -169,3 +169,20 @@ def test_cpp_ops_run_on_torchs_current_stream(cpp_gpu):
     assert maxabs(y, want) <= 2e-3
     assert maxabs(ym, want.float() - b.float()) <= 2e-3
     assert maxabs(ys, wy) <= 5e-3 and maxabs(hn, whn) <= 5e-3 and maxabs(cn, wcn) <= 5e-3
+
+
+@pytest.mark.gpu
+def test_cpp_plan_cache_follows_weight_updates(cpp_gpu):
+    params, x, h0, c0 = oracle.lstm_inputs(126, 64, 128, 1, False, 20)
+    pd = [p.to(DEV) for p in params]
+    args = (x.to(DEV), [h0.to(DEV), c0.to(DEV)], pd, True, 1, 0.0, False, False, False)
+    y0 = cpp_gpu.atenLstm1(*args)[0]
+    assert maxabs(y0, oracle.torch_lstm(x, h0, c0, params, True, 1, False)[0]) <= 2e-3
+    params2 = [p.clone() for p in params]
+    params2[0] = (params2[0] * 0.5).half()
+    params2[3] = (params2[3] - 0.25).half()
+    pd[0].copy_(params2[0].to(DEV))
+    pd[3].copy_(params2[3].to(DEV))
+    y1 = cpp_gpu.atenLstm1(*args)[0]
+    assert maxabs(y1, oracle.torch_lstm(x, h0, c0, params2, True, 1, False)[0]) <= 2e-3
+    assert cpp_gpu.invalidateLstmPlans(pd) == 1 and cpp_gpu.invalidateLstmPlans(pd) == 0

@@ -59,6 +59,9 @@ CASES = [  # I, H, L, bidirectional, T, biases
     # 1024 < H <= 2048: the persistent kernel with 32 columns per lane, one layer (or two directions) per launch
     (32, 2048, 1, False, 5, True), (16, 1536, 2, False, 4, True), (24, 2048, 2, True, 3, True), (8, 1040, 3, False, 6, False),
     (8, 2056, 1, False, 3, True),
+    # layer 1 of a bidirectional stack at 65 <= T <= 256 with a 2048-wide input: the packed projection with
+    # eight wavefronts per block and 32-column tiles
+    (64, 1024, 2, True, 70, True),
 ]
 
 
@@ -283,6 +286,59 @@ def test_persistent_kernel_wait_gives_up_and_reports(ops):
     assert maxabs(y, want[0]) <= 2e-3
 
 
+def test_a_timeout_nobody_asked_about_is_raised_by_the_next_call(ops):
+    """aten_lstm1 never calls status(): a wait that gave up (forced from the host with a spin limit of 0; the kernel
+    still runs to its end) must make the NEXT call on those weights raise instead of vanishing, exactly once; the call
+    after that starts from a re-initialised exchange buffer and is right again."""
+    params, x, h0, c0 = oracle.lstm_inputs(124, 64, 1024, 1, False, 30)
+    pd = [p.to(DEV) for p in params]
+    xd, hx = x.to(DEV), (h0.to(DEV), c0.to(DEV))
+    plan = ops.prepare_lstm(pd, True, 1, False, 30)
+    plan.set_mode(2)
+    plan.set_spin_limit(0)
+    ops.aten_lstm1(xd, hx, pd, True, 1, 0.0, False, False, False)     # gives up inside the kernel, returns normally
+    torch.cuda.synchronize()
+    plan.set_spin_limit(1 << 22)
+    with pytest.raises(ops.NNRuntimeException, match="gave up a wait"):
+        ops.aten_lstm1(xd, hx, pd, True, 1, 0.0, False, False, False)
+    y, hn, cn = ops.aten_lstm1(xd, hx, pd, True, 1, 0.0, False, False, False)
+    plan.status()
+    want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
+    assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
+    ops.invalidate_lstm_plans(pd)
+
+
+def test_plan_cache_follows_weight_updates_and_is_bounded(ops):
+    """A cached plan holds values derived from the weights (the summed biases, w_ih in matrix-core order): an in-place
+    update seen by torch's version counter gives a new plan, invalidate_lstm_plans drops plans on request, and the cache
+    never holds more than PLAN_CACHE_MAX plans."""
+    from pimaicompiler_amd import ops as O
+    params, x, h0, c0 = oracle.lstm_inputs(125, 64, 128, 1, False, 20)
+    pd = [p.to(DEV) for p in params]
+    xd, hx = x.to(DEV), (h0.to(DEV), c0.to(DEV))
+    y0 = ops.aten_lstm1(xd, hx, pd, True, 1, 0.0, False, False, False)[0]
+    assert maxabs(y0, oracle.torch_lstm(x, h0, c0, params, True, 1, False)[0]) <= 2e-3
+    plan0 = O._plan_for(pd, True, 1, False, 20)
+    # in-place update of w_ih (packed copy) and b_ih (summed bias): both live in the plan, not in the caller's tensors
+    params2 = [p.clone() for p in params]
+    params2[0] = (params2[0] * 0.5).half()
+    params2[2] = (params2[2] + 0.25).half()
+    pd[0].copy_(params2[0].to(DEV))
+    pd[2].copy_(params2[2].to(DEV))
+    y1 = ops.aten_lstm1(xd, hx, pd, True, 1, 0.0, False, False, False)[0]
+    assert O._plan_for(pd, True, 1, False, 20) is not plan0
+    assert maxabs(y1, oracle.torch_lstm(x, h0, c0, params2, True, 1, False)[0]) <= 2e-3
+    assert ops.invalidate_lstm_plans(pd) == 1 and ops.invalidate_lstm_plans(pd) == 0
+    # bound
+    keep = []
+    for i in range(O.PLAN_CACHE_MAX + 3):
+        prm, *_ = oracle.lstm_inputs(300 + i, 8, 8, 1, False, 2)
+        keep.append([p.to(DEV) for p in prm])
+        O._plan_for(keep[-1], True, 1, False, 2)
+    assert len(O._plan_cache) == O.PLAN_CACHE_MAX
+    assert ops.invalidate_lstm_plans() == O.PLAN_CACHE_MAX
+
+
 @pytest.mark.parametrize("mode", [2, 3])
 def test_persistent_kernel_survives_a_nan_input(ops, mode):
     """A NaN cannot carry the exchange's flag bit, so it is exchanged as 0; the cell state keeps it, and y is NaN from
@@ -301,7 +357,8 @@ def test_persistent_kernel_survives_a_nan_input(ops, mode):
 
 # ---- input projection (the MFMA kernel) against fp32 torch on the host ---------------------------------------------
 @pytest.mark.parametrize("T,K,N", [(1, 8, 16), (5, 24, 40), (16, 32, 16), (17, 40, 100), (50, 1024, 4096), (50, 2048, 4096),
-                                   (200, 240, 4096), (200, 1024, 4096), (341, 240, 4096), (700, 64, 256)])
+                                   (200, 240, 4096), (200, 1024, 4096), (341, 240, 4096), (700, 64, 256),
+                                   (200, 2048, 4096), (130, 4096, 256), (70, 2048, 520)])
 def test_input_projection_matches_fp32_matmul(ops, T, K, N):
     g = torch.Generator().manual_seed(T + K + N)
     x = torch.randn(T, K, generator=g).half()
