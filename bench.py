@@ -163,7 +163,8 @@ def main():
     progress("sweep timed")
     # ---- LSTM: RNNT-style 2 layers, I=240, H=1024, T=200 (400 layer-steps per call) ------------------------------
     from oracle import oracle  # seeded inputs only; the oracle's arithmetic is not called here
-    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    from pimaicompiler_amd import workloads
+    params, x, h0, c0 = workloads.lstm_inputs(3001, 240, 1024, 2, False, 200)
     lstm = {"persistent": None, "per_step_launches": None}
     for mode, name in ((2, "persistent"), (1, "per_step_launches")) if "lstm" in sections else ():
         plan = P.LstmPlan([p.to(dev) for p in params], True, 2, False, 200)
@@ -245,7 +246,7 @@ def main():
         gn = []
         seq = torch.randn(50, 1024, device=dev).half()
         for li, (in_w, bidir) in enumerate([(1024, True), (2048, False), (1024, False), (1024, False)]):
-            prm, _, h0g, c0g = oracle.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
+            prm, _, h0g, c0g = workloads.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
             gn.append((P.LstmPlan([q.to(dev) for q in prm], True, 1, bidir, 50), h0g.to(dev), c0g.to(dev)))
 
         def gnmt_stack():
@@ -257,7 +258,7 @@ def main():
         # the same four calls (eight launches) replayed from a HIP graph
         other["gnmt_lstm_stack_us_per_layer_step_hip_graph"] = round(graph_timed_us(lambda _s: gnmt_stack(), 1) / 250, 3)
         # one decoder step (seq_len 1, I = H = 1024): the fused step kernel, W_ih and W_hh streamed once (16.8 MB)
-        prm, _, h0d, c0d = oracle.lstm_inputs(4101, 1024, 1024, 1, False, 1)
+        prm, _, h0d, c0d = workloads.lstm_inputs(4101, 1024, 1024, 1, False, 1)
         plan_d = P.LstmPlan([q.to(dev) for q in prm], True, 1, False, 1)
         xd1, h0d, c0d = torch.randn(1, 1024, device=dev).half(), h0d.to(dev).contiguous(), c0d.to(dev).contiguous()
         yd1, hnd, cnd = torch.empty(1024, dtype=torch.float16, device=dev), torch.empty_like(h0d), torch.empty_like(c0d)

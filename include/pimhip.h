@@ -210,6 +210,56 @@ int pimhip_pack_projection_weight(void* packed, const void* w, int64_t in_w, int
 int pimhip_input_projection_packed(void* out, const void* x, const void* packed, const void* bias, int64_t seq_len,
                                    int64_t in_w, int64_t n_out, void* stream);
 
+/* ---- decoder step ---------------------------------------------------------------------------- */
+
+typedef struct PimHipDecoderPlan PimHipDecoderPlan;
+
+/* One launch for one step of a GNMT-style decoder stack.  Replaces, for that step, the chain of operator calls the
+ * reference's interpreter makes in its decoder loop: executeAtenLSTM1 with seq_len == 1 once per layer
+ * (aten_ops_executor.cpp:2135-2307; miopen_ops_executor.cpp:170-228 for where hy / cy / out land), executeAtenBmm for the
+ * attention context (aten_ops_executor.cpp:668-747), executeAtenAdd for the residual sums (aten_ops_executor.cpp:43-179)
+ * and executeAtenAddmm for the classifier (aten_ops_executor.cpp:181-216):
+ *
+ *     ctx    = att[1, S] . enc[S, H]                               (or ctx_in)
+ *     y_0    = lstm_0(x)            or lstm_0(cat(x, ctx)) when first_takes_context
+ *     y_k    = lstm_k(cat(in_k, ctx)),  in_1 = out_0, in_{k+1} = out_k          (k >= 1)
+ *     out_k  = y_k + in_k  for k >= first_residual_layer (in_0 = x), else y_k
+ *     logits = classifier_w[vocab, H] . out_last + classifier_b                 (when classifier_w is given)
+ *
+ * The whole GNMT decoder step is (4 layers, first_takes_context 0, first_residual_layer 2, classifier); where other
+ * operators sit between layer 0 and the context (the attention scores), layer 0 stays a pimhip_lstm_forward call and
+ * the rest of the step is a plan with (3 layers, first_takes_context 1, first_residual_layer 1).
+ *   params: host array of device pointers in LibTorch order per layer (w_ih [4H, in_w], w_hh [4H, H], then b_ih, b_hh
+ *           [4H] when has_biases), gate order (i, f, g, o); in_w = input_size for a plain first layer, 2H for every layer
+ *           that takes cat(in, ctx).  num_layers 1..4, hidden_size a multiple of 8 up to 1024, input_size a multiple
+ *           of 8 (== hidden_size when first_takes_context or first_residual_layer == 0).
+ * The plan keeps the weight pointers (they must outlive it), pre-adds the biases and owns a small exchange buffer.
+ * Runs on `stream` and synchronises it. */
+int pimhip_decoder_plan_create(PimHipDecoderPlan** plan, const void* const* params, int n_params, int has_biases,
+                               int num_layers, int first_takes_context, int first_residual_layer, int64_t input_size,
+                               int64_t hidden_size, const void* classifier_w, const void* classifier_b, int64_t vocab,
+                               void* stream);
+
+int pimhip_decoder_plan_destroy(PimHipDecoderPlan* plan);
+
+/* One step.  x [input_size]; att [enc_len] and enc [enc_len, H] (row-major, dense), or ctx_in [H] instead of both;
+ * h_prev, c_prev, hn, cn, layer_outs: host arrays of num_layers device pointers to [H] vectors (the rows of a state
+ * buffer, for instance); layer_outs, or any entry of it, may be NULL, otherwise entry k receives out_k; the context is
+ * also stored to the n_ctx_outs (0..4) buffers of ctx_outs; logits [vocab].  hn[k] / cn[k] may be the buffers
+ * h_prev[k] / c_prev[k] were read from (a one-layer plan without a classifier excepted); no other output may alias an
+ * input.  All blocks of the launch have to be resident at once, so the call is ordered like a sequence call of
+ * pimhip_lstm_forward against the device's other such launches, and steps sharing a plan must be ordered on one stream.
+ * Records one kernel.  Every wait inside is bounded: see pimhip_decoder_plan_status. */
+int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const void* att, const void* enc, int64_t enc_len,
+                        const void* ctx_in, const void* const* h_prev, const void* const* c_prev, void* const* hn,
+                        void* const* cn, void* const* layer_outs, void* const* ctx_outs, int n_ctx_outs, void* logits,
+                        void* stream);
+
+/* As pimhip_lstm_plan_status / pimhip_lstm_plan_set_spin_limit: a wait that gave up is reported exactly once, by the
+ * status call (after the stream has been synchronised) or by the next pimhip_decoder_step, which then launches nothing. */
+int pimhip_decoder_plan_status(PimHipDecoderPlan* plan);
+int pimhip_decoder_plan_set_spin_limit(PimHipDecoderPlan* plan, unsigned int spin_limit);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,7 @@ from .ops import (  # noqa: F401
     input_projection_packed,
     pack_projection_weight,
     LstmPlan,
+    DecoderPlan,
     prepare_lstm,
     invalidate_lstm_plans,
 )

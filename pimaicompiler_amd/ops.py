@@ -551,6 +551,114 @@ class LstmPlan:
         return y, hn, cn
 
 
+class DecoderPlan:
+    """One launch per decoder step of a GNMT-style LSTM stack (pimhip_decoder_step): the seq_len-1 cells of every layer,
+    the attention context, the residual sums and the classifier, which the reference's interpreter runs as separate
+    operators (executeAtenLSTM1 / executeAtenBmm / executeAtenAdd / executeAtenAddmm, aten_ops_executor.cpp:2135-2307,
+    668-747, 43-179, 181-216).
+
+    params: LibTorch order per layer (w_ih, w_hh[, b_ih, b_hh]); layer 0 takes x [input_size], or cat(x, ctx) when
+    first_takes_context; every later layer takes cat(in, ctx); layers from first_residual_layer on add their input to
+    their output; classifier = (W [vocab, H], b [vocab] or None) or None."""
+
+    def __init__(self, params, has_biases, num_layers, first_takes_context=False, first_residual_layer=2, classifier=None,
+                 stream=None):
+        lib = L.load()
+        _require_half_cuda(*params)
+        _ensure_init(params[0])
+        self.params = [p.contiguous() for p in params]
+        self.has_biases = bool(has_biases)
+        self.num_layers = int(num_layers)
+        per_cell = 4 if has_biases else 2
+        if len(self.params) != self.num_layers * per_cell:
+            raise NNRuntimeException(f"expected {self.num_layers * per_cell} parameter tensors, got {len(self.params)}")
+        self.hidden = self.params[1].size(1)
+        self.first_takes_context = bool(first_takes_context)
+        self.input_size = self.params[0].size(1) - (self.hidden if self.first_takes_context else 0)
+        for l in range(self.num_layers):
+            in_w = self.input_size + (self.hidden if self.first_takes_context else 0) if l == 0 else 2 * self.hidden
+            w_ih, w_hh = self.params[l * per_cell], self.params[l * per_cell + 1]
+            if tuple(w_ih.shape) != (4 * self.hidden, in_w) or tuple(w_hh.shape) != (4 * self.hidden, self.hidden):
+                raise NNRuntimeException(f"parameter shapes of layer {l} do not match this decoder wiring")
+        self.device = self.params[0].device
+        self.cls_w = self.cls_b = None
+        self.vocab = 0
+        if classifier is not None:
+            w, b = classifier
+            _require_half_cuda(w, *([b] if b is not None else []))
+            if w.dim() != 2 or w.size(1) != self.hidden or (b is not None and b.numel() != w.size(0)):
+                raise NNRuntimeException("classifier must be W [vocab, H] with an optional bias [vocab]")
+            self.cls_w, self.cls_b = w.contiguous(), (b.contiguous() if b is not None else None)
+            self.vocab = self.cls_w.size(0)
+        n = len(self.params)
+        arr = (ctypes.c_void_p * n)(*[p.data_ptr() for p in self.params])
+        handle = ctypes.c_void_p()
+        _check(lib.pimhip_decoder_plan_create(
+            ctypes.byref(handle), arr, n, int(self.has_biases), self.num_layers, int(self.first_takes_context),
+            int(first_residual_layer), self.input_size, self.hidden, self.cls_w.data_ptr() if self.cls_w is not None else None,
+            self.cls_b.data_ptr() if self.cls_b is not None else None, self.vocab, _stream_handle(stream)))
+        self._handle = handle
+        self._finalizer = weakref.finalize(self, DecoderPlan._destroy, handle.value)
+
+    @staticmethod
+    def _destroy(handle_value):
+        try:
+            L.load().pimhip_decoder_plan_destroy(ctypes.c_void_p(handle_value))
+        except Exception:  # interpreter shutdown
+            pass
+
+    def set_spin_limit(self, limit):
+        _check(L.load().pimhip_decoder_plan_set_spin_limit(self._handle, limit))
+
+    def status(self):
+        """Raises NNRuntimeException if a step's kernel gave up a wait since the last report.  Synchronises."""
+        torch.cuda.synchronize(self.device)
+        _check(L.load().pimhip_decoder_plan_status(self._handle))
+
+    def bind(self, x, h_prev, c_prev, att=None, enc=None, ctx=None, hn=None, cn=None, outs=None, ctx_outs=(), logits=None):
+        """Fixes the buffers of a step (lists of [H] tensors per layer; hn / cn default to h_prev / c_prev, i.e. the state is
+        updated in place) and returns a callable step(stream=None) that launches it without touching Python tensors
+        again: what a decoder loop or a graph capture calls per step."""
+        lib = L.load()
+        n, H = self.num_layers, self.hidden
+        hn = list(h_prev) if hn is None else list(hn)
+        cn = list(c_prev) if cn is None else list(cn)
+        outs = [None] * n if outs is None else list(outs)
+        vecs = [x] + list(h_prev) + list(c_prev) + hn + cn + [o for o in outs if o is not None] + list(ctx_outs)
+        for t in (att, enc, ctx, logits):
+            if t is not None:
+                vecs.append(t)
+        _require_half_cuda(*vecs)
+        for t in vecs:
+            if not t.is_contiguous():
+                raise NNRuntimeException("decoder step buffers must be contiguous")
+        if len(h_prev) != n or len(c_prev) != n or len(hn) != n or len(cn) != n or len(outs) != n:
+            raise NNRuntimeException(f"state lists must have {n} entries")
+        for t in list(h_prev) + list(c_prev) + hn + cn + [o for o in outs if o is not None] + list(ctx_outs) + ([ctx] if ctx is not None else []):
+            if t.numel() != H:
+                raise NNRuntimeException(f"state, output and context vectors must have {H} elements")
+        if x.numel() != self.input_size:
+            raise NNRuntimeException(f"x must have {self.input_size} elements")
+        enc_len = 0
+        if ctx is None and att is not None:
+            enc_len = att.numel()
+            if enc is None or enc.numel() != enc_len * H:
+                raise NNRuntimeException("enc must be [len(att), H]")
+        if self.vocab and (logits is None or logits.numel() != self.vocab):
+            raise NNRuntimeException(f"logits must have {self.vocab} elements")
+        mk = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() if t is not None else None for t in ts])  # noqa: E731
+        a_hp, a_cp, a_hn, a_cn, a_out = mk(h_prev), mk(c_prev), mk(hn), mk(cn), mk(outs)
+        a_ctx = mk(list(ctx_outs)) if ctx_outs else None
+        keep = (vecs, a_hp, a_cp, a_hn, a_cn, a_out, a_ctx)
+        ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+        args = (self._handle, ptr(x), ptr(att), ptr(enc), enc_len, ptr(ctx), a_hp, a_cp, a_hn, a_cn, a_out, a_ctx, len(ctx_outs),
+                ptr(logits))
+
+        def step(stream=None, _keep=keep):
+            _check(lib.pimhip_decoder_step(*args, _stream_handle(stream)))
+        return step
+
+
 def _overlap(a, b):
     """True if the two tensors' storage ranges intersect (both are dense here)."""
     a0, b0 = a.data_ptr(), b.data_ptr()

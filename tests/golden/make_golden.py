@@ -17,6 +17,7 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "..", ".."))
 from oracle import oracle  # noqa: E402
+from pimaicompiler_amd import workloads
 
 torch.set_num_threads(8)
 
@@ -39,7 +40,7 @@ def digest(*tensors):
 def gemv_goldens():
     out = {}
     for name, (seed, n, k) in GEMV_CASES.items():
-        W, x, b = oracle.gemv_inputs(seed, n, k)
+        W, x, b = workloads.gemv_inputs(seed, n, k)
         y = oracle.torch_addmm(b, x, W).reshape(-1)
         out[name + "_inputs_sha256"] = digest(W, x, b)
         if n <= 1024:
@@ -80,7 +81,7 @@ def lstm_tiny_goldens():
         for bidir in (False, True):
             for has_b in (True, False):
                 seed = 7000 + case
-                params, x, h0, c0 = oracle.lstm_inputs(seed, 16, 32, L, bidir, 5, has_b)
+                params, x, h0, c0 = workloads.lstm_inputs(seed, 16, 32, L, bidir, 5, has_b)
                 g = torch.Generator().manual_seed(seed + 500)
                 h0 = (0.5 * torch.randn(h0.shape, generator=g)).half()
                 c0 = (0.5 * torch.randn(c0.shape, generator=g)).half()
@@ -102,7 +103,7 @@ def lstm_tiny_goldens():
 def lstm_large_goldens():
     out = {}
     # C3: RNNT-style, 2 layers unidirectional, I=240, H=1024, T=200.
-    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    params, x, h0, c0 = workloads.lstm_inputs(3001, 240, 1024, 2, False, 200)
     y, hn, cn = oracle.torch_lstm(x, h0, c0, params, True, 2, False)
     out["c3_inputs_sha256"] = digest(x, *params)
     out["c3_hn"] = hn.numpy()
@@ -113,7 +114,7 @@ def lstm_large_goldens():
     g_in = 1024
     seq = None
     for li, (in_w, bidir) in enumerate([(1024, True), (2048, False), (1024, False), (1024, False)]):
-        params, x0, h0, c0 = oracle.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
+        params, x0, h0, c0 = workloads.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
         if seq is None:
             seq = x0
         y, hn, cn = oracle.torch_lstm(seq, h0, c0, params, True, 1, bidir)
@@ -121,7 +122,7 @@ def lstm_large_goldens():
         out[f"c4_l{li}_cn"] = cn.numpy()
         out[f"c4_l{li}_y_samples"] = y.numpy().reshape(50, -1)[::7, ::32]
         seq = y
-    W, _, b = oracle.gemv_inputs(4010, 32000, 1024)
+    W, _, b = workloads.gemv_inputs(4010, 32000, 1024)
     logits = oracle.torch_addmm(b, seq[-1].reshape(1, 1024), W).reshape(-1)
     idx = np.arange(0, 32000, 500)
     out["c4_logits_idx"] = idx

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 
 DEV = "cuda:0"
 
@@ -94,7 +95,7 @@ def test_cpp_custom_gemv_unit_test(cpp_gpu):
 
 @pytest.mark.gpu
 def test_cpp_addmm_matches_libtorch_cpu_and_python_mirror(cpp_gpu, ops):
-    W, x, b = oracle.gemv_inputs(2001, 4096, 4096)
+    W, x, b = workloads.gemv_inputs(2001, 4096, 4096)
     want = oracle.torch_addmm(b, x, W).reshape(-1)
     y = cpp_gpu.customAtenAddmm("none", b.to(DEV), W.to(DEV), x.to(DEV).t(), 1.0, 1.0)
     assert list(y.shape) == [4096, 1] and maxabs(y, want) <= 2e-3
@@ -118,7 +119,7 @@ def test_cpp_addmm_matches_libtorch_cpu_and_python_mirror(cpp_gpu, ops):
 
 @pytest.mark.gpu
 def test_cpp_lstm_matches_libtorch_cpu(cpp_gpu):
-    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    params, x, h0, c0 = workloads.lstm_inputs(3001, 240, 1024, 2, False, 200)
     wy, whn, wcn = oracle.torch_lstm(x, h0, c0, params, True, 2, False)
     pd = [p.to(DEV) for p in params]
     y, hn, cn = cpp_gpu.atenLstm1(x.to(DEV), [h0.to(DEV), c0.to(DEV)], pd, True, 2, 0.0, False, False, False)
@@ -130,7 +131,7 @@ def test_cpp_lstm_matches_libtorch_cpu(cpp_gpu):
                                      pd, True, 2, 0.0, False, False)
     assert list(yp.shape) == [200, 1024] and torch.equal(yp.reshape(-1), y.reshape(-1)) and torch.equal(hnp, hn)
     # bidirectional, one step at a time as the decoders call it
-    params, x, h0, c0 = oracle.lstm_inputs(77, 64, 128, 1, True, 6)
+    params, x, h0, c0 = workloads.lstm_inputs(77, 64, 128, 1, True, 6)
     wy, whn, wcn = oracle.torch_lstm(x, h0, c0, params, True, 1, True)
     y, hn, cn = cpp_gpu.atenLstm1(x.to(DEV), [h0.to(DEV), c0.to(DEV)], [p.to(DEV) for p in params], True, 1, 0.0, False, True, False)
     assert maxabs(y, wy) <= 2e-3 and maxabs(hn, whn) <= 2e-3 and maxabs(cn, wcn) <= 2e-3
@@ -144,8 +145,8 @@ def test_cpp_ops_run_on_torchs_current_stream(cpp_gpu):
     that is current in torch, the one their inputs were produced on and their outputs are allocated for.  The side
     stream is kept busy before the inputs are written; a launch on the null stream would read the inputs too early
     (torch's side streams do not synchronise with it)."""
-    W, x, b = oracle.gemv_inputs(2101, 1024, 1024)
-    params, xs, h0, c0 = oracle.lstm_inputs(78, 64, 128, 1, False, 9)
+    W, x, b = workloads.gemv_inputs(2101, 1024, 1024)
+    params, xs, h0, c0 = workloads.lstm_inputs(78, 64, 128, 1, False, 9)
     wy, whn, wcn = oracle.torch_lstm(xs, h0, c0, params, True, 1, False)
     want = oracle.torch_addmm(b, x, W).reshape(-1)
     Wd, bd = W.to(DEV), b.to(DEV)
@@ -173,7 +174,7 @@ def test_cpp_ops_run_on_torchs_current_stream(cpp_gpu):
 
 @pytest.mark.gpu
 def test_cpp_plan_cache_follows_weight_updates(cpp_gpu):
-    params, x, h0, c0 = oracle.lstm_inputs(126, 64, 128, 1, False, 20)
+    params, x, h0, c0 = workloads.lstm_inputs(126, 64, 128, 1, False, 20)
     pd = [p.to(DEV) for p in params]
     args = (x.to(DEV), [h0.to(DEV), c0.to(DEV)], pd, True, 1, 0.0, False, False, False)
     y0 = cpp_gpu.atenLstm1(*args)[0]

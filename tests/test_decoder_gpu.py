@@ -1,0 +1,251 @@
+"""The fused decoder step (pimhip_decoder_step: every layer's seq_len-1 LSTM cell, the attention context, the residual
+sums and the classifier in one launch) against LibTorch CPU running the same wiring operator by operator in fp16, and
+against the product's own operator-by-operator path.
+
+Tolerances: max abs error <= 5e-3 on layer outputs, h, c and logits (fp32 gates and accumulation here, fp16 between
+the operators in LibTorch), <= 2e-3 on the context (a GEMV output)."""
+import pytest
+import torch
+
+from pimaicompiler_amd import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+STATE_TOL = 5e-3
+GEMV_TOL = 2e-3
+
+
+def maxabs(a, b):
+    return float((a.detach().float().cpu().reshape(-1) - b.detach().float().cpu().reshape(-1)).abs().max())
+
+
+class Case:
+    """Random weights and one step's inputs for a decoder wiring; everything on the CPU in fp16."""
+
+    def __init__(self, seed, H, in0, L, first_ctx, first_res, vocab, src_len):
+        g = torch.Generator().manual_seed(seed)
+        self.H, self.in0, self.L, self.first_ctx, self.first_res, self.vocab = H, in0, L, first_ctx, first_res, vocab
+        self.params = []
+        for k in range(L):
+            in_w = (in0 + (H if first_ctx else 0)) if k == 0 else 2 * H
+            self.params += workloads.lstm_inputs(seed + 10 + k, in_w, H, 1, False, 1)[0]
+        self.x = torch.randn(in0, generator=g).half()
+        self.h = [(0.3 * torch.randn(H, generator=g)).half() for _ in range(L)]
+        self.c = [(0.3 * torch.randn(H, generator=g)).half() for _ in range(L)]
+        self.enc = torch.randn(src_len, H, generator=g).half()
+        self.att = torch.softmax(torch.randn(src_len, generator=g), -1).half()
+        self.Wc = (0.02 * torch.randn(vocab, H, generator=g)).half() if vocab else None
+        self.bc = (0.01 * torch.randn(vocab, generator=g)).half() if vocab else None
+
+    def cpu_step(self, x, h, c):
+        """The wiring with LibTorch CPU operators in fp16: returns ctx, outs, hn, cn, logits."""
+        H = self.H
+        ctx = torch.matmul(self.att.view(1, -1).float(), self.enc.float()).half()     # bmm: fp32 accumulate, one rounding
+        inp = x.view(1, -1)
+        outs, hns, cns = [], [], []
+        for k in range(self.L):
+            takes = k > 0 or self.first_ctx
+            full = torch.cat([inp, ctx], 1) if takes else inp
+            y, hn, cn = torch.lstm(full.view(1, 1, -1), (h[k].view(1, 1, H), c[k].view(1, 1, H)), self.params[4 * k:4 * k + 4],
+                                   True, 1, 0.0, False, False, False)
+            y = y.view(1, H)
+            out = y + inp if k >= self.first_res else y
+            outs.append(out.view(-1))
+            hns.append(hn.view(-1))
+            cns.append(cn.view(-1))
+            inp = out
+        logits = torch.addmm(self.bc, inp, self.Wc.t()).view(-1) if self.vocab else None
+        return ctx.view(-1), outs, hns, cns, logits
+
+    def plan(self, P):
+        cls = (self.Wc.to(DEV), self.bc.to(DEV)) if self.vocab else None
+        return P.DecoderPlan([p.to(DEV) for p in self.params], True, self.L, first_takes_context=self.first_ctx,
+                             first_residual_layer=self.first_res, classifier=cls)
+
+
+def run_fused(P, case, plan, x, h, c, n_ctx_outs=1, use_ctx_in=None):
+    H, L = case.H, case.L
+    nanv = lambda n: torch.full((n,), float("nan"), dtype=torch.float16, device=DEV)  # noqa: E731
+    hn, cn, outs = [nanv(H) for _ in range(L)], [nanv(H) for _ in range(L)], [nanv(H) for _ in range(L)]
+    ctx_outs = [nanv(H) for _ in range(n_ctx_outs)]
+    logits = nanv(case.vocab) if case.vocab else None
+    step = plan.bind(x.to(DEV), [t.to(DEV) for t in h], [t.to(DEV) for t in c],
+                     att=None if use_ctx_in is not None else case.att.to(DEV), enc=None if use_ctx_in is not None else case.enc.to(DEV),
+                     ctx=use_ctx_in, hn=hn, cn=cn, outs=outs, ctx_outs=ctx_outs, logits=logits)
+    step()
+    plan.status()
+    return ctx_outs, outs, hn, cn, logits
+
+
+def check(case, got, want, ctx_given=False):
+    ctx_outs, outs, hn, cn, logits = got
+    wctx, wouts, whn, wcn, wlogits = want
+    for cbuf in ctx_outs:
+        assert maxabs(cbuf, wctx) <= (0.0 if ctx_given else GEMV_TOL)
+    for k in range(case.L):
+        assert maxabs(outs[k], wouts[k]) <= STATE_TOL, k
+        assert maxabs(hn[k], whn[k]) <= STATE_TOL, k
+        assert maxabs(cn[k], wcn[k]) <= STATE_TOL, k
+    if case.vocab:
+        assert not bool(torch.isnan(logits).any())
+        assert maxabs(logits, wlogits) <= STATE_TOL
+
+
+# (H, in0, L, first_ctx, first_res, vocab, src_len)
+WIRINGS = [
+    (1024, 1024, 4, False, 2, 4096, 50),     # the whole GNMT decoder step
+    (1024, 1024, 3, True, 1, 32000, 50),     # layers 1..3 + classifier, layer 0 and the attention scores outside
+    (1024, 1024, 1, False, 9, 0, 50),        # a single plain cell, no classifier
+    (1024, 2048, 2, False, 1, 1001, 7),      # wide plain input, ragged vocabulary
+    (72, 40, 2, False, 1, 1001, 7),          # 9 pieces per row: the two halves of a row differ in length
+    (8, 8, 4, True, 0, 5, 1),                # the smallest shapes, residual around every layer
+    (520, 520, 4, False, 2, 640, 13),
+    (256, 64, 3, False, 2, 0, 3),            # no classifier: the last layer's exchange is left out
+]
+
+
+@pytest.mark.parametrize("H,in0,L,first_ctx,first_res,vocab,src_len", WIRINGS)
+def test_fused_decoder_step_matches_libtorch_cpu(ops, H, in0, L, first_ctx, first_res, vocab, src_len):
+    case = Case(1000 + H + L, H, in0, L, first_ctx, first_res, vocab, src_len)
+    print(f"decoder step H={H} in0={in0} L={L} first_ctx={first_ctx} first_res={first_res} vocab={vocab} S={src_len}", flush=True)
+    plan = case.plan(ops)
+    want = case.cpu_step(case.x, case.h, case.c)
+    check(case, run_fused(ops, case, plan, case.x, case.h, case.c, n_ctx_outs=3), want)
+    # the context handed in instead of att and enc: the same bits everywhere downstream of it
+    got = run_fused(ops, case, plan, case.x, case.h, case.c, n_ctx_outs=1, use_ctx_in=want[0].to(DEV))
+    check(case, got, want, ctx_given=True)
+
+
+def test_fused_decoder_steps_update_the_state_in_place(ops):
+    """A decoder loop: hn / cn are the buffers h_prev / c_prev are read from, three steps in a row, against the CPU
+    running the same three steps; then the same three steps again into separate buffers give the same bits."""
+    case = Case(77, 1024, 1024, 4, False, 2, 2048, 20)
+    plan = case.plan(ops)
+    g = torch.Generator().manual_seed(5)
+    xs = [torch.randn(1024, generator=g).half() for _ in range(3)]
+    h, c = [t.clone() for t in case.h], [t.clone() for t in case.c]
+    hd, cd = [t.to(DEV) for t in case.h], [t.to(DEV) for t in case.c]
+    xd = torch.zeros(1024, dtype=torch.float16, device=DEV)
+    logits = torch.zeros(case.vocab, dtype=torch.float16, device=DEV)
+    step = plan.bind(xd, hd, cd, att=case.att.to(DEV), enc=case.enc.to(DEV), logits=logits)     # in place
+    all_logits = []
+    for x in xs:
+        xd.copy_(x.to(DEV))
+        step()
+        _, _, h, c, wl = case.cpu_step(x, h, c)
+        plan.status()
+        for k in range(4):
+            assert maxabs(hd[k], h[k]) <= STATE_TOL and maxabs(cd[k], c[k]) <= STATE_TOL
+        assert maxabs(logits, wl) <= STATE_TOL
+        all_logits.append(logits.clone())
+    h2, c2 = [t.to(DEV) for t in case.h], [t.to(DEV) for t in case.c]
+    for i, x in enumerate(xs):
+        hn, cn = [torch.empty_like(t) for t in h2], [torch.empty_like(t) for t in c2]
+        plan.bind(x.to(DEV), h2, c2, att=case.att.to(DEV), enc=case.enc.to(DEV), hn=hn, cn=cn, logits=logits)()
+        torch.cuda.synchronize()
+        assert torch.equal(logits, all_logits[i])
+        h2, c2 = hn, cn
+    for k in range(4):
+        assert torch.equal(h2[k], hd[k]) and torch.equal(c2[k], cd[k])
+
+
+def test_fused_decoder_step_agrees_with_the_operator_by_operator_path(ops):
+    """Same weights and inputs through pimhip_lstm_forward x 4, bmm, add x 2 and the classifier GEMV (eight launches):
+    the same mathematics with another order of the fp32 sums."""
+    case = Case(31, 1024, 1024, 4, False, 2, 32000, 50)
+    H = 1024
+    plan = case.plan(ops)
+    got = run_fused(ops, case, plan, case.x, case.h, case.c, n_ctx_outs=1)
+    prm = [p.to(DEV) for p in case.params]
+    cell = [ops.LstmPlan(prm[4 * k:4 * k + 4], True, 1, False, 1) for k in range(4)]
+    ctx = ops.aten_bmm(case.att.view(1, 1, -1).to(DEV), case.enc.view(1, -1, H).to(DEV)).view(1, H)
+    inp, hs, cs = case.x.view(1, H).to(DEV), [], []
+    for k in range(4):
+        full = torch.cat([inp, ctx], 1) if k > 0 else inp
+        y, hn, cn = cell[k].forward(full, case.h[k].view(1, H).to(DEV), case.c[k].view(1, H).to(DEV))
+        out = ops.aten_add(y, inp) if k >= 2 else y
+        hs.append(hn)
+        cs.append(cn)
+        inp = out
+        assert maxabs(got[1][k], out) <= 1e-3
+    logits = ops.custom_aten_addmm("none", case.bc.to(DEV), case.Wc.to(DEV), inp.t())
+    assert maxabs(got[0][0], ctx) <= 1e-3
+    for k in range(4):
+        assert maxabs(got[2][k], hs[k]) <= 1e-3 and maxabs(got[3][k], cs[k]) <= 1e-3
+    assert maxabs(got[4], logits) <= 2e-3
+
+
+def test_fused_decoder_step_replays_from_a_graph(ops):
+    case = Case(41, 1024, 1024, 4, False, 2, 32000, 50)
+    plan = case.plan(ops)
+    g = torch.Generator().manual_seed(9)
+    xs = [torch.randn(1024, generator=g).half().to(DEV) for _ in range(3)]
+    xd = torch.zeros(1024, dtype=torch.float16, device=DEV)
+    h0, c0 = [t.to(DEV) for t in case.h], [t.to(DEV) for t in case.c]
+    hn, cn = [torch.empty_like(t) for t in h0], [torch.empty_like(t) for t in c0]
+    logits = torch.zeros(case.vocab, dtype=torch.float16, device=DEV)
+    step = plan.bind(xd, h0, c0, att=case.att.to(DEV), enc=case.enc.to(DEV), hn=hn, cn=cn, logits=logits)
+    eager = []
+    for x in xs:
+        xd.copy_(x)
+        step()
+        torch.cuda.synchronize()
+        eager.append([logits.clone()] + [t.clone() for t in hn + cn])
+    plan.status()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step(torch.cuda.current_stream())
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    scratch = torch.randn(1 << 20, device=DEV)
+    for rep in range(2):
+        for x, want in zip(xs, eager):
+            xd.copy_(x)
+            for t in hn + cn + [logits]:
+                t.fill_(float("nan"))
+            graph.replay()
+            scratch = scratch * 1.0001 + 1.0
+            torch.cuda.synchronize()
+            for got, w in zip([logits] + hn + cn, want):
+                assert torch.equal(got, w)
+    plan.status()
+
+
+def test_fused_decoder_step_wait_gives_up_and_reports(ops):
+    """Forced from the host: with a spin limit of 0 every wait gives up at its first unsuccessful poll, the kernel still
+    runs to its end; the time-out is reported once (here by the next step, nobody having asked for the status), and the
+    step after that is right again."""
+    case = Case(51, 1024, 1024, 4, False, 2, 1024, 10)
+    plan = case.plan(ops)
+    want = case.cpu_step(case.x, case.h, case.c)
+    plan.set_spin_limit(0)
+    hn, cn = [torch.empty(1024, dtype=torch.float16, device=DEV) for _ in range(4)], [torch.empty(1024, dtype=torch.float16, device=DEV) for _ in range(4)]
+    logits = torch.empty(1024, dtype=torch.float16, device=DEV)
+    step = plan.bind(case.x.to(DEV), [t.to(DEV) for t in case.h], [t.to(DEV) for t in case.c], att=case.att.to(DEV),
+                     enc=case.enc.to(DEV), hn=hn, cn=cn, logits=logits)
+    step()
+    torch.cuda.synchronize()
+    plan.set_spin_limit(1 << 22)
+    with pytest.raises(ops.NNRuntimeException, match="gave up a wait"):
+        step()
+    step()
+    plan.status()
+    assert maxabs(logits, want[4]) <= STATE_TOL
+    for k in range(4):
+        assert maxabs(hn[k], want[2][k]) <= STATE_TOL
+
+
+def test_decoder_plan_refuses_what_the_kernel_does_not_take(ops):
+    prm = [p.to(DEV) for p in workloads.lstm_inputs(3, 2056, 2056, 1, False, 1)[0]]
+    with pytest.raises(ops.NNRuntimeException, match="hidden_size"):
+        ops.DecoderPlan(prm, True, 1)
+    prm = [p.to(DEV) for p in workloads.lstm_inputs(3, 64, 64, 1, False, 1)[0]]
+    with pytest.raises(ops.NNRuntimeException):
+        ops.DecoderPlan(prm * 5, True, 5)
+    plan = ops.DecoderPlan(prm, True, 1, first_residual_layer=9)
+    v = torch.zeros(64, dtype=torch.float16, device=DEV)
+    with pytest.raises(ops.NNRuntimeException, match="in place"):
+        plan.bind(v.clone(), [v], [v.clone()])()          # one layer, no classifier: no exchange to order the update behind

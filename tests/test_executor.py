@@ -10,6 +10,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 from pimaicompiler_amd import executor as E
 from pimaicompiler_amd.executor import DataType, LayerType
 
@@ -245,7 +246,7 @@ def _gate_graph(seed, n_gates, out_w, in_w):
     lists the MULTISTREAM layer followed by its duplicated sub-layers, as the reference's builder leaves them."""
     Ws, bs, x = [], [], None
     for i in range(n_gates):
-        W, x, b = oracle.gemv_inputs(seed + i, out_w, in_w)
+        W, x, b = workloads.gemv_inputs(seed + i, out_w, in_w)
         Ws.append(W)
         bs.append(b)
     subs, blobs = [], {"b0": x.t().to(DEV)}
@@ -305,7 +306,7 @@ def test_grouped_and_streamed_multi_stream_agree_bit_for_bit(ops):
 
 @pytest.mark.gpu
 def test_addmm_vm_order_and_none_bias(ops):
-    W, x, b = oracle.gemv_inputs(3, 320, 256)
+    W, x, b = workloads.gemv_inputs(3, 320, 256)
     A = W.t().contiguous()
     ex = E.StreamExecutor([], device=0)
     _blobs(ex, b0=b.to(DEV), b1=x.to(DEV), b2=A.to(DEV), b3=None)
@@ -321,7 +322,7 @@ def test_addmm_vm_order_and_none_bias(ops):
 @pytest.mark.gpu
 @pytest.mark.parametrize("bidirectional,num_layers", [(False, 2), (True, 1)])
 def test_lstm1_layer_with_flags_from_blobs(ops, bidirectional, num_layers):
-    params, x, h0, c0 = oracle.lstm_inputs(11, 64, 128, num_layers, bidirectional, 9)
+    params, x, h0, c0 = workloads.lstm_inputs(11, 64, 128, num_layers, bidirectional, 9)
     g = torch.Generator().manual_seed(5)
     h0 = (0.1 * torch.randn(h0.shape, generator=g)).half()
     c0 = (0.1 * torch.randn(c0.shape, generator=g)).half()
@@ -342,7 +343,7 @@ def test_lstm1_layer_with_flags_from_blobs(ops, bidirectional, num_layers):
 
 @pytest.mark.gpu
 def test_lstm2_layer_on_the_rnnt_feature_shape(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(12, 240, 256, 2, False, 21)
+    params, x, h0, c0 = workloads.lstm_inputs(12, 240, 256, 2, False, 21)
     ex = E.StreamExecutor([], device=0)
     _blobs(ex, b0=x.reshape(21, 240).to(DEV), b1=torch.ones(21, dtype=torch.int64), b2=[h0.to(DEV), c0.to(DEV)])
     layer = E.AtenLSTM2Layer(LayerType.ATENLSTM2, 0, [0, 1, 2], [20, 21, 22], has_biases=1, num_layers=2, dropout=0.0,
@@ -387,8 +388,8 @@ def test_built_model_lstm_then_linear_on_the_rnnt_feature(ops):
     import os
     feat = io.load_tensor(os.path.join(os.path.dirname(__file__), "golden", "rnnt_feature_341x1x240_f16.bin"), [341, 1, 240], "FLOAT16")
     x = feat[:30].contiguous()
-    params, _, h0, c0 = oracle.lstm_inputs(21, 240, 128, 2, False, 30)
-    W, _, b = oracle.gemv_inputs(22, 64, 128)
+    params, _, h0, c0 = workloads.lstm_inputs(21, 240, 128, 2, False, 30)
+    W, _, b = workloads.gemv_inputs(22, 64, 128)
     lstm = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1], [2, 3, 4], has_biases=1, num_layers=2, dropout=0.0, train=0,
                             bidirectional=0, batch_first=0, weights=[params[i] for i in (0, 1, 4, 5)],
                             biases=[params[i] for i in (2, 3, 6, 7)])
@@ -412,7 +413,7 @@ def test_gnmt_decoder_steps_write_into_the_state_and_attention_buffers(ops):
     layer by layer with explicit states."""
     H, steps = 256, 3
     g = torch.Generator().manual_seed(31)
-    layer_params = [oracle.lstm_inputs(40 + k, H, H, 1, False, 1)[0] for k in range(4)]
+    layer_params = [workloads.lstm_inputs(40 + k, H, H, 1, False, 1)[0] for k in range(4)]
     state = (0.2 * torch.randn(8, 1, H, generator=g)).half()
     xs = torch.randn(steps, 4, 1, 1, H, generator=g).half()           # an independent input per step and layer
     ex = E.StreamExecutor([], model_type="GNMT", device=0)

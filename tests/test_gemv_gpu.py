@@ -11,6 +11,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 
 pytestmark = pytest.mark.gpu
 GEMV_TOL = 2e-3
@@ -45,7 +46,7 @@ SHAPES = [(1, 8), (1, 1), (3, 5), (7, 17), (16, 8), (64, 64), (100, 264), (255, 
 @pytest.mark.parametrize("n,k", SHAPES)
 @pytest.mark.parametrize("bias,relu", [(True, False), (True, True), (False, False)])
 def test_gemv_both_orders_match_oracle(ops, n, k, bias, relu):
-    W, x, b = oracle.gemv_inputs(100 + n + k, n, k, bias=True)
+    W, x, b = workloads.gemv_inputs(100 + n + k, n, k, bias=True)
     W = (W * 5).half()
     want = oracle.gemv_mv(W.numpy(), x.numpy().reshape(-1), b.numpy() if bias else None, relu=relu)
     from pimaicompiler_amd import _lib as L
@@ -63,7 +64,7 @@ def test_gemv_both_orders_match_oracle(ops, n, k, bias, relu):
 def test_gemv_result_is_correctly_rounded_almost_everywhere(ops):
     """fp32 accumulation then one rounding: the result is within one fp16 ulp of the exactly rounded value and
     equal to it for all but near-tie elements."""
-    W, x, b = oracle.gemv_inputs(77, 2048, 2048)
+    W, x, b = workloads.gemv_inputs(77, 2048, 2048)
     want = oracle.gemv_mv(W.numpy(), x.numpy().reshape(-1), b.numpy())
     y = ops.aten_linear(x.to(DEV), W.to(DEV), b.to(DEV)).cpu().numpy().reshape(-1)
     assert np.all(np.abs(y.astype(np.float64) - want.astype(np.float64)) <= ulp_f16(want))
@@ -120,7 +121,7 @@ CONFIGS = [("c1_1024x1024", 1001, 1024, 1024), ("c2_4096x4096", 2001, 4096, 4096
 
 @pytest.mark.parametrize("name,seed,n,k", CONFIGS)
 def test_gemv_configs_match_libtorch_cpu_addmm(ops, golden, name, seed, n, k):
-    W, x, b = oracle.gemv_inputs(seed, n, k)
+    W, x, b = workloads.gemv_inputs(seed, n, k)
     want = oracle.torch_addmm(b, x, W).reshape(-1)            # at::addmm(b, x, W^T), CPU, fp16
     # the op as the runtime issues it after its rewrite passes: addmm(b, W[out,in], x^T[in,1])
     y = ops.custom_aten_addmm("none", b.to(DEV), W.to(DEV), x.to(DEV).t())
@@ -241,7 +242,7 @@ def test_against_the_references_own_hip_kernels(ops):
     ref = oracle.ref_lib()
     if ref is None:
         pytest.skip("oracle/_ref was not built (reference tree absent at build time)")
-    W, x, b = oracle.gemv_inputs(31, 4096, 1024)
+    W, x, b = workloads.gemv_inputs(31, 4096, 1024)
     Wd, xd, bd = W.to(DEV), x.to(DEV).reshape(-1), b.to(DEV)
     s = torch.cuda.current_stream().cuda_stream
     out = torch.zeros(4096, dtype=torch.float16, device=DEV)

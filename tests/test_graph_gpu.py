@@ -6,6 +6,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -21,7 +22,7 @@ class DecoderStep:
         in_w = [H, 2 * H, 2 * H, 2 * H]
         self.plans, self.state = [], []
         for k in range(4):
-            params = oracle.lstm_inputs(seed + 10 + k, in_w[k], H, 1, False, 1)[0]
+            params = workloads.lstm_inputs(seed + 10 + k, in_w[k], H, 1, False, 1)[0]
             self.plans.append(P.LstmPlan([p.to(DEV) for p in params], True, 1, False, 1))
             self.state.append(((0.1 * torch.randn(1, H, generator=g)).half().to(DEV), (0.1 * torch.randn(1, H, generator=g)).half().to(DEV)))
         self.enc = torch.randn(1, src_len, H, generator=g).half().to(DEV)          # encoder outputs
@@ -132,7 +133,7 @@ def test_sequence_forward_replays_from_a_graph(ops):
     graph must not record, the re-initialisation of the exchange buffer after a change of mode, is refused."""
     T, I, Hs = 7, 64, 256
     for layers, bidir in ((2, False), (1, True), (1, False)):
-        params, x, h0, c0 = oracle.lstm_inputs(7101 + layers + 2 * bidir, I, Hs, layers, bidir, T)
+        params, x, h0, c0 = workloads.lstm_inputs(7101 + layers + 2 * bidir, I, Hs, layers, bidir, T)
         plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, bidir, T)
         xd, hd, cd = x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV)
         x2 = (0.5 * xd + 0.25).contiguous()

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 
 pytestmark = pytest.mark.gpu
 LSTM_TOL = 5e-3
@@ -70,7 +71,7 @@ CASES = [  # I, H, L, bidirectional, T, biases
 def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
     if mode >= 2 and H > 2048:
         pytest.skip("the persistent kernel takes hidden sizes up to 2048; larger ones run step by step")
-    params, x, h0, c0 = oracle.lstm_inputs(900 + I + H + T, I, H, L, bidir, T, has_b)
+    params, x, h0, c0 = workloads.lstm_inputs(900 + I + H + T, I, H, L, bidir, T, has_b)
     g = torch.Generator().manual_seed(T)
     h0 = (0.3 * torch.randn(h0.shape, generator=g)).half()
     c0 = (0.3 * torch.randn(c0.shape, generator=g)).half()
@@ -82,7 +83,7 @@ def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
 
 
 def test_persistent_kernel_refuses_what_it_cannot_hold(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(1, 16, 2056, 1, False, 2)
+    params, x, h0, c0 = workloads.lstm_inputs(1, 16, 2056, 1, False, 2)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 2)
     with pytest.raises(ops.NNRuntimeException):
         plan.set_mode(2)
@@ -92,7 +93,7 @@ def test_persistent_kernel_refuses_what_it_cannot_hold(ops):
 @pytest.mark.parametrize("mode", MODES)
 def test_lstm_c3_rnnt_matches_libtorch_cpu(ops, golden, mode):
     """2 layers unidirectional, I=240, H=1024, T=200."""
-    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    params, x, h0, c0 = workloads.lstm_inputs(3001, 240, 1024, 2, False, 200)
     wy, whn, wcn = oracle.torch_lstm(x, h0, c0, params, True, 2, False)                      # fp16 CPU (arbiter)
     fy, fhn, fcn = oracle.torch_lstm(x.float(), h0.float(), c0.float(), [p.float() for p in params], True, 2, False)
     y, hn, cn = run_plan(ops, params, x, h0, c0, True, 2, False, mode)
@@ -110,7 +111,7 @@ def test_lstm_c4_gnmt_stack_matches_libtorch_cpu(ops, golden):
     g = golden["lstm_large"]
     seq_dev, seq_cpu = None, None
     for li, (in_w, bidir) in enumerate([(1024, True), (2048, False), (1024, False), (1024, False)]):
-        params, x0, h0, c0 = oracle.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
+        params, x0, h0, c0 = workloads.lstm_inputs(4001 + li, in_w, 1024, 1, bidir, 50)
         if seq_dev is None:
             seq_dev, seq_cpu = x0.to(DEV), x0
         wy, whn, wcn = oracle.torch_lstm(seq_cpu, h0, c0, params, True, 1, bidir)
@@ -122,7 +123,7 @@ def test_lstm_c4_gnmt_stack_matches_libtorch_cpu(ops, golden):
         assert maxabs(hn, g[f"c4_l{li}_hn"]) <= LSTM_TOL and maxabs(cn, g[f"c4_l{li}_cn"]) <= LSTM_TOL
         assert maxabs(y.reshape(50, -1)[::7, ::32], g[f"c4_l{li}_y_samples"]) <= LSTM_TOL
         seq_dev, seq_cpu = y, wy
-    W, _, b = oracle.gemv_inputs(4010, 32000, 1024)
+    W, _, b = workloads.gemv_inputs(4010, 32000, 1024)
     logits = ops.aten_linear(seq_dev[-1].reshape(1, 1024), W.to(DEV), b.to(DEV)).reshape(-1)
     want = oracle.torch_addmm(b, seq_cpu[-1].reshape(1, 1024), W).reshape(-1)
     # the GEMV input differs by the LSTM's own error (<= 5e-3 per element) times |W| summed: allow for it
@@ -132,7 +133,7 @@ def test_lstm_c4_gnmt_stack_matches_libtorch_cpu(ops, golden):
 
 # ---- interface forms --------------------------------------------------------------------------------------------
 def test_lstm1_batch_first_and_lstm2_packed_agree(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(55, 32, 64, 2, True, 6)
+    params, x, h0, c0 = workloads.lstm_inputs(55, 32, 64, 2, True, 6)
     pd = [p.to(DEV) for p in params]
     hx = (h0.to(DEV), c0.to(DEV))
     y, hn, cn = ops.aten_lstm1(x.to(DEV), hx, pd, True, 2, 0.5, False, True, False)       # dropout is ignored
@@ -154,7 +155,7 @@ def test_lstm_decode_loop_step_by_step_equals_one_sequence_call(ops):
     """The decoders call aten::lstm with seq_len == 1 inside prim::Loop, feeding (hy, cy) back: T such calls must
     reproduce one call over the whole sequence (same rounding points: h fp16 every step; c passes through fp16
     between calls, so c is compared to tolerance)."""
-    params, x, h0, c0 = oracle.lstm_inputs(66, 64, 256, 2, False, 12)
+    params, x, h0, c0 = workloads.lstm_inputs(66, 64, 256, 2, False, 12)
     pd = [p.to(DEV) for p in params]
     y_all, hn_all, cn_all = ops.aten_lstm1(x.to(DEV), (h0.to(DEV), c0.to(DEV)), pd, True, 2, 0.0, False, False, False)
     h, c = h0.to(DEV), c0.to(DEV)
@@ -167,7 +168,7 @@ def test_lstm_decode_loop_step_by_step_equals_one_sequence_call(ops):
 
 
 def test_lstm_zero_length_sequence_passes_state_through(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(77, 16, 32, 1, False, 4)
+    params, x, h0, c0 = workloads.lstm_inputs(77, 16, 32, 1, False, 4)
     g = torch.Generator().manual_seed(1)
     h0 = torch.randn(h0.shape, generator=g).half()
     c0 = torch.randn(c0.shape, generator=g).half()
@@ -177,7 +178,7 @@ def test_lstm_zero_length_sequence_passes_state_through(ops):
 
 
 def test_lstm_plan_reuse_and_sequence_longer_than_plan(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(88, 16, 64, 1, False, 20)
+    params, x, h0, c0 = workloads.lstm_inputs(88, 16, 64, 1, False, 20)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 10)
     with pytest.raises(ops.NNRuntimeException):
         plan.forward(x.reshape(20, 16).to(DEV), h0.to(DEV), c0.to(DEV))
@@ -208,7 +209,7 @@ def test_lstm_full_size_zero_weights_closed_form(ops):
 
 
 def test_lstm_bidirectional_equals_forward_on_reversed_input(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(99, 128, 1024, 1, True, 24)
+    params, x, h0, c0 = workloads.lstm_inputs(99, 128, 1024, 1, True, 24)
     y, hn, cn = run_plan(ops, params, x, h0, c0, True, 1, True, 2)
     yf, hf, cf = run_plan(ops, params[:4], x, h0[:1], c0[:1], True, 1, False, 2)
     yb, hb, cb = run_plan(ops, params[4:], x.flip(0), h0[1:], c0[1:], True, 1, False, 2)
@@ -220,7 +221,7 @@ def test_lstm_bidirectional_equals_forward_on_reversed_input(ops):
 
 
 def test_step_and_sequence_kernels_agree(ops):
-    params, x, h0, c0 = oracle.lstm_inputs(111, 1024, 1024, 1, False, 50)
+    params, x, h0, c0 = workloads.lstm_inputs(111, 1024, 1024, 1, False, 50)
     y1, h1, c1 = run_plan(ops, params, x, h0, c0, True, 1, False, 1)
     y2, h2, c2 = run_plan(ops, params, x, h0, c0, True, 1, False, 2)
     assert maxabs(y1, y2.cpu()) <= 1e-3 and maxabs(c1, c2.cpu()) <= 1e-3
@@ -229,7 +230,7 @@ def test_step_and_sequence_kernels_agree(ops):
 def test_switching_the_block_shape_on_one_plan_restarts_the_exchange(ops):
     """Modes 2 and 3 lay out a single layer's exchange entries differently; a plan that switches must not read what
     the other layout left behind."""
-    params, x, h0, c0 = oracle.lstm_inputs(77, 64, 1024, 1, False, 23)
+    params, x, h0, c0 = workloads.lstm_inputs(77, 64, 1024, 1, False, 23)
     want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 23)
     outs = []
@@ -250,7 +251,7 @@ def test_sequence_kernels_issued_on_two_streams_do_not_starve_each_other(ops):
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
     cases = []
     for i, st in enumerate(streams):
-        params, x, h0, c0 = oracle.lstm_inputs(200 + i, 64, 1024, 2, False, 40)
+        params, x, h0, c0 = workloads.lstm_inputs(200 + i, 64, 1024, 2, False, 40)
         plan = ops.LstmPlan([p.to(DEV) for p in params], True, 2, False, 40)
         plan.set_mode(2)
         plan.set_spin_limit(1 << 16)
@@ -272,7 +273,7 @@ def test_sequence_kernels_issued_on_two_streams_do_not_starve_each_other(ops):
 def test_persistent_kernel_wait_gives_up_and_reports(ops):
     """Forced from the host: with a spin limit of 0 every wait gives up at its first unsuccessful poll, the kernel
     still runs to its end, and the plan reports the time-out.  A later forward with the default limit works."""
-    params, x, h0, c0 = oracle.lstm_inputs(123, 64, 1024, 1, False, 30)
+    params, x, h0, c0 = workloads.lstm_inputs(123, 64, 1024, 1, False, 30)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 30)
     plan.set_mode(2)
     plan.set_spin_limit(0)
@@ -290,7 +291,7 @@ def test_a_timeout_nobody_asked_about_is_raised_by_the_next_call(ops):
     """aten_lstm1 never calls status(): a wait that gave up (forced from the host with a spin limit of 0; the kernel
     still runs to its end) must make the NEXT call on those weights raise instead of vanishing, exactly once; the call
     after that starts from a re-initialised exchange buffer and is right again."""
-    params, x, h0, c0 = oracle.lstm_inputs(124, 64, 1024, 1, False, 30)
+    params, x, h0, c0 = workloads.lstm_inputs(124, 64, 1024, 1, False, 30)
     pd = [p.to(DEV) for p in params]
     xd, hx = x.to(DEV), (h0.to(DEV), c0.to(DEV))
     plan = ops.prepare_lstm(pd, True, 1, False, 30)
@@ -313,7 +314,7 @@ def test_plan_cache_follows_weight_updates_and_is_bounded(ops):
     update seen by torch's version counter gives a new plan, invalidate_lstm_plans drops plans on request, and the cache
     never holds more than PLAN_CACHE_MAX plans."""
     from pimaicompiler_amd import ops as O
-    params, x, h0, c0 = oracle.lstm_inputs(125, 64, 128, 1, False, 20)
+    params, x, h0, c0 = workloads.lstm_inputs(125, 64, 128, 1, False, 20)
     pd = [p.to(DEV) for p in params]
     xd, hx = x.to(DEV), (h0.to(DEV), c0.to(DEV))
     y0 = ops.aten_lstm1(xd, hx, pd, True, 1, 0.0, False, False, False)[0]
@@ -332,7 +333,7 @@ def test_plan_cache_follows_weight_updates_and_is_bounded(ops):
     # bound
     keep = []
     for i in range(O.PLAN_CACHE_MAX + 3):
-        prm, *_ = oracle.lstm_inputs(300 + i, 8, 8, 1, False, 2)
+        prm, *_ = workloads.lstm_inputs(300 + i, 8, 8, 1, False, 2)
         keep.append([p.to(DEV) for p in prm])
         O._plan_for(keep[-1], True, 1, False, 2)
     assert len(O._plan_cache) == O.PLAN_CACHE_MAX
@@ -343,7 +344,7 @@ def test_plan_cache_follows_weight_updates_and_is_bounded(ops):
 def test_persistent_kernel_survives_a_nan_input(ops, mode):
     """A NaN cannot carry the exchange's flag bit, so it is exchanged as 0; the cell state keeps it, and y is NaN from
     that step on exactly as in LibTorch.  No wait times out."""
-    params, x, h0, c0 = oracle.lstm_inputs(5, 64, 512, 1, False, 12)
+    params, x, h0, c0 = workloads.lstm_inputs(5, 64, 512, 1, False, 12)
     x = x.clone()
     x[7, 0, 3] = float("nan")
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 12)

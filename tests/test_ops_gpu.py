@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -209,7 +210,7 @@ def test_bmm_with_rows_or_batches_takes_libtorch(ops):
 def test_decoder_step_writes_into_consumer_buffers(ops):
     """seq_len == 1 LSTM step with hy / cy / y placed straight into preallocated buffers (the GNMT decoder's
     [8, 1, 1024] state buffer and [1, 1, 2048] concatenation buffer, miopen_ops_executor.cpp:170-228)."""
-    params, x, h0, c0 = oracle.lstm_inputs(5, 1024, 1024, 1, False, 1)
+    params, x, h0, c0 = workloads.lstm_inputs(5, 1024, 1024, 1, False, 1)
     g = torch.Generator().manual_seed(5)
     h0, c0 = (0.3 * torch.randn(1, 1, 1024, generator=g)).half(), (0.3 * torch.randn(1, 1, 1024, generator=g)).half()
     want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
@@ -229,7 +230,7 @@ def test_rnnt_encoder_lstm_on_the_references_feature_file(ops):
     import os
     from pimaicompiler_amd import io
     feat = io.load_tensor(os.path.join(os.path.dirname(__file__), "golden", "rnnt_feature_341x1x240_f16.bin"), [341, 1, 240], "FLOAT16")
-    params, _, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 1)
+    params, _, h0, c0 = workloads.lstm_inputs(3001, 240, 1024, 2, False, 1)
     want = oracle.torch_lstm(feat, h0, c0, params, True, 2, False)
     y, hn, cn = ops.aten_lstm1(feat.to(DEV), (h0.to(DEV), c0.to(DEV)), [p.to(DEV) for p in params], True, 2, 0.0, False, False, False)
     assert list(y.shape) == [341, 1, 1024]

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 
 GEMV_TOL = 2e-3   # max abs error allowed on GEMV outputs
 LSTM_TOL = 5e-3   # max abs error allowed on y / h / c
@@ -45,7 +46,7 @@ def test_double_to_half_rounds_to_nearest_even():
 
 # ---- GEMV: LibTorch golden vectors ---------------------------------------------------------------------------
 def test_gemv_mv_c1_matches_libtorch_addmm(golden):
-    W, x, b = oracle.gemv_inputs(1001, 1024, 1024)
+    W, x, b = workloads.gemv_inputs(1001, 1024, 1024)
     y = oracle.gemv_mv(W.numpy(), x.numpy().reshape(-1), b.numpy())
     g = golden["gemv"]["c1_1024x1024_y"]
     assert maxabs(y, g) <= GEMV_TOL
@@ -56,7 +57,7 @@ def test_gemv_mv_c1_matches_libtorch_addmm(golden):
 @pytest.mark.parametrize("name,seed,n,k", [("c2_4096x4096", 2001, 4096, 4096), ("c2_16384x4096", 2002, 16384, 4096),
                                           ("c2_4096x16384", 2003, 4096, 16384), ("c2_32000x1024", 2004, 32000, 1024)])
 def test_gemv_mv_sweep_samples_match_libtorch(golden, name, seed, n, k):
-    W, x, b = oracle.gemv_inputs(seed, n, k)
+    W, x, b = workloads.gemv_inputs(seed, n, k)
     idx = golden["gemv"][name + "_idx"]
     y = oracle.gemv_mv(W.numpy()[idx], x.numpy().reshape(-1), b.numpy()[idx])
     assert maxabs(y, golden["gemv"][name + "_y_samples"]) <= GEMV_TOL
@@ -170,7 +171,7 @@ def test_lstm_tiny_matches_libtorch(golden, key):
 
 
 def test_lstm_c3_final_state_matches_libtorch(golden):
-    params, x, h0, c0 = oracle.lstm_inputs(3001, 240, 1024, 2, False, 200)
+    params, x, h0, c0 = workloads.lstm_inputs(3001, 240, 1024, 2, False, 200)
     y, hn, cn = oracle.lstm(x.numpy().reshape(200, 240), h0.numpy(), c0.numpy(), [p.numpy() for p in params], True, 2, False)
     g = golden["lstm_large"]
     assert maxabs(hn, g["c3_hn"].reshape(hn.shape)) <= LSTM_TOL

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from pimaicompiler_amd import workloads
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -30,7 +31,7 @@ def test_static_entry_point_matches_the_allocating_one_on_two_calls_in_a_row(ops
     from pimaicompiler_amd import _lib as L
     lib = L.load()
     for (n, k) in (first, second):
-        W, x, b = oracle.gemv_inputs(7000 + n + k, n, k, bias=True)
+        W, x, b = workloads.gemv_inputs(7000 + n + k, n, k, bias=True)
         want = oracle.gemv_mv(W.numpy(), x.numpy().reshape(-1), b.numpy(), relu=True)
         At = W.t().contiguous().to(DEV)
         xd, bd = x.to(DEV).reshape(-1), b.to(DEV)
@@ -59,7 +60,7 @@ def test_static_entry_point_records_on_a_stream_it_has_never_seen(ops):
     from pimaicompiler_amd import _lib as L
     lib = L.load()
     n, k = 2048, 4096
-    W, x, b = oracle.gemv_inputs(7100, n, k, bias=True)
+    W, x, b = workloads.gemv_inputs(7100, n, k, bias=True)
     At, xd, bd = W.t().contiguous().to(DEV), x.to(DEV).reshape(-1), b.to(DEV)
     rc, eager = _call(lib.pimhip_execute_gemv_static, At, xd, bd, k, n, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
     assert rc == 0, lib.pimhip_last_error()
