@@ -242,7 +242,16 @@ int pimhip_decoder_plan_create(PimHipDecoderPlan** plan, const void* const* para
 
 int pimhip_decoder_plan_destroy(PimHipDecoderPlan* plan);
 
-/* One step.  x [input_size]; att [enc_len] and enc [enc_len, H] (row-major, dense), or ctx_in [H] instead of both;
+/* Once per sentence (whenever the encoder outputs change): enc [enc_len, H], row-major and dense.  The context columns
+ * of every layer's W_ih are multiplied with enc here, once (enc . W_ih[:, H:2H]^T, fp32, on the matrix cores), because
+ * W_ih[:, H:2H] . (att . enc) = (W_ih[:, H:2H] . enc^T) . att: a step then reads enc_len values per gate row instead of
+ * streaming those H columns, and needs no context vector.  The plan keeps the pointer (enc must stay valid and unchanged
+ * until the next call; it is read again only by steps that store the context).  Enqueues on `stream`; a call that needs
+ * a larger buffer than the plan has synchronises the stream and allocates (not on a capturing stream). */
+int pimhip_decoder_plan_set_encoder(PimHipDecoderPlan* plan, const void* enc, int64_t enc_len, void* stream);
+
+/* One step.  x [input_size]; att [enc_len], the attention weights over the encoder outputs given to
+ * pimhip_decoder_plan_set_encoder, or instead ctx_in [H], a context computed elsewhere (its columns are then streamed);
  * h_prev, c_prev, hn, cn, layer_outs: host arrays of num_layers device pointers to [H] vectors (the rows of a state
  * buffer, for instance); layer_outs, or any entry of it, may be NULL, otherwise entry k receives out_k; the context is
  * also stored to the n_ctx_outs (0..4) buffers of ctx_outs; logits [vocab].  hn[k] / cn[k] may be the buffers
@@ -250,8 +259,8 @@ int pimhip_decoder_plan_destroy(PimHipDecoderPlan* plan);
  * input.  All blocks of the launch have to be resident at once, so the call is ordered like a sequence call of
  * pimhip_lstm_forward against the device's other such launches, and steps sharing a plan must be ordered on one stream.
  * Records one kernel.  Every wait inside is bounded: see pimhip_decoder_plan_status. */
-int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const void* att, const void* enc, int64_t enc_len,
-                        const void* ctx_in, const void* const* h_prev, const void* const* c_prev, void* const* hn,
+int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const void* att, const void* ctx_in,
+                        const void* const* h_prev, const void* const* c_prev, void* const* hn,
                         void* const* cn, void* const* layer_outs, void* const* ctx_outs, int n_ctx_outs, void* logits,
                         void* stream);
 

@@ -48,7 +48,8 @@ SIGNATURES = {
                                                   ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
                                                   ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
     "pimhip_decoder_plan_destroy": (ctypes.c_int, [ctypes.c_void_p]),
-    "pimhip_decoder_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+    "pimhip_decoder_plan_set_encoder": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
+    "pimhip_decoder_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                            ctypes.c_void_p, c_void_pp, c_void_pp, c_void_pp, c_void_pp, c_void_pp, c_void_pp,
                                            ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
     "pimhip_decoder_plan_status": (ctypes.c_int, [ctypes.c_void_p]),

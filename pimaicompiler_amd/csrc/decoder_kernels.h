@@ -11,22 +11,38 @@
 //     logits = W_c . out_last + b_c
 //
 // Each of these is a matrix-vector product of a few MB, so the chain is bound by launch ramps, not by bytes.  Here the
-// step is ONE persistent launch.  Only W_ih[:, 0:H] . in_k depends on the layer before; W_hh . h_prev, the context
-// columns W_ih[:, H:2H] . ctx and layer 0's input product do not, so every block streams those for all layers at once
-// at the start, prefetches the dependent columns into registers, and the layers then hand their outputs over through
-// the flagged exchange described below, one round per layer.  The classifier streams after the last round.
+// step is ONE persistent launch that streams every weight once, in layer order, as fast as memory delivers it, while
+// the layers hand their outputs from block to block through a flagged exchange.
 //
-// Grid: NB = ceil(H / 4) blocks of 512 lanes, all resident at once (H <= 1024).  Block b owns hidden units 4b .. 4b+3 of
-// every layer; two wavefronts share a unit and split the columns of every weight row between them (lane l of a
-// wavefront holds one 16-byte piece of each row).  Accumulator slot v holds gate {i, g, f, o}[v], so that the
-// transpose-sum leaves gate k in lane k (as in the sequence kernel).
+// The context columns of W_ih need not be streamed at all while the encoder outputs stay the same (every step of one
+// sentence): W_ih[:, H:2H] . ctx = (W_ih[:, H:2H] . enc^T) . att, and the 4H x S matrix in brackets is computed once per
+// sentence by the input-projection kernel (pimhip_decoder_plan_set_encoder).  A step then reads S values per gate row
+// instead of H, and needs no context vector.  A caller that has the context instead passes it (ctx_in) and the columns
+// are streamed.
 //
-// Exchange: hx[stage][NB] entries of 64 bytes, of which a block uses the first 8: its four fp16 outputs of layer
-// `stage`.  |y| <= 1, so bit 14 of each fp16 carries a flag, the parity of the launch count g (a device word read at
-// the start and advanced by block 0 at the end): a slot written by launch g - 1 cannot pass for launch g, and the buffer
-// starts as zeros with g = 1.  A NaN (bit 14 set) travels as the otherwise unused pattern 0x3fff.  Every wait is bounded:
-// after `spin_limit` polls a lane raises the abort flags, all lanes stop waiting, the kernel runs to its end with
-// undefined results and the host reports a time-out.
+// Grid: NB = ceil(H / 4) blocks (H <= 1024), all resident at once, of kDecStreamWaves + kDecPollWaves wavefronts each.
+//   * Wavefronts 0..7 stream.  Block b owns hidden units 4b .. 4b+3 of every layer; two wavefronts share a unit and
+//     split the columns of every weight row between them (lane l holds one 16-byte piece of each row).  Their
+//     instruction stream holds no poll: loads return in order, so a poll behind a weight load could not be read before
+//     that load has arrived.  Layer 0's weights go out first and its gate sums are delivered as soon as they arrive;
+//     everything else that needs no other layer (W_hh . h_prev, the context term) is consumed as it arrives while layer
+//     0's output travels, and the columns that wait for the layer before sit in registers until that layer's output is
+//     there.  Each layer's four gate sums (slot v holds gate {i, g, f, o}[v], so that the transpose-sum leaves gate k in
+//     lane k) are left in LDS.
+//   * The other wavefronts hold no weights.  The first of them adds the partial sums of the block's four units,
+//     applies the gates (lanes 4u .. 4u+3 = the gates of unit u), stores the state and publishes the block's four
+//     outputs with one 8-byte store; all of them poll the other blocks' entries and put the layer's whole output into
+//     LDS for the streamers.
+// Two barriers per layer: gate sums ready, next input ready.  (All wavefronts of a CU share its path to memory, and a
+// load is served after every load issued before it: polls that are issued while weights are still queued are slow.  So
+// the layers' chain after layer 0 runs with the weights already in registers and little else in flight.)
+//
+// Exchange: hx[stage][NB] entries of 64 bytes: a block's four fp16 outputs of layer `stage` in the first 8 bytes.
+// |y| <= 1, so bit 14 of each fp16 carries a flag, the parity of the launch count g (a device word read at the start and
+// advanced by block 0 at the end): a slot written by launch g - 1 cannot pass for launch g, and the buffer starts as
+// zeros with g = 1.  A NaN (bit 14 set) travels as the otherwise unused pattern 0x3fff.  Every wait is bounded: after
+// `spin_limit` polls a lane raises the abort flags, all lanes stop waiting, the kernel runs to its end with undefined
+// results and the host reports a time-out.
 #pragma once
 
 #include "device_common.h"
@@ -35,10 +51,16 @@
 namespace pimhip
 {
 static constexpr int kDecMaxLayers = 4;
-static constexpr int kDecThreads = 512;
+static constexpr int kDecStreamWaves = 8;
+#ifndef PIMHIP_DEC_POLL_WAVES
+#define PIMHIP_DEC_POLL_WAVES 4
+#endif
+static constexpr int kDecPollWaves = PIMHIP_DEC_POLL_WAVES;   // 1, 2 or 4: each lane polls 4 / kDecPollWaves entries
+static constexpr int kDecThreads = 64 * (kDecStreamWaves + kDecPollWaves);
 static constexpr int kDecUnits = 4;          // hidden units per block
 static constexpr int kDecMaxH = 1024;        // 2 wavefronts x 64 lanes x 8 columns per row
 static constexpr int kDecEntryWords = 16;    // 32-bit words between the entries of consecutive blocks (64 bytes)
+static constexpr int kDecStages = kDecMaxLayers;      // exchange stages: one per layer
 static constexpr int kDecMaxCtxOuts = 4;
 static constexpr unsigned short kDecNanCode = 0x3fffu;
 
@@ -46,6 +68,7 @@ struct DecoderLayerArgs {
     const half_t* w_ih;    // [4H, in_w]
     const half_t* w_hh;    // [4H, H]
     const float* bsum;     // [4H] fp32, b_ih + b_hh
+    const float* cx_proj;  // [4H, S] fp32 = W_ih[:, H:2H] . enc^T, or null: then the context columns are streamed (ctx_in)
     const half_t* h_prev;  // [H]
     const half_t* c_prev;  // [H]
     half_t* hn;            // [H]
@@ -62,22 +85,36 @@ struct DecoderStepArgs {
     const half_t* x;       // input of layer 0 (without the context part), x_w elements
     int x_w;
     const half_t* ctx_in;  // [H] or null
-    const half_t* att;     // [S]: ctx = att . enc when ctx_in is null
-    const half_t* enc;     // [S, H]
-    int enc_len;
+    const half_t* att;     // [S] attention weights (with cx_proj; and for ctx_out)
+    const half_t* enc;     // [S, H] encoder outputs, only read for ctx_out
+    int enc_len;           // S
     half_t* ctx_out[kDecMaxCtxOuts];
     int n_ctx_out;
     const half_t* cls_w;   // [vocab, H] or null
     const half_t* cls_b;   // [vocab] or null
     half_t* logits;        // [vocab]
     int vocab;
-    unsigned int* hx;          // [kDecMaxLayers][NB][kDecEntryWords]
+    unsigned int* hx;          // [kDecStages][NB][kDecEntryWords]
     unsigned int* g_counter;   // launches this buffer has seen, plus 1
     unsigned int* abort_flag;
     unsigned int* abort_host;
     unsigned int spin_limit;
     int H;
+#ifdef PIMHIP_DECODER_TRACE
+    unsigned long long* trace;  // [blocks][16 wavefronts][32] timestamps (100 MHz), for tuning builds only
+#endif
 };
+
+#ifdef PIMHIP_DECODER_TRACE
+#define DEC_TRACE(slot)                                                                                            \
+    do {                                                                                                           \
+        if (p.trace && lane == 0) p.trace[((long)blockIdx.x * 16 + wave) * 32 + (slot)] = wall_clock64();           \
+    } while (0)
+#else
+#define DEC_TRACE(slot) \
+    do {                \
+    } while (0)
+#endif
 
 // Transpose-sum of four per-lane partial sums over the wavefront: lane l ends up with the total of slot
 // 2 * (l & 1) + ((l >> 1) & 1), i.e. with slots {0, 2, 1, 3} in lanes {0, 1, 2, 3} (and every lane with lane & 3 alike).
@@ -90,277 +127,438 @@ __device__ __forceinline__ float transpose_sum4(const float (&acc)[4], int lane)
     return wave_sum_mod4(a);
 }
 
+__device__ __forceinline__ unsigned int readlane_u32(unsigned int v, int l)
+{
+    return (unsigned int)__builtin_amdgcn_readlane((int)v, l);
+}
+
+// L = p.n_layers, a template parameter so that the order of loads and uses, and with it the lifetime of every register,
+// is fixed at compile time.
+template <int L>
 __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderStepArgs p)
 {
-    __shared__ __align__(16) half_t in_vec[kDecMaxH];   // the current layer's input without the context part
-    __shared__ __align__(16) half_t ctx_vec[kDecMaxH];
-    __shared__ float comb[kDecUnits][4];                // gate sums of the second wavefront of each unit
-    __shared__ __align__(8) unsigned short pub[kDecUnits];
+    static_assert(L >= 1 && L <= kDecMaxLayers, "layers per step");
+    static_assert(kDecPollWaves == 1 || kDecPollWaves == 2 || kDecPollWaves == 4, "entries per polling lane");
+    __shared__ __align__(16) half_t in_vec[kDecMaxH];                  // the current layer's input without the context part
+    __shared__ __align__(16) half_t ctx_vec[kDecMaxH];                 // a given context (ctx_in)
+    __shared__ __align__(16) half_t hprev[kDecMaxLayers][kDecMaxH];    // the previous hidden state of the layers after the first
+    __shared__ float part[kDecStreamWaves][4];                         // a layer's gate sums: [wavefront][gate]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int u = wave >> 1;   // unit of the block
-    const int hf = wave & 1;   // which half of every row's columns
     const int H = p.H;
     const int nb = gridDim.x;
-    const int j = blockIdx.x * kDecUnits + u;
-    const bool unit_ok = j < H;
-    const int jc = unit_ok ? j : H - 1;
-    const int L = p.n_layers;
     const bool has_cls = p.cls_w != nullptr;
-
-    const unsigned int g = __builtin_amdgcn_readfirstlane(__hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    const unsigned short flag = (unsigned short)((g & 1u) << 14);
-
-    // This wavefront's 16-byte piece of an H-wide row: pieces [0, n0) belong to half 0, [n0, nchunks) to half 1.
     const int nchunks = H >> 3;
-    const int n0 = (nchunks + 1) >> 1;
-    const int my_cnt = hf ? nchunks - n0 : n0;
-    const bool active = lane < my_cnt;
-    const int chunk = active ? (hf ? n0 : 0) + lane : 0;
-    const int gate_of_slot[4] = {0, 2, 1, 3};
+    bool any_ctx = false;
+#pragma unroll
+    for (int k = 0; k < L; ++k) any_ctx = any_ctx || p.layer[k].takes_ctx;
+    // a first layer that takes a given context needs it in LDS before its first product (one barrier more, for every wavefront)
+    const bool staged_ctx_first = p.ctx_in && p.layer[0].takes_ctx;
     half8_t zero8;
 #pragma unroll
     for (int e = 0; e < 8; ++e) zero8[e] = (half_t)0.0f;
+    DEC_TRACE(0);
 
-    // ---- 0a. everything that does not wait for another layer: first W_hh of every layer and its h_prev ----
-    half8_t w_a[kDecMaxLayers][4];
-    half8_t hvec[kDecMaxLayers];
-#pragma unroll
-    for (int k = 0; k < kDecMaxLayers; ++k) {
-        if (k < L) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-                w_a[k][v] = load_stream(reinterpret_cast<const half8_t*>(p.layer[k].w_hh + ((long)gate_of_slot[v] * H + jc) * H) + chunk);
-            hvec[k] = active ? reinterpret_cast<const half8_t*>(p.layer[k].h_prev)[chunk] : zero8;
-        }
-    }
+    if (wave < kDecStreamWaves) {
+        // =========================================== the streaming wavefronts ===========================================
+        const int u = wave >> 1;   // unit of the block
+        const int hf = wave & 1;   // which half of every row's columns
+        const int j = blockIdx.x * kDecUnits + u;
+        const int jc = j < H ? j : H - 1;
+        // This wavefront's 16-byte piece of an H-wide row: pieces [0, n0) belong to half 0, [n0, nchunks) to half 1.
+        const int n0 = (nchunks + 1) >> 1;
+        const int my_cnt = hf ? nchunks - n0 : n0;
+        const bool active = lane < my_cnt;
+        const int chunk = active ? (hf ? n0 : 0) + lane : 0;
+        const int gate_of_slot[4] = {0, 2, 1, 3};
+        // layer 0's input without the context: any width, split between the two halves like the rows
+        const int xw = p.layer[0].takes_ctx ? H : p.layer[0].in_w;
+        const int xchunks = xw >> 3;
+        const int xn0 = (xchunks + 1) >> 1;
+        const int x_begin = hf ? xn0 : 0, x_end = hf ? xchunks : xn0;
+        const bool x_one_piece = x_end - x_begin <= 64;
+        const bool x_active = lane < x_end - x_begin;
+        const int x_chunk = x_active ? x_begin + lane : 0;
 
-    // ---- 0b. the attention context, whole, in every block (S x H fp16 from the cache: cheaper than an exchange) ----
-    bool any_ctx = false;
+        // Weights per layer, one 16-byte piece of each of the four gate rows per lane, in two groups:
+        //   A(k): W_hh, the context term and, for layer 0, its input columns: what needs no other layer
+        //   D(k): the input columns of W_ih of a layer k >= 1, which wait for layer k - 1's output
+        half8_t w_hh[L][4], w_cx[L][4], w_in[L][4];
+        float m_cx[L][4];  // projected context: this unit's four gate rows of the layer's 4H x S matrix at position e_mine
+        half8_t xvec = zero8;
+        // the two wavefronts of a unit take alternate runs of 64 encoder positions: lane l the position 64 hf + l (+ 128 i)
+        const int S = p.enc_len;
+        const int e_mine = 64 * hf + lane;
+        const float att_mine = (any_ctx && p.att && e_mine < S) ? (float)p.att[e_mine] : 0.0f;
+        auto row_ptr = [&](const half_t* base, int v, long pitch, long col0) {
+            return reinterpret_cast<const half8_t*>(base + ((long)gate_of_slot[v] * H + jc) * pitch + col0);
+        };
+        auto issue_a = [&](int k) __attribute__((always_inline)) {
+            const DecoderLayerArgs& ly = p.layer[k];
 #pragma unroll
-    for (int k = 0; k < kDecMaxLayers; ++k) any_ctx = any_ctx || (k < L && p.layer[k].takes_ctx);
-    {
-        const int col = tid * 2;
-        if (col < H) {
-            if (any_ctx || p.n_ctx_out > 0) {
-                half2_t cv;
-                if (p.ctx_in) {
-                    cv = *reinterpret_cast<const half2_t*>(p.ctx_in + col);
+            for (int v = 0; v < 4; ++v) w_hh[k][v] = load_stream(row_ptr(ly.w_hh, v, H, 0) + chunk);
+            if (ly.takes_ctx) {
+                if (ly.cx_proj) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) m_cx[k][v] = ly.cx_proj[((long)gate_of_slot[v] * H + jc) * S + min(e_mine, S - 1)];
                 } else {
-                    float c0 = 0.0f, c1 = 0.0f;
-#pragma unroll 8
-                    for (int e = 0; e < p.enc_len; ++e) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) w_cx[k][v] = load_stream(row_ptr(ly.w_ih, v, ly.in_w, H) + chunk);
+                }
+            }
+            if (k == 0 && x_one_piece) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) w_in[0][v] = load_stream(row_ptr(ly.w_ih, v, ly.in_w, 0) + x_chunk);
+                if (x_active) xvec = reinterpret_cast<const half8_t*>(p.x)[x_chunk];
+            }
+        };
+        auto issue_d = [&](int k) __attribute__((always_inline)) {
+            const DecoderLayerArgs& ly = p.layer[k];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) w_in[k][v] = load_stream(row_ptr(ly.w_ih, v, ly.in_w, 0) + chunk);
+        };
+
+        // The classifier's rows are dealt to the streaming wavefronts of the whole grid four at a time.  A wavefront's first
+        // groups are fetched behind the layers' weights, the next ones as soon as the last layer's registers are free.
+        constexpr int CH = kDecMaxH / 8 / 64;  // 16-byte pieces of a classifier row per lane
+        const int gw = blockIdx.x * kDecStreamWaves + wave;
+        const int nw = nb * kDecStreamWaves;
+        const int V = p.vocab;
+        half8_t cbuf[4][4][CH];
+        auto cls_row0 = [&](int it) { return ((long)it * nw + gw) * 4; };
+        auto cls_issue = [&](half8_t (&dst)[4][CH], int it) __attribute__((always_inline)) {
+            const long r0 = cls_row0(it);
+            if (has_cls && r0 < V) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const long row = min(r0 + v, (long)V - 1);
+                    const half8_t* wp = reinterpret_cast<const half8_t*>(p.cls_w + row * H);
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) dst[v][c] = load_stream(wp + min(c * 64 + lane, nchunks - 1));
+                }
+            }
+        };
+        float acc[L][4];
+        auto consume_a = [&](int k, const half8_t& cvec, const half8_t& hv) __attribute__((always_inline)) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_hh[k][v], hv, 0.0f);
+            if (p.layer[k].takes_ctx) {
+                if (p.layer[k].cx_proj) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[k][v] = fmaf(att_mine, m_cx[k][v], acc[k][v]);
+                    for (int e = e_mine + 128; e < S; e += 128) {  // more than 128 encoder positions
                         const float a = (float)p.att[e];
-                        const half2_t ev = *reinterpret_cast<const half2_t*>(p.enc + (long)e * H + col);
-                        c0 = fmaf(a, (float)ev[0], c0);
-                        c1 = fmaf(a, (float)ev[1], c1);
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            acc[k][v] = fmaf(a, p.layer[k].cx_proj[((long)gate_of_slot[v] * H + jc) * S + e], acc[k][v]);
                     }
-                    cv[0] = (half_t)c0;
-                    cv[1] = (half_t)c1;
-                }
-                *reinterpret_cast<half2_t*>(&ctx_vec[col]) = cv;
-                if ((col >> 2) == (int)blockIdx.x) {
-                    for (int o = 0; o < p.n_ctx_out; ++o) *reinterpret_cast<half2_t*>(p.ctx_out[o] + col) = cv;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_cx[k][v], cvec, acc[k][v]);
                 }
             }
-            // layer 0's input, for its residual sum (only defined when it is H wide)
-            if (p.x_w == H) *reinterpret_cast<half2_t*>(&in_vec[col]) = *reinterpret_cast<const half2_t*>(p.x + col);
-        }
-    }
-    __syncthreads();
+        };
+        auto deliver = [&](int k) __attribute__((always_inline)) {
+            const float a = transpose_sum4(acc[k], lane);  // gate (lane & 3), this wavefront's half of the columns
+            if (lane < 4) part[wave][lane] = a;
+            DEC_TRACE(8 + 4 * k);
+            __syncthreads();  // B1: the gate sums of layer k are in LDS
+        };
 
-    // ---- 0c. W_hh . h_prev ----
-    float acc[kDecMaxLayers][4];
+        // Layer 0 waits for nothing but its own weights: its h_prev comes straight from memory, ahead of them.
+        const half8_t hv0 = active ? reinterpret_cast<const half8_t*>(p.layer[0].h_prev)[chunk] : zero8;
+        issue_a(0);
+        DEC_TRACE(1);
+        if (staged_ctx_first) __syncthreads();  // B0: a given context is in LDS (a first layer that takes it)
+        DEC_TRACE(2);
+        half8_t cvec = (staged_ctx_first && active) ? *reinterpret_cast<const half8_t*>(&ctx_vec[chunk * 8]) : zero8;
+        consume_a(0, cvec, hv0);
+        if (x_one_piece) {
 #pragma unroll
-    for (int k = 0; k < kDecMaxLayers; ++k) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[k][v] = (k < L) ? dot8(w_a[k][v], hvec[k], 0.0f) : 0.0f;
-    }
-
-    // ---- 0d. the context columns of W_ih ----
-    {
-        const half8_t cvec = active ? *reinterpret_cast<const half8_t*>(&ctx_vec[chunk * 8]) : zero8;
-#pragma unroll
-        for (int k = 0; k < kDecMaxLayers; ++k) {
-            if (k < L && p.layer[k].takes_ctx) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    w_a[k][v] = load_stream(reinterpret_cast<const half8_t*>(p.layer[k].w_ih + ((long)gate_of_slot[v] * H + jc) * p.layer[k].in_w + H) + chunk);
-            }
-        }
-        // ---- 0f. the columns that wait for the layer before: into registers now, used after that layer's exchange ----
-        half8_t w_dep[kDecMaxLayers - 1][4];
-#pragma unroll
-        for (int k = 1; k < kDecMaxLayers; ++k) {
-            if (k < L) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    w_dep[k - 1][v] = load_stream(reinterpret_cast<const half8_t*>(p.layer[k].w_ih + ((long)gate_of_slot[v] * H + jc) * p.layer[k].in_w) + chunk);
-            }
-        }
-        // ---- 0e. layer 0's own input columns (x is an argument of the step): any width, split between the halves ----
-        {
-            const int xw = p.layer[0].takes_ctx ? H : p.layer[0].in_w;
-            const int xchunks = xw >> 3;
-            const int x0 = (xchunks + 1) >> 1;
-            const int begin = hf ? x0 : 0, end = hf ? xchunks : x0;
+            for (int v = 0; v < 4; ++v) acc[0][v] = dot8(w_in[0][v], xvec, acc[0][v]);
+        } else {
+            // a first layer with a wide plain input: its columns in a loop
             const half8_t* xv = reinterpret_cast<const half8_t*>(p.x);
-            for (int c = begin + lane; c < end; c += 64) {
+            for (int c = x_begin + lane; c < x_end; c += 64) {
                 half8_t wr[4];
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    wr[v] = load_stream(reinterpret_cast<const half8_t*>(p.layer[0].w_ih + ((long)gate_of_slot[v] * H + jc) * p.layer[0].in_w) + c);
+                for (int v = 0; v < 4; ++v) wr[v] = load_stream(row_ptr(p.layer[0].w_ih, v, p.layer[0].in_w, 0) + c);
                 const half8_t xr = xv[c];
 #pragma unroll
                 for (int v = 0; v < 4; ++v) acc[0][v] = dot8(wr[v], xr, acc[0][v]);
             }
         }
+        deliver(0);
+        // everything else that needs no other layer goes out now and is consumed as it arrives, while layer 0's output travels
 #pragma unroll
-        for (int k = 0; k < kDecMaxLayers; ++k) {
-            if (k < L && p.layer[k].takes_ctx) {
+        for (int k = 1; k < L; ++k) issue_a(k);
+        // (after B1 of layer 0: every later layer's h_prev and a given context are in LDS)
+        if (p.ctx_in && active) cvec = *reinterpret_cast<const half8_t*>(&ctx_vec[chunk * 8]);
+        auto hv_of = [&](int k) { return active ? *reinterpret_cast<const half8_t*>(&hprev[k][chunk * 8]) : zero8; };
+        // The registers freed by each consumed group take the next loads: D(1..), then classifier rows.  A wavefront's first
+        // four groups of classifier rows go out at fixed points: kPre of them behind the layers' weights, then kPer after
+        // each later layer's gate sums (they travel while that layer's output is exchanged), the rest after the last layer.
+#ifndef PIMHIP_DEC_PRE
+#define PIMHIP_DEC_PRE 2
+#endif
+#ifndef PIMHIP_DEC_PER
+#define PIMHIP_DEC_PER 0
+#endif
+        constexpr int kPre = PIMHIP_DEC_PRE, kPer = PIMHIP_DEC_PER;
+        int cls_next = 0;  // (a compile-time value at every use: the code below is straight-line in L)
+        auto cls_prefetch = [&](int n) __attribute__((always_inline)) {
 #pragma unroll
-                for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_a[k][v], cvec, acc[k][v]);
+            for (int i = 0; i < 4; ++i) {
+                if (i < n && cls_next < 4) {
+                    if (cls_next == 0) cls_issue(cbuf[0], 0);
+                    if (cls_next == 1) cls_issue(cbuf[1], 1);
+                    if (cls_next == 2) cls_issue(cbuf[2], 2);
+                    if (cls_next == 3) cls_issue(cbuf[3], 3);
+                    ++cls_next;
+                }
+            }
+        };
+        if (L >= 2) {
+            consume_a(1, cvec, hv_of(1));
+            issue_d(1);
+            if (L >= 3) issue_d(2);
+        }
+        if (L >= 3) {
+            consume_a(2, cvec, hv_of(2));
+            if (L >= 4) issue_d(3);
+        }
+        if (L >= 4) consume_a(3, cvec, hv_of(3));
+        cls_prefetch(L == 1 ? 4 : kPre);
+        if (L > 1 || has_cls) {
+            __syncthreads();  // B3 of layer 0: its whole output (the next input) is in LDS
+            DEC_TRACE(10);
+        }
+#pragma unroll
+        for (int k = 1; k < L; ++k) {
+            const half8_t pv = active ? *reinterpret_cast<const half8_t*>(&in_vec[chunk * 8]) : zero8;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_in[k][v], pv, acc[k][v]);
+            deliver(k);
+            cls_prefetch(k + 1 == L ? 4 : kPer);
+            if (k + 1 < L || has_cls) {
+                __syncthreads();  // B3: the layer's whole output (the next input) is in LDS
+                DEC_TRACE(10 + 4 * k);
             }
         }
 
-        // ---- the layers, one exchange round each ----
-        bool gave_up = false;
-        half_t keep_h = (half_t)0.0f, keep_c = (half_t)0.0f;  // layer 0's new state, stored once every block has read h_prev
-        const int my_gate = lane & 3;
+        // ---- the classifier: logits = W_c . out_last + b_c ----
+        if (has_cls) {
+            half8_t vv[CH];
 #pragma unroll
-        for (int k = 0; k < kDecMaxLayers; ++k) {
-            if (k < L) {
-                const DecoderLayerArgs& ly = p.layer[k];
-                if (k > 0) {
-                    const half8_t pv = active ? *reinterpret_cast<const half8_t*>(&in_vec[chunk * 8]) : zero8;
+            for (int c = 0; c < CH; ++c) vv[c] = (c * 64 + lane < nchunks) ? *reinterpret_cast<const half8_t*>(&in_vec[(c * 64 + lane) * 8]) : zero8;
+            auto cls_finish = [&](const half8_t (&src)[4][CH], int it) __attribute__((always_inline)) {
+                const long r0 = cls_row0(it);
+                float s[4];
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_dep[k - 1][v], pv, acc[k][v]);
+                for (int v = 0; v < 4; ++v) {
+                    s[v] = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) s[v] = dot8(src[v][c], vv[c], s[v]);
                 }
-                float a = transpose_sum4(acc[k], lane);  // gate (lane & 3), this wavefront's half of the columns
-                if (hf == 1 && lane < 4) comb[u][lane] = a;
-                __syncthreads();
-                if (hf == 0) {
-                    a += comb[u][my_gate] + ly.bsum[(long)my_gate * H + jc];
-                    const bool is_g = my_gate == 2;
-                    const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
-                    const float act = is_g ? 2.0f * sg - 1.0f : sg;
-                    const float g_i = dpp_mov_f32<0x00>(act);
-                    const float g_f = dpp_mov_f32<0x55>(act);
-                    const float g_g = dpp_mov_f32<0xAA>(act);
-                    const float g_o = dpp_mov_f32<0xFF>(act);
-                    const float c_new = g_f * (float)ly.c_prev[jc] + g_i * g_g;
-                    const half_t h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
-                    if (lane == 0) {
-                        const bool is_number = (c_new == c_new) && (g_o == g_o);
-                        const unsigned short hbits = is_number ? __builtin_bit_cast(unsigned short, h_new) : kDecNanCode;
-                        pub[u] = unit_ok ? (unsigned short)(hbits | flag) : flag;
-                        if (unit_ok) {
-                            const bool later = k == 0 && (L > 1 || has_cls);
-                            if (later) {
-                                keep_h = h_new;
-                                keep_c = (half_t)c_new;
-                            } else {
-                                ly.hn[j] = h_new;
-                                ly.cn[j] = (half_t)c_new;
-                            }
-                            if (ly.out) {
-                                half_t o = h_new;
-                                if (ly.residual) o = (half_t)((float)h_new + (float)(k == 0 ? p.x[j] : in_vec[j]));
-                                ly.out[j] = o;
-                            }
-                        }
+                const float tot = transpose_sum4(s, lane);
+                if (lane < 4) {
+                    const long row = r0 + gate_of_slot[lane];  // lane l holds slot {0, 2, 1, 3}[l]
+                    if (row < V) {
+                        float r = tot;
+                        if (p.cls_b) r += (float)p.cls_b[row];
+                        p.logits[row] = (half_t)r;
                     }
                 }
-                __syncthreads();
-                if (k + 1 < L || has_cls) {
-                    unsigned long long* slot = reinterpret_cast<unsigned long long*>(p.hx + ((long)k * nb) * kDecEntryWords);
-                    if (tid == 0)
-                        __hip_atomic_store(slot + (long)blockIdx.x * (kDecEntryWords / 2), *reinterpret_cast<const unsigned long long*>(&pub[0]),
-                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (tid < nb) {
-                        const unsigned long long want = flag ? 0x4000400040004000ull : 0ull;
-                        unsigned long long word = 0ull;
-                        unsigned int spins = 0;
-                        while (true) {
-                            word = __hip_atomic_load(slot + (long)tid * (kDecEntryWords / 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                            if ((word & 0x4000400040004000ull) == want || gave_up) break;
-                            ++spins;
-                            if ((spins & 255u) == 0u) {
-                                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
-                            }
-                            if (spins >= p.spin_limit) {
-                                __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                                __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                                gave_up = true;
-                            }
-                        }
-                        // the four outputs of block `tid`; with a residual connection the next input is y + in
-                        half4_t nv;
-                        half4_t old;
+            };
+            if (cls_row0(0) < V) cls_finish(cbuf[0], 0);
+            cls_issue(cbuf[0], 4);
+            if (cls_row0(1) < V) cls_finish(cbuf[1], 1);
+            cls_issue(cbuf[1], 5);
+            if (cls_row0(2) < V) cls_finish(cbuf[2], 2);
+            if (cls_row0(3) < V) cls_finish(cbuf[3], 3);
+            for (int it = 4; cls_row0(it) < V; it += 2) {  // vocabularies beyond 16 rows per wavefront
+                cls_finish(cbuf[0], it);
+                cls_issue(cbuf[0], it + 2);
+                if (cls_row0(it + 1) >= V) break;
+                cls_finish(cbuf[1], it + 1);
+                cls_issue(cbuf[1], it + 3);
+            }
+        }
+        DEC_TRACE(25);
+    } else {
+        // ========================= the wavefronts that activate, publish and poll (no weights) =========================
+        const int pw = wave - kDecStreamWaves;         // 0: also activates and publishes
+        constexpr int QP = 4 / kDecPollWaves;          // entries polled per lane: blocks lane + 64 (pw * QP + q)
+        const unsigned int g = __hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // lanes 4u .. 4u+3 are the gates i, f, g, o of unit u of this block (lanes 16.. repeat them)
+        const int pu = (lane >> 2) & 3, pg = lane & 3;
+        const int pj = blockIdx.x * kDecUnits + pu;
+        const bool p_ok = pj < H;
+        const int pjc = p_ok ? pj : H - 1;
+        const bool owner = pw == 0 && pg == 0 && lane < 16 && p_ok;
+        float bias_r[L], cprev_r[L];
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) old[e] = in_vec[min(tid * 4 + e, kDecMaxH - 1)];
+        for (int k = 0; k < L; ++k) {
+            bias_r[k] = cprev_r[k] = 0.0f;
+            if (pw == 0) {
+                bias_r[k] = p.layer[k].bsum[(long)pg * H + pjc];
+                cprev_r[k] = (float)p.layer[k].c_prev[pjc];
+            }
+        }
+        // the later layers' h_prev, layer 0's input (for its residual sum, when it is H wide) and a given context into LDS
+        for (int c = pw * 64 + lane; c < nchunks; c += 64 * kDecPollWaves) {
+#pragma unroll
+            for (int k = 1; k < L; ++k) *reinterpret_cast<half8_t*>(&hprev[k][c * 8]) = reinterpret_cast<const half8_t*>(p.layer[k].h_prev)[c];
+            if (p.x_w == H) *reinterpret_cast<half8_t*>(&in_vec[c * 8]) = reinterpret_cast<const half8_t*>(p.x)[c];
+            if (p.ctx_in) *reinterpret_cast<half8_t*>(&ctx_vec[c * 8]) = reinterpret_cast<const half8_t*>(p.ctx_in)[c];
+        }
+        const unsigned short flag = (unsigned short)((g & 1u) << 14);
+        bool gave_up = false;
+        // one step of a bounded wait: true when the caller should stop waiting
+        auto give_up_check = [&](unsigned int& spins) {
+            ++spins;
+            if ((spins & 255u) == 0u) {
+                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
+            }
+            if (spins >= p.spin_limit) {
+                __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                gave_up = true;
+            }
+            return gave_up;
+        };
+
+        // ---- where the caller wants the attention context stored, this block stores its own four columns ----
+        if (pw == 0 && p.n_ctx_out > 0 && blockIdx.x * kDecUnits + kDecUnits <= H) {
+            const int col0 = blockIdx.x * kDecUnits;
+            if (p.ctx_in) {
+                if (lane < 2) {
+                    for (int o = 0; o < p.n_ctx_out; ++o)
+                        *reinterpret_cast<half2_t*>(p.ctx_out[o] + col0 + 2 * lane) = *reinterpret_cast<const half2_t*>(p.ctx_in + col0 + 2 * lane);
+                }
+            } else {
+                float cs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                for (int e = lane; e < p.enc_len; e += 64) {
+                    const float a = (float)p.att[e];
+                    const half2_t e01 = *reinterpret_cast<const half2_t*>(p.enc + (long)e * H + col0);
+                    const half2_t e23 = *reinterpret_cast<const half2_t*>(p.enc + (long)e * H + col0 + 2);
+                    cs[0] = fmaf(a, (float)e01[0], cs[0]);
+                    cs[1] = fmaf(a, (float)e01[1], cs[1]);
+                    cs[2] = fmaf(a, (float)e23[0], cs[2]);
+                    cs[3] = fmaf(a, (float)e23[1], cs[3]);
+                }
+                const float tot = transpose_sum4(cs, lane);  // lanes 0..3 hold columns {0, 2, 1, 3}
+                const unsigned int mine = (unsigned int)__builtin_bit_cast(unsigned short, (half_t)tot);
+                const unsigned int c0 = readlane_u32(mine, 0), c1 = readlane_u32(mine, 2), c2 = readlane_u32(mine, 1), c3 = readlane_u32(mine, 3);
+                if (lane < 2) {
+                    half2_t cv;
+                    cv[0] = __builtin_bit_cast(half_t, (unsigned short)(lane == 0 ? c0 : c2));
+                    cv[1] = __builtin_bit_cast(half_t, (unsigned short)(lane == 0 ? c1 : c3));
+                    for (int o = 0; o < p.n_ctx_out; ++o) *reinterpret_cast<half2_t*>(p.ctx_out[o] + col0 + 2 * lane) = cv;
+                }
+            }
+        }
+        DEC_TRACE(1);
+        if (staged_ctx_first) __syncthreads();  // B0
+        DEC_TRACE(2);
+
+        half_t keep_h = (half_t)0.0f, keep_c = (half_t)0.0f;  // layer 0's new state, stored once every block has read h_prev
+#pragma unroll
+        for (int k = 0; k < L; ++k) {
+            const DecoderLayerArgs& ly = p.layer[k];
+            __syncthreads();  // B1: the gate sums of layer k are in LDS
+            DEC_TRACE(8 + 4 * k);
+            const bool exchange = k + 1 < L || has_cls;
+            if (pw == 0) {
+                // (the streamers leave gate k in lane k, i.e. in part[.][k])
+                const float a = part[2 * pu][pg] + part[2 * pu + 1][pg] + bias_r[k];
+                const bool is_g = pg == 2;
+                const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
+                const float act = is_g ? 2.0f * sg - 1.0f : sg;
+                const float g_i = dpp_mov_f32<0x00>(act);
+                const float g_f = dpp_mov_f32<0x55>(act);
+                const float g_g = dpp_mov_f32<0xAA>(act);
+                const float g_o = dpp_mov_f32<0xFF>(act);
+                const float c_new = g_f * cprev_r[k] + g_i * g_g;
+                const half_t h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
+                const bool is_number = (c_new == c_new) && (g_o == g_o);
+                const unsigned int hbits = p_ok ? (unsigned int)((is_number ? __builtin_bit_cast(unsigned short, h_new) : kDecNanCode) | flag)
+                                                : (unsigned int)flag;
+                if (owner) {
+                    if (k == 0 && exchange) {
+                        keep_h = h_new;
+                        keep_c = (half_t)c_new;
+                    } else {
+                        ly.hn[pj] = h_new;
+                        ly.cn[pj] = (half_t)c_new;
+                    }
+                    if (ly.out) {
+                        half_t o = h_new;
+                        if (ly.residual) o = (half_t)((float)h_new + (float)in_vec[pj]);
+                        ly.out[pj] = o;
+                    }
+                }
+                DEC_TRACE(9 + 4 * k);
+                if (exchange) {
+                    unsigned long long* slot = reinterpret_cast<unsigned long long*>(p.hx + ((long)k * nb) * kDecEntryWords);
+                    const unsigned long long word = (unsigned long long)readlane_u32(hbits, 0) | ((unsigned long long)readlane_u32(hbits, 4) << 16) |
+                                                    ((unsigned long long)readlane_u32(hbits, 8) << 32) | ((unsigned long long)readlane_u32(hbits, 12) << 48);
+                    if (lane == 0)
+                        __hip_atomic_store(slot + (long)blockIdx.x * (kDecEntryWords / 2), word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            if (exchange) {
+                const unsigned long long* slot = reinterpret_cast<const unsigned long long*>(p.hx + ((long)k * nb) * kDecEntryWords);
+                const unsigned long long want = flag ? 0x4000400040004000ull : 0ull;
+                unsigned long long got[QP];
+#pragma unroll
+                for (int q = 0; q < QP; ++q) got[q] = want;
+                unsigned int spins = 0;
+                while (true) {
+                    bool ok = true;
+#pragma unroll
+                    for (int q = 0; q < QP; ++q) {
+                        const int blk = lane + 64 * (pw * QP + q);
+                        if (blk < nb)
+                            got[q] = __hip_atomic_load(const_cast<unsigned long long*>(slot) + (long)blk * (kDecEntryWords / 2), __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int q = 0; q < QP; ++q) ok = ok && (got[q] & 0x4000400040004000ull) == want;
+                    if (ok || gave_up) break;
+                    if (give_up_check(spins)) break;
+                }
+                // the outputs of this lane's blocks; with a residual connection the next input is y + in
+#pragma unroll
+                for (int q = 0; q < QP; ++q) {
+                    const int blk = lane + 64 * (pw * QP + q);
+                    if (blk < nb) {
+                        const half4_t old = *reinterpret_cast<const half4_t*>(&in_vec[blk * 4]);
+                        half4_t nv;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const unsigned short bits = (unsigned short)((word >> (16 * e)) & 0xbfffu);
+                            const unsigned short bits = (unsigned short)((got[q] >> (16 * e)) & 0xbfffu);
                             half_t yv = __builtin_bit_cast(half_t, bits);
                             if ((bits & 0x7fffu) == kDecNanCode) yv = __builtin_bit_cast(half_t, (unsigned short)0x7e00u);
                             nv[e] = ly.residual ? (half_t)((float)yv + (float)old[e]) : yv;
                         }
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (tid * 4 + e < H) in_vec[tid * 4 + e] = nv[e];
+                        *reinterpret_cast<half4_t*>(&in_vec[blk * 4]) = nv;
                     }
-                    __syncthreads();
-                    if (k == 0 && hf == 0 && lane == 0 && unit_ok) {
-                        // every block has published layer 0's output, so every block is past its reads of h_prev:
-                        // hn / cn may be the very buffers h_prev / c_prev were read from
-                        ly.hn[j] = keep_h;
-                        ly.cn[j] = keep_c;
-                    }
+                }
+                DEC_TRACE(10 + 4 * k);
+                __syncthreads();  // B3: the next input is in LDS
+                if (k == 0 && owner) {
+                    // every block has published layer 0's output, so every block is past its reads of h_prev:
+                    // hn / cn may be the very buffers h_prev / c_prev were read from
+                    ly.hn[pj] = keep_h;
+                    ly.cn[pj] = keep_c;
                 }
             }
         }
+        if (blockIdx.x == 0 && pw == 0 && lane == 0) __hip_atomic_store(p.g_counter, g + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-
-    // ---- the classifier: logits = W_c . out_last + b_c, rows dealt to the wavefronts of the whole grid four at a time ----
-    if (has_cls) {
-        const int gw = blockIdx.x * (kDecThreads / 64) + wave;
-        const int nw = nb * (kDecThreads / 64);
-        constexpr int CH = kDecMaxH / 8 / 64;  // 16-byte pieces of a row per lane
-        half8_t vv[CH];
-#pragma unroll
-        for (int c = 0; c < CH; ++c) vv[c] = (c * 64 + lane < nchunks) ? *reinterpret_cast<const half8_t*>(&in_vec[(c * 64 + lane) * 8]) : zero8;
-        const int V = p.vocab;
-        for (long r0 = (long)gw * 4; r0 < V; r0 += (long)nw * 4) {
-            half8_t wr[4][CH];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const long row = min(r0 + v, (long)V - 1);
-                const half8_t* wp = reinterpret_cast<const half8_t*>(p.cls_w + row * H);
-#pragma unroll
-                for (int c = 0; c < CH; ++c) wr[v][c] = (c * 64 + lane < nchunks) ? load_stream(wp + c * 64 + lane) : zero8;
-            }
-            float s[4];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                s[v] = 0.0f;
-#pragma unroll
-                for (int c = 0; c < CH; ++c) s[v] = dot8(wr[v][c], vv[c], s[v]);
-            }
-            const float tot = transpose_sum4(s, lane);
-            if (lane < 4) {
-                const long row = r0 + gate_of_slot[lane];  // lane l holds slot {0, 2, 1, 3}[l]
-                if (row < V) {
-                    float r = tot;
-                    if (p.cls_b) r += (float)p.cls_b[row];
-                    p.logits[row] = (half_t)r;
-                }
-            }
-        }
-    }
-    if (blockIdx.x == 0 && tid == 0) __hip_atomic_store(p.g_counter, g + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace pimhip

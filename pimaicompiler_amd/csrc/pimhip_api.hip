@@ -499,8 +499,10 @@ namespace
 {
 // out_p[T, N] = x[T, K] . w_p[N, K]^T + bias_p for p < count (1, or 2 for the two directions of a bidirectional layer).
 int launch_input_projection(int count, float* const* out, const half_t* x, const half_t* const* w, const float* const* bias,
-                            int64_t T, int64_t K, int64_t N, hipStream_t s)
+                            int64_t T, int64_t K, int64_t N, hipStream_t s, int64_t ldx = 0, int64_t ldw = 0)
 {
+    if (ldx == 0) ldx = K;
+    if (ldw == 0) ldw = K;
     if (T <= 0 || N <= 0) return PIMHIP_OK;
     if (K % 8 != 0 || !aligned16(x))
         return fail(PIMHIP_ERR_UNSUPPORTED, "input projection needs in_w %% 8 == 0 (got %lld) and 16-byte aligned x and w", (long long)K);
@@ -520,10 +522,10 @@ int launch_input_projection(int count, float* const* out, const half_t* x, const
     auto blocks = [&](int cols) { return (unsigned)(((N + cols - 1) / cols + 7) / 8 * 8) * row_blocks; };
     if (row_blocks >= 2) {
         pr.blocks_per_problem = (int)blocks(32);
-        input_projection_f16_kernel<2><<<blocks(32) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, (long)K, (int)row_blocks);
+        input_projection_f16_kernel<2><<<blocks(32) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)ldx, (long)ldw, (int)row_blocks);
     } else {
         pr.blocks_per_problem = (int)blocks(16);
-        input_projection_f16_kernel<1><<<blocks(16) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, (long)K, (int)row_blocks);
+        input_projection_f16_kernel<1><<<blocks(16) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)ldx, (long)ldw, (int)row_blocks);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(PIMHIP_ERR_HIP, "input projection launch failed: %s", hipGetErrorString(e));
@@ -1152,7 +1154,11 @@ struct PimHipDecoderPlan {
     const half_t* cls_w = nullptr;
     const half_t* cls_b = nullptr;
     float* bsum = nullptr;            // [num_layers][4H]
-    unsigned int* hx = nullptr;       // [kDecMaxLayers][blocks][kDecEntryWords], zero when *g_counter == 1
+    float* cx_proj = nullptr;         // [num_layers][4H][enc_cap] fp32: W_ih[:, H:2H] . enc^T of the layers that take the context
+    int64_t enc_cap = 0;              // encoder positions cx_proj has room for
+    const half_t* enc = nullptr;      // the encoder outputs the projection was made from (read again only for ctx_outs)
+    int64_t enc_len = 0;
+    unsigned int* hx = nullptr;       // [kDecStages][blocks][kDecEntryWords], zero when *g_counter == 1
     unsigned int* g_counter = nullptr;
     unsigned int* abort_flag = nullptr;
     unsigned int* abort_host = nullptr;
@@ -1172,6 +1178,7 @@ int destroy_decoder_plan_locked(PimHipDecoderPlan* plan)
     hipSetDevice(plan->device);
     hipDeviceSynchronize();
     if (plan->bsum) hipFree(plan->bsum);
+    if (plan->cx_proj) hipFree(plan->cx_proj);
     if (plan->hx) hipFree(plan->hx);
     if (plan->g_counter) hipFree(plan->g_counter);
     if (plan->abort_flag) hipFree(plan->abort_flag);
@@ -1226,7 +1233,7 @@ extern "C" int pimhip_decoder_plan_create(PimHipDecoderPlan** plan_out, const vo
 
     const int blocks = (int)((H + kDecUnits - 1) / kDecUnits);
     int per_cu = 0;
-    PIMHIP_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decoder_step_f16_kernel, kDecThreads, 0));
+    PIMHIP_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decoder_step_f16_kernel<kDecMaxLayers>, kDecThreads, 0));
     if ((int64_t)per_cu * st->num_cus < blocks)
         return fail(PIMHIP_ERR_UNSUPPORTED, "the %d blocks of the decoder step cannot all be resident on this device", blocks);
 
@@ -1265,7 +1272,7 @@ extern "C" int pimhip_decoder_plan_create(PimHipDecoderPlan** plan_out, const vo
                                                                              plan->bsum + (size_t)l * 4 * H, (int)(4 * H));
     }
     DEC_HIP_CHECK(hipGetLastError());
-    const size_t words = (size_t)kDecMaxLayers * blocks * kDecEntryWords;
+    const size_t words = (size_t)kDecStages * blocks * kDecEntryWords;
     DEC_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned int)));
     fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->hx, words, 0u);
     DEC_HIP_CHECK(hipMalloc(&plan->g_counter, sizeof(unsigned int)));
@@ -1286,6 +1293,18 @@ extern "C" int pimhip_decoder_plan_create(PimHipDecoderPlan** plan_out, const vo
     return PIMHIP_OK;
 }
 
+#ifdef PIMHIP_DECODER_TRACE
+namespace
+{
+unsigned long long* g_decoder_trace = nullptr;
+}
+extern "C" int pimhip_decoder_debug_set_trace(void* buffer)
+{
+    g_decoder_trace = static_cast<unsigned long long*>(buffer);
+    return PIMHIP_OK;
+}
+#endif
+
 extern "C" int pimhip_decoder_plan_destroy(PimHipDecoderPlan* plan)
 {
     if (!plan) return PIMHIP_OK;
@@ -1294,6 +1313,49 @@ extern "C" int pimhip_decoder_plan_destroy(PimHipDecoderPlan* plan)
     for (PimHipDecoderPlan* q : g_decoder_plans) known = known || (q == plan);
     if (!known) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "unknown or already destroyed decoder plan");
     return destroy_decoder_plan_locked(plan);
+}
+
+extern "C" int pimhip_decoder_plan_set_encoder(PimHipDecoderPlan* plan, const void* enc, int64_t enc_len, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    int dev = -1;
+    PIMHIP_HIP_CHECK(hipGetDevice(&dev));
+    if (dev != plan->device) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan belongs to device %d, current device is %d", plan->device, dev);
+    if (!enc || enc_len < 1 || enc_len > INT32_MAX / 8) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "enc must be non-null and enc_len positive");
+    if (!aligned16(enc)) return fail(PIMHIP_ERR_UNSUPPORTED, "enc must be 16-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t H = plan->hidden;
+    const int L = plan->num_layers;
+    if (enc_len > plan->enc_cap) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
+        if (capture != hipStreamCaptureStatusNone)
+            return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's projection buffer has to grow for %lld encoder positions, which a graph must not "
+                                                "record: call pimhip_decoder_plan_set_encoder once with that length before the capture", (long long)enc_len);
+        PIMHIP_HIP_CHECK(hipStreamSynchronize(s));  // steps already queued may still read the old buffer
+        if (plan->cx_proj) PIMHIP_HIP_CHECK(hipFree(plan->cx_proj));
+        plan->cx_proj = nullptr;
+        plan->enc_cap = 0;
+        int64_t cap = enc_len < 64 ? 64 : enc_len;
+        PIMHIP_HIP_CHECK(hipMalloc(&plan->cx_proj, sizeof(float) * (size_t)L * cap * 4 * H));
+        plan->enc_cap = cap;
+    }
+    for (int l = 0; l < L; ++l) {
+        if (!(l > 0 || plan->first_takes_context)) continue;
+        // out[4H, S] = W_ih[:, H:2H] (4H rows of pitch 2H) . enc[S, H]^T: the kernel's "x" is the weight, its "w" the encoder
+        // outputs, so that a gate row's S values are contiguous for the step kernel
+        float* out = plan->cx_proj + (size_t)l * plan->enc_cap * 4 * H;
+        const half_t* w = (const half_t*)enc;
+        const float* no_bias = nullptr;
+        rc = launch_input_projection(1, &out, plan->w_ih[l] + H, &w, &no_bias, 4 * H, H, enc_len, s, 2 * H, H);
+        if (rc != PIMHIP_OK) return rc;
+    }
+    plan->enc = (const half_t*)enc;
+    plan->enc_len = enc_len;
+    return PIMHIP_OK;
 }
 
 extern "C" int pimhip_decoder_plan_set_spin_limit(PimHipDecoderPlan* plan, unsigned int spin_limit)
@@ -1314,8 +1376,8 @@ extern "C" int pimhip_decoder_plan_status(PimHipDecoderPlan* plan)
     return PIMHIP_OK;
 }
 
-extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const void* att, const void* enc, int64_t enc_len,
-                                   const void* ctx_in, const void* const* h_prev, const void* const* c_prev, void* const* hn,
+extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const void* att, const void* ctx_in,
+                                   const void* const* h_prev, const void* const* c_prev, void* const* hn,
                                    void* const* cn, void* const* layer_outs, void* const* ctx_outs, int n_ctx_outs, void* logits,
                                    void* stream)
 {
@@ -1335,13 +1397,13 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
     if (n_ctx_outs < 0 || n_ctx_outs > kDecMaxCtxOuts) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "n_ctx_outs=%d not in [0, %d]", n_ctx_outs, kDecMaxCtxOuts);
     if (n_ctx_outs > 0 && !ctx_outs) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "ctx_outs is null");
     if ((any_ctx || n_ctx_outs > 0) && !ctx_in) {
-        if (!att || !enc) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "the context needs ctx_in, or att and enc");
-        if (enc_len < 0 || enc_len > INT32_MAX) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "enc_len=%lld out of range", (long long)enc_len);
+        if (!att) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "the context needs ctx_in, or att");
+        if (plan->enc_len < 1)
+            return fail(PIMHIP_ERR_INVALID_ARGUMENT, "att needs the encoder outputs: call pimhip_decoder_plan_set_encoder first (once per sentence)");
     }
     if (plan->cls_w && !logits) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "logits must be non-null for a plan with a classifier");
     if (!aligned16(x)) return fail(PIMHIP_ERR_UNSUPPORTED, "x must be 16-byte aligned");
     if (ctx_in && (reinterpret_cast<uintptr_t>(ctx_in) & 3u)) return fail(PIMHIP_ERR_UNSUPPORTED, "ctx_in must be 4-byte aligned");
-    if (enc && (reinterpret_cast<uintptr_t>(enc) & 3u)) return fail(PIMHIP_ERR_UNSUPPORTED, "enc must be 4-byte aligned");
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
@@ -1360,7 +1422,7 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
         if (capturing)
             return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's exchange buffer has to be re-initialised after a time-out, which a graph must not "
                                                 "record: run one step outside the capture first");
-        const size_t words = (size_t)kDecMaxLayers * plan->blocks * kDecEntryWords;
+        const size_t words = (size_t)kDecStages * plan->blocks * kDecEntryWords;
         fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->hx, words, 0u);
         fill_u32_kernel<<<1, 64, 0, s>>>(plan->g_counter, 1, 1u);
         fill_u32_kernel<<<1, 64, 0, s>>>(plan->abort_flag, 1, 0u);
@@ -1384,6 +1446,7 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
         ly.cn = (half_t*)cn[l];
         ly.out = layer_outs ? (half_t*)layer_outs[l] : nullptr;
         ly.takes_ctx = (l > 0 || plan->first_takes_context) ? 1 : 0;
+        ly.cx_proj = (ly.takes_ctx && !ctx_in) ? plan->cx_proj + (size_t)l * plan->enc_cap * 4 * H : nullptr;
         ly.in_w = (int)(l == 0 ? (plan->first_takes_context ? 2 * H : plan->input_size) : 2 * H);
         ly.residual = l >= plan->first_residual_layer ? 1 : 0;
     }
@@ -1392,9 +1455,9 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
     a.x = (const half_t*)x;
     a.x_w = (int)plan->input_size;
     a.ctx_in = (const half_t*)ctx_in;
-    a.att = (const half_t*)att;
-    a.enc = (const half_t*)enc;
-    a.enc_len = (int)enc_len;
+    a.att = ctx_in ? nullptr : (const half_t*)att;
+    a.enc = plan->enc;
+    a.enc_len = ctx_in ? 0 : (int)plan->enc_len;
     a.n_ctx_out = n_ctx_outs;
     for (int o = 0; o < n_ctx_outs; ++o) {
         if (!ctx_outs[o] || (reinterpret_cast<uintptr_t>(ctx_outs[o]) & 3u)) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "ctx_outs[%d] is null or not 4-byte aligned", o);
@@ -1410,12 +1473,20 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
     a.abort_host = plan->abort_host_dev;
     a.spin_limit = plan->spin_limit;
     a.H = (int)H;
+#ifdef PIMHIP_DECODER_TRACE
+    a.trace = g_decoder_trace;
+#endif
     // All blocks have to be resident at once, like the sequence kernel's: ordered after it on other streams.
     if (!capturing) {
         rc = order_after_previous_sequence_launch(st, s);
         if (rc != PIMHIP_OK) return rc;
     }
-    decoder_step_f16_kernel<<<plan->blocks, kDecThreads, 0, s>>>(a);
+    switch (L) {
+        case 1: decoder_step_f16_kernel<1><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
+        case 2: decoder_step_f16_kernel<2><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
+        case 3: decoder_step_f16_kernel<3><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
+        default: decoder_step_f16_kernel<4><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
+    }
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
 }

@@ -599,6 +599,21 @@ class DecoderPlan:
             self.cls_b.data_ptr() if self.cls_b is not None else None, self.vocab, _stream_handle(stream)))
         self._handle = handle
         self._finalizer = weakref.finalize(self, DecoderPlan._destroy, handle.value)
+        self._enc = None
+        self._enc_key = None
+
+    def set_encoder(self, enc, stream=None):
+        """Once per sentence: enc [S, H], the encoder outputs the attention weights of the following steps refer to.
+        Multiplies the context columns of every layer's W_ih with enc (pimhip_decoder_plan_set_encoder); the plan keeps
+        enc alive.  A call with the tensor (and version) it already has does nothing."""
+        _require_half_cuda(enc)
+        if enc.dim() != 2 or enc.size(1) != self.hidden or not enc.is_contiguous():
+            raise NNRuntimeException(f"enc must be a contiguous [S, {self.hidden}] tensor")
+        key = (enc.data_ptr(), enc._version, enc.size(0))
+        if key == self._enc_key:
+            return
+        _check(L.load().pimhip_decoder_plan_set_encoder(self._handle, enc.data_ptr(), enc.size(0), _stream_handle(stream)))
+        self._enc, self._enc_key = enc, key
 
     @staticmethod
     def _destroy(handle_value):
@@ -618,7 +633,9 @@ class DecoderPlan:
     def bind(self, x, h_prev, c_prev, att=None, enc=None, ctx=None, hn=None, cn=None, outs=None, ctx_outs=(), logits=None):
         """Fixes the buffers of a step (lists of [H] tensors per layer; hn / cn default to h_prev / c_prev, i.e. the state is
         updated in place) and returns a callable step(stream=None) that launches it without touching Python tensors
-        again: what a decoder loop or a graph capture calls per step."""
+        again: what a decoder loop or a graph capture calls per step.  The context comes from `att` [S], the attention
+        weights over the encoder outputs (`enc`, handed to set_encoder here unless it is the tensor the plan already has),
+        or from `ctx` [H], a context computed elsewhere."""
         lib = L.load()
         n, H = self.num_layers, self.hidden
         hn = list(h_prev) if hn is None else list(hn)
@@ -639,11 +656,11 @@ class DecoderPlan:
                 raise NNRuntimeException(f"state, output and context vectors must have {H} elements")
         if x.numel() != self.input_size:
             raise NNRuntimeException(f"x must have {self.input_size} elements")
-        enc_len = 0
         if ctx is None and att is not None:
-            enc_len = att.numel()
-            if enc is None or enc.numel() != enc_len * H:
-                raise NNRuntimeException("enc must be [len(att), H]")
+            if enc is not None:
+                self.set_encoder(enc.reshape(-1, H))
+            if self._enc is None or self._enc.size(0) != att.numel():
+                raise NNRuntimeException("att needs encoder outputs [len(att), H]: pass enc or call set_encoder first")
         if self.vocab and (logits is None or logits.numel() != self.vocab):
             raise NNRuntimeException(f"logits must have {self.vocab} elements")
         mk = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() if t is not None else None for t in ts])  # noqa: E731
@@ -651,8 +668,7 @@ class DecoderPlan:
         a_ctx = mk(list(ctx_outs)) if ctx_outs else None
         keep = (vecs, a_hp, a_cp, a_hn, a_cn, a_out, a_ctx)
         ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
-        args = (self._handle, ptr(x), ptr(att), ptr(enc), enc_len, ptr(ctx), a_hp, a_cp, a_hn, a_cn, a_out, a_ctx, len(ctx_outs),
-                ptr(logits))
+        args = (self._handle, ptr(x), ptr(att), ptr(ctx), a_hp, a_cp, a_hn, a_cn, a_out, a_ctx, len(ctx_outs), ptr(logits))
 
         def step(stream=None, _keep=keep):
             _check(lib.pimhip_decoder_step(*args, _stream_handle(stream)))
