@@ -1233,7 +1233,7 @@ extern "C" int pimhip_decoder_plan_create(PimHipDecoderPlan** plan_out, const vo
 
     const int blocks = (int)((H + kDecUnits - 1) / kDecUnits);
     int per_cu = 0;
-    PIMHIP_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decoder_step_f16_kernel<kDecMaxLayers>, kDecThreads, 0));
+    PIMHIP_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decoder_step_f16_kernel<kDecMaxLayers, true>, kDecThreads, 0));
     if ((int64_t)per_cu * st->num_cus < blocks)
         return fail(PIMHIP_ERR_UNSUPPORTED, "the %d blocks of the decoder step cannot all be resident on this device", blocks);
 
@@ -1481,11 +1481,21 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
         rc = order_after_previous_sequence_launch(st, s);
         if (rc != PIMHIP_OK) return rc;
     }
-    switch (L) {
-        case 1: decoder_step_f16_kernel<1><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
-        case 2: decoder_step_f16_kernel<2><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
-        case 3: decoder_step_f16_kernel<3><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
-        default: decoder_step_f16_kernel<4><<<plan->blocks, kDecThreads, 0, s>>>(a); break;
+    const dim3 grid(plan->blocks), block(kDecThreads);
+    if (plan->cls_w) {
+        switch (L) {
+            case 1: decoder_step_f16_kernel<1, true><<<grid, block, 0, s>>>(a); break;
+            case 2: decoder_step_f16_kernel<2, true><<<grid, block, 0, s>>>(a); break;
+            case 3: decoder_step_f16_kernel<3, true><<<grid, block, 0, s>>>(a); break;
+            default: decoder_step_f16_kernel<4, true><<<grid, block, 0, s>>>(a); break;
+        }
+    } else {
+        switch (L) {
+            case 1: decoder_step_f16_kernel<1, false><<<grid, block, 0, s>>>(a); break;
+            case 2: decoder_step_f16_kernel<2, false><<<grid, block, 0, s>>>(a); break;
+            case 3: decoder_step_f16_kernel<3, false><<<grid, block, 0, s>>>(a); break;
+            default: decoder_step_f16_kernel<4, false><<<grid, block, 0, s>>>(a); break;
+        }
     }
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
