@@ -210,6 +210,13 @@ int pimhip_pack_projection_weight(void* packed, const void* w, int64_t in_w, int
 int pimhip_input_projection_packed(void* out, const void* x, const void* packed, const void* bias, int64_t seq_len,
                                    int64_t in_w, int64_t n_out, void* stream);
 
+/* ---- measurement ----------------------------------------------------------------------------- */
+
+/* No counterpart in the reference.  Reads `bytes` bytes (a multiple of 16, 16-byte aligned) once with the streaming loads
+ * of the GEMV kernels and keeps nothing: what one launch of it takes is the floor for any kernel that has to read
+ * those bytes, launch included.  The benchmark reports each GEMV beside it. */
+int pimhip_probe_stream_read(const void* data, int64_t bytes, void* stream);
+
 /* ---- decoder step ---------------------------------------------------------------------------- */
 
 typedef struct PimHipDecoderPlan PimHipDecoderPlan;

@@ -26,6 +26,7 @@ SIGNATURES = {
     "pimhip_execute_gemv_static": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                   ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_void_p]),
+    "pimhip_probe_stream_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
     "pimhip_execute_dot": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                           ctypes.c_void_p]),
     "pimhip_execute_gemv_group": (ctypes.c_int, [ctypes.c_int, c_void_pp, c_void_pp, c_void_pp, c_void_pp,

@@ -438,6 +438,27 @@ __global__ __launch_bounds__(256) void add_f16_generic_kernel(const half_t* A, c
 }
 
 // ---------------------------------------------------------------------------------------------
+// Measurement aid: reads n16 16-byte pieces with the same streaming loads the GEMV kernels use and keeps nothing
+// (the sum only exists so that the loads are not removed; `sink` is written if it equals an impossible value).  What
+// a launch of this kernel takes is the floor for any kernel that has to read the same bytes once.
+// ---------------------------------------------------------------------------------------------
+typedef float float4_probe_t __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void stream_read_probe_kernel(const float4_probe_t* __restrict__ data, long n16, float* sink)
+{
+    constexpr int U = 8;
+    float s = 0.0f;
+    const long stride = (long)gridDim.x * 256 * U;
+    for (long base = (long)blockIdx.x * 256 * U + threadIdx.x; base < n16; base += stride) {
+        float4_probe_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(data + min(base + (long)u * 256, n16 - 1));
+#pragma unroll
+        for (int u = 0; u < U; ++u) s += v[u][0] + v[u][3];
+    }
+    if (s == 1234.5f && sink) sink[0] = s;
+}
+
+// ---------------------------------------------------------------------------------------------
 // VV: y[0] = sum_k a[k] * b[k].  One block of 1024 lanes; any K and alignment.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void dot_f16_kernel(const half_t* __restrict__ a, const half_t* __restrict__ b,

@@ -435,6 +435,21 @@ extern "C" int pimhip_execute_add(void* c, const void* a, const void* b, int64_t
     return PIMHIP_OK;
 }
 
+extern "C" int pimhip_probe_stream_read(const void* data, int64_t bytes, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!data || bytes < 16 || bytes % 16 != 0 || !aligned16(data))
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "data must be 16-byte aligned and bytes a positive multiple of 16");
+    const long n16 = (long)(bytes / 16);
+    long grid = (n16 + 2047) / 2048;
+    if (grid > 4L * st->num_cus) grid = 4L * st->num_cus;
+    stream_read_probe_kernel<<<(unsigned)grid, 256, 0, static_cast<hipStream_t>(stream)>>>((const float4_probe_t*)data, n16, nullptr);
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
 extern "C" int pimhip_execute_dot(void* out, const void* a, const void* b, int64_t in_w, void* stream)
 {
     DeviceState* st = nullptr;

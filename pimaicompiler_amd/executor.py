@@ -177,6 +177,37 @@ class StreamExecutor:
     def update_blob(self, blob_id, dtype, value):
         self.global_blobs[blob_id] = (dtype, value)
 
+    def preload_constants(self, constants):
+        """The prim::Constant pass of preProcess (stream_executor.cpp:59-134, prim_ops_executor.cpp:101): constant tensors
+        go to the GPU and into the blob store once.
+
+        A 2-D constant that the graph uses only as the right operand of addmm / matmul (y = x . A, the I_X_W order, A
+        stored [in, out]) is kept TRANSPOSED in memory behind the same logical shape and values: every later product
+        then streams contiguous rows with the W_X_I kernel instead of the column-sliced I_X_W one, at no cost per call,
+        where the reference makes such operands contiguous on every call (aten_ops.cpp:630-632).  Returns the ids whose
+        layout was changed."""
+        right, other = set(), set()
+        for layer in _flatten(self.layers):
+            ids = list(layer.in_stensor_ids)
+            if layer.type == LayerType.ATENADDMM and len(ids) >= 3:
+                right.add(ids[2])
+                other.update(ids[:2])
+            elif layer.type == LayerType.ATENMATMUL and len(ids) >= 2:
+                right.add(ids[1])
+                other.add(ids[0])
+            else:
+                other.update(ids)
+        relaid = []
+        dev = torch.device("cuda", self.device) if isinstance(self.device, int) else self.device
+        for blob_id, t in constants.items():
+            t = t.to(dev)
+            if blob_id in right and blob_id not in other and t.dim() == 2 and t.dtype == torch.float16 and t.is_contiguous() \
+                    and min(t.shape) > 1:
+                t = t.t().contiguous().t()   # [in, out] with strides (1, in): the same values, rows of A^T contiguous
+                relaid.append(blob_id)
+            self.update_blob(blob_id, DataType.TENSOR, t)
+        return relaid
+
     def find_blob(self, blob_id):
         return self.global_blobs.get(blob_id, (DataType.UNDEFINED, None))
 

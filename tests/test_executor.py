@@ -320,6 +320,32 @@ def test_addmm_vm_order_and_none_bias(ops):
 
 
 @pytest.mark.gpu
+def test_constant_weights_of_the_vm_order_are_laid_out_once_at_preload(ops):
+    """preload_constants keeps a constant right operand of addmm / matmul transposed in memory behind the same shape and
+    values: the products take the W_X_I kernel on it and agree with the products on the row-major original (both within
+    the GEMV tolerance of the oracle); constants with another use keep their layout."""
+    W, x, b = workloads.gemv_inputs(4, 1024, 512)
+    A = W.t().contiguous()                                   # [in, out], the operand of y = x . A
+    layers = [E.AtenAddmmLayer(LayerType.ATENADDMM, 0, [0, 1, 2], [5]), E.NNLayer(LayerType.ATENMATMUL, 0, [1, 2], [6]),
+              E.NNLayer(LayerType.ATENMATMUL, 0, [3, 1], [7])]            # blob 3 is a left operand too: untouched
+    ex = E.StreamExecutor(layers, device=0)
+    relaid = ex.preload_constants({0: b, 2: A, 3: W})
+    assert relaid == [2]
+    a_dev = ex.find_blob(2)[1]
+    assert list(a_dev.shape) == [512, 1024] and a_dev.stride() == (1, 512) and torch.equal(a_dev.cpu(), A)
+    assert ex.find_blob(3)[1].is_contiguous()
+    ex.update_blob(1, DataType.TENSOR, x.to(DEV))
+    E.execute_aten_addmm(layers[0], ex)
+    E.execute_aten_matmul(layers[1], ex)
+    want = oracle.gemv_vm(x.numpy().reshape(-1), A.numpy(), b.numpy())
+    assert list(ex.find_blob(5)[1].shape) == [1, 1024] and maxabs(ex.find_blob(5)[1], want) <= TOL_GEMV
+    assert maxabs(ex.find_blob(6)[1], oracle.gemv_vm(x.numpy().reshape(-1), A.numpy(), None)) <= TOL_GEMV
+    # the same product on the row-major original (the I_X_W kernel)
+    direct = ops.custom_aten_addmm("none", b.to(DEV), x.to(DEV), A.to(DEV))
+    assert maxabs(direct, want) <= TOL_GEMV
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("bidirectional,num_layers", [(False, 2), (True, 1)])
 def test_lstm1_layer_with_flags_from_blobs(ops, bidirectional, num_layers):
     params, x, h0, c0 = workloads.lstm_inputs(11, 64, 128, num_layers, bidirectional, 9)
