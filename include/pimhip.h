@@ -210,6 +210,17 @@ int pimhip_pack_projection_weight(void* packed, const void* w, int64_t in_w, int
 int pimhip_input_projection_packed(void* out, const void* x, const void* packed, const void* bias, int64_t seq_len,
                                    int64_t in_w, int64_t n_out, void* stream);
 
+/* No counterpart in the reference (the PIM SDK's PimExecuteGemm reports nothing either, aten_ops.cpp:659).
+ * A sliced I_X_W product whose reducing blocks gave up waiting for partial sums (a bounded wait: other work kept
+ * part of the GPU from running the blocks that produce them) is reported by the NEXT sliced product on that stream,
+ * which returns PIMHIP_ERR_TIMEOUT.  A caller that wants to know before it uses the result synchronises the stream and
+ * asks here: *gave_up gets bit 0 if a product of pimhip_execute_gemv / _bmm on `stream` gave up since the last
+ * re-initialisation, bit 1 if one of pimhip_execute_gemv_static on this GPU did.  Nothing is cleared.
+ * pimhip_set_gemv_spin_limit sets the number of polls per record for the current GPU (default 2^22, seconds); with 0 a
+ * reducing block gives up without polling, which is how tests force the condition while every kernel still ends. */
+int pimhip_gemv_status(void* stream, int* gave_up);
+int pimhip_set_gemv_spin_limit(unsigned int spin_limit);
+
 /* ---- measurement ----------------------------------------------------------------------------- */
 
 /* No counterpart in the reference.  Reads `bytes` bytes (a multiple of 16, 16-byte aligned) once with the streaming loads

@@ -28,4 +28,7 @@ from .ops import (  # noqa: F401
     DecoderPlan,
     prepare_lstm,
     invalidate_lstm_plans,
+    gemv_status,
+    synchronize_and_check,
+    set_gemv_spin_limit,
 )

@@ -197,10 +197,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_generic_kernel(const h
 // the reducing block polls each record until none of its words is kVmEmpty, adds it and writes kVmEmpty back for the
 // next launch.  Records travel with device-scope (sc1) stores and loads; there is no fence (a device-scope fence writes
 // back and invalidates the XCD's whole L2, once per block) and no ticket counter (store, acknowledgement, atomic,
-// loads would be three trips through the memory side after the last block's arithmetic; polling is one).  Blocks are
-// dispatched in order of their linear id, so the reducing blocks start last; the producers never wait for anything, so
-// they finish whatever else occupies the GPU.  A wait still is bounded: after `spin_limit` polls the lane sets *status
-// (host-visible) and goes on with what it has; the host then reports the failure and re-initialises the records.
+// loads would be three trips through the memory side after the last block's arithmetic; polling is one).
+//
+// What the scheme assumes of the dispatcher, and what it does not: the producers never wait for anything, so each of
+// them finishes whatever else occupies the GPU, in any dispatch order; results never depend on the order.  That the
+// reducing blocks seldom wait long does: workgroups are dealt to the eight XCDs round-robin by linear id and each
+// XCD starts its share in that order, so within every XCD the producers (slices 0..last-1) are started before that
+// XCD's reducing blocks (the last slice), and a reducing block on one XCD waits at most for the other XCDs to get
+// through the producers dealt to them.  When other work holds CUs of one XCD (a resident sequence kernel on another
+// stream) that wait grows by as much as that XCD is held up.  It is bounded all the same: after `spin_limit` polls
+// of one record (none at all with a limit of 0, which is how a test forces the condition from the host) the lane
+// sets *status (host-visible) and goes on with what it has; the host then reports the failure and re-initialises
+// the records.
 // ---------------------------------------------------------------------------------------------
 // Destinations of a VM product: the same result is stored to `count` buffers (the GNMT attention context goes
 // straight into three concatenation buffers, runtime/source/executor/op_executor/aten_ops_executor.cpp:694-737).
@@ -331,16 +339,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
             float4_t lo, hi;
             unsigned int spins = 0;
             while (true) {
+                if (spins++ >= spin_limit) {
+                    __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    lo = hi = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                    break;
+                }
                 load32_device_scope_one(rec, lo, hi);
                 bool ok = true;
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     ok = ok && __builtin_bit_cast(unsigned int, lo[j]) != kVmEmpty && __builtin_bit_cast(unsigned int, hi[j]) != kVmEmpty;
                 if (ok) break;
-                if (++spins > spin_limit) {
-                    __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                    break;
-                }
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {

@@ -79,6 +79,8 @@ struct DeviceState {
     float* static_partial = nullptr;
     unsigned int* static_status = nullptr;
     unsigned int* static_status_dev = nullptr;
+    // Polls of one record before a reducing lane of the sliced I_X_W kernel gives up (pimhip_set_gemv_spin_limit).
+    unsigned int vm_spin_limit = 1u << 22;
 };
 
 std::mutex g_mutex;
@@ -169,9 +171,6 @@ int gemv_mv(const half_t* W, const half_t* x, const half_t* bias, half_t* y, int
     return PIMHIP_OK;
 }
 
-// Polls of one record before a reducing lane of the VM kernel gives up (seconds; a record normally arrives within
-// microseconds of its producer's last load).
-constexpr unsigned int kVmSpinLimit = 1u << 22;
 
 // The records of the static scratch array instead of the stream's workspace: nothing is allocated, freed or
 // synchronised (pimhip_execute_gemv_static).
@@ -254,7 +253,7 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     }
     dim3 grid(col_blocks, slices);
     gemv_vm_f16_kernel<WAVES, U, LPR><<<grid, WAVES * 64, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu,
-                                                                    k_per_slice, partial, status, kVmSpinLimit);
+                                                                    k_per_slice, partial, status, st->vm_spin_limit);
     return PIMHIP_OK;
 }
 
@@ -382,6 +381,31 @@ extern "C" int pimhip_execute_gemv_static(void* out, const void* in, const void*
                                           int64_t out_w, int64_t ld_weight, int act, int order, void* stream)
 {
     return execute_gemv(out, in, weight, bias, in_w, out_w, ld_weight, act, order, stream, true);
+}
+
+extern "C" int pimhip_gemv_status(void* stream, int* gave_up)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!gave_up) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "gave_up must be non-null");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    int flags = 0;
+    auto it = st->workspaces.find(static_cast<hipStream_t>(stream));
+    if (it != st->workspaces.end() && it->second.status && *it->second.status != 0u) flags |= 1;
+    if (st->static_status && *st->static_status != 0u) flags |= 2;
+    *gave_up = flags;
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_set_gemv_spin_limit(unsigned int spin_limit)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    st->vm_spin_limit = spin_limit;
+    return PIMHIP_OK;
 }
 
 extern "C" int pimhip_execute_bmm(void* const* outs, int n_outs, const void* x, const void* A, int64_t k, int64_t n,

@@ -84,6 +84,32 @@ def _stream_handle(stream):
     return int(stream)
 
 
+def gemv_status(stream=None):
+    """After the caller has synchronised `stream`: has a sliced I_X_W product given up waiting for partial sums since the
+    workspace was last re-initialised?  Returns (on_this_stream, static_entry_point).  The next sliced product on the
+    stream raises in any case; this is for a caller that wants to know before it uses the result."""
+    flags = ctypes.c_int(0)
+    _check(L.load().pimhip_gemv_status(_stream_handle(stream), ctypes.byref(flags)))
+    return bool(flags.value & 1), bool(flags.value & 2)
+
+
+def synchronize_and_check(stream=None):
+    """Synchronises `stream` (torch's current one by default) and raises if a sliced I_X_W product on it gave up."""
+    s = stream if isinstance(stream, torch.cuda.Stream) else (torch.cuda.current_stream() if stream is None else None)
+    if s is not None:
+        s.synchronize()
+    else:
+        torch.cuda.synchronize()
+    on_stream, static = gemv_status(stream)
+    if on_stream or static:
+        raise NNRuntimeException("a sliced I_X_W product gave up waiting for partial sums: its result is undefined")
+
+
+def set_gemv_spin_limit(spin_limit):
+    """Polls of one record before a reducing block of the sliced I_X_W kernel gives up (default 2**22; 0 gives up at once)."""
+    _check(L.load().pimhip_set_gemv_spin_limit(int(spin_limit)))
+
+
 def _require_half_cuda(*tensors):
     for t in tensors:
         if t is None:

@@ -196,6 +196,39 @@ def test_gemv_vm_order_full_size_properties(ops, n, k):
     assert all(torch.equal(o, ynb) for o in outs)
 
 
+def test_sliced_vm_product_that_gives_up_is_reported_and_the_workspace_recovers(ops):
+    """A reducing block that gives up its wait (forced from the host: with a spin limit of 0 it does not poll at all, and
+    every kernel still ends by itself) sets the stream's status word.  A caller that synchronises can read it; the next
+    sliced product on the stream is refused with a time-out and re-initialises the records; the one after is right."""
+    from pimaicompiler_amd import _lib as L
+    n, k = 4096, 4096
+    g = torch.Generator().manual_seed(77)
+    A = (0.02 * torch.randn(k, n, generator=g)).half().to(DEV)
+    x = (2 * torch.rand(k, generator=g) - 1).half().to(DEV)
+    rc, y0 = raw_gemv(ops, A, x, None, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert ops.gemv_status() == (False, False)
+    ops.set_gemv_spin_limit(0)
+    try:
+        rc, _ = raw_gemv(ops, A, x, None, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+        assert rc == 0  # the launch itself succeeds; its result is undefined
+        torch.cuda.synchronize()
+        assert ops.gemv_status() == (True, False)
+        with pytest.raises(ops.NNRuntimeException, match="gave up"):
+            ops.synchronize_and_check()
+    finally:
+        ops.set_gemv_spin_limit(1 << 22)
+    rc, _ = raw_gemv(ops, A, x, None, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+    assert rc == L.PIMHIP_ERR_TIMEOUT
+    assert b"gave up" in L.load().pimhip_last_error()
+    torch.cuda.synchronize()
+    assert ops.gemv_status() == (False, False)
+    rc, y = raw_gemv(ops, A, x, None, k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W)
+    assert rc == 0 and torch.equal(y, y0)
+    ops.synchronize_and_check()
+
+
 def test_moe_ffn_decode_step_matches_libtorch(ops, golden):
     import importlib.util, os
     spec = importlib.util.spec_from_file_location("make_golden", os.path.join(os.path.dirname(__file__), "golden", "make_golden.py"))
