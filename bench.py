@@ -48,7 +48,8 @@ def main():
                          "a kernel of known traffic that scales rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--sections", default="sweep,lstm,other",
                     help="comma list of what to run: sweep (the timed steps, always run), lstm (LSTM and input projection "
-                         "figures), other (the other kernels of the path); counter runs use --sections sweep")
+                         "figures), other (the other kernels of the path), decoder (the one-launch decoder step alone, "
+                         "issued eagerly; not in the default set); counter runs use one of sweep, lstm, decoder at a time")
     args = ap.parse_args()
     sections = set(args.sections.split(","))
 
@@ -503,6 +504,33 @@ def main():
             other["reference_hip_gemv_kernel"] = ref_times
 
     progress("other kernels timed")
+    # ---- the one-launch decoder step alone, issued eagerly: what a counter run of that kernel uses (no graph is recorded
+    # or replayed here, so the section may run under rocprofv3 --pmc) ------------------------------------------------
+    if "decoder" in sections:
+        kq = 1.0 / 32.0
+        dprm = []
+        for in_w in (1024, 2048, 2048, 2048):
+            dprm += [((2 * torch.rand(sh_, device=dev) - 1) * kq).half() for sh_ in ((4096, in_w), (4096, 1024), (4096,), (4096,))]
+        cls_w = shapes[3]["pool"][0]
+        eplan = P.DecoderPlan(dprm, True, 4, first_takes_context=False, first_residual_layer=2, classifier=(cls_w, None))
+        e_x = torch.randn(1024, device=dev).half()
+        e_h = [torch.zeros(1024, dtype=torch.float16, device=dev) for _ in range(4)]
+        e_c = [torch.zeros(1024, dtype=torch.float16, device=dev) for _ in range(4)]
+        e_hn = [torch.zeros(1024, dtype=torch.float16, device=dev) for _ in range(4)]
+        e_cn = [torch.zeros(1024, dtype=torch.float16, device=dev) for _ in range(4)]
+        e_att = torch.softmax(torch.randn(50, device=dev), 0).half()
+        e_enc = torch.randn(50, 1024, device=dev).half()
+        e_logits = torch.zeros(32000, dtype=torch.float16, device=dev)
+        estep = eplan.bind(e_x, e_h, e_c, att=e_att, enc=e_enc, hn=e_hn, cn=e_cn, logits=e_logits)
+        estep()
+        torch.cuda.synchronize()
+        eplan.status()
+        n_steps = 20 if counter_run else 200
+        other["decoder_step_one_launch_eager_section"] = {
+            "issued_from_python_us": round(timed_us(estep, n_steps, settle_s=0.3), 2),
+            "bytes": (2 * 4096 * 1024 + 3 * 2 * 4096 * 1024) * 2 + 3 * 4096 * 50 * 4 + 32000 * 1024 * 2}
+        eplan.status()
+        progress("decoder step timed")
     # ---- CPU baseline: LibTorch CPU at::addmm in fp16 on the same sweep, bounded sample ---------------------------
     cpu = None
     if not args.no_cpu_baseline:
