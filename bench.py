@@ -251,8 +251,23 @@ def main():
             torch.cuda.synchronize()
             us_ = e0.elapsed_time(e1) * 1e3 / 100
             tf_ = 2 * T_ * I_ * 4096 / us_ / 1e6
+            # the floor beside it: one launch that only reads the (warm) weight, as the product does once per launch;
+            # no kernel that has to read those bytes in a launch of its own can be faster, whatever it computes
+            def ro_(pk_=pk_):
+                lib.pimhip_probe_stream_read(pk_.data_ptr(), pk_.numel() * pk_.element_size(), sh)
+            for _ in range(5):
+                ro_()
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for _ in range(100):
+                ro_()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            ro_us = e0.elapsed_time(e1) * 1e3 / 100
             xp_shapes.append({"T": T_, "I": I_, "four_H": 4096, "us": round(us_, 2), "tflops": round(tf_, 2),
-                              "mfma_utilisation": round(tf_ / MFMA_FP16_PEAK_TFLOPS, 5)})
+                              "mfma_utilisation": round(tf_ / MFMA_FP16_PEAK_TFLOPS, 5),
+                              "read_only_kernel_over_the_weight_us": round(ro_us, 2),
+                              "mfma_utilisation_if_it_took_only_that": round(2 * T_ * I_ * 4096 / ro_us / 1e6 / MFMA_FP16_PEAK_TFLOPS, 5)})
     progress("lstm and input projection timed")
 
     # ---- the other kernels of the path (reported beside the headline figures, not part of `value`) ---------------

@@ -101,6 +101,8 @@ WIRINGS = [
     (8, 8, 4, True, 0, 5, 1),                # the smallest shapes, residual around every layer
     (520, 520, 4, False, 2, 640, 13),
     (256, 64, 3, False, 2, 0, 3),            # no classifier: the last layer's exchange is left out
+    (1024, 1024, 4, False, 2, 1000, 100),    # 65..128 source positions: both halves of a unit's wavefront pair hold one
+    (512, 512, 2, True, 1, 0, 300),          # more than 128 source positions: the tail loop; the plan's buffer grows past 64
 ]
 
 
@@ -114,6 +116,21 @@ def test_fused_decoder_step_matches_libtorch_cpu(ops, H, in0, L, first_ctx, firs
     # the context handed in instead of att and enc: the same bits everywhere downstream of it
     got = run_fused(ops, case, plan, case.x, case.h, case.c, n_ctx_outs=1, use_ctx_in=want[0].to(DEV))
     check(case, got, want, ctx_given=True)
+
+
+def test_one_plan_serves_sentences_of_different_lengths(ops):
+    """set_encoder once per sentence: a long sentence after a short one makes the projection buffer grow, a short one after
+    it reuses the larger buffer with another row pitch; every step is checked against the CPU."""
+    H, L = 512, 3
+    base = Case(4242, H, H, L, False, 2, 777, 5)
+    plan = base.plan(ops)
+    for i, S in enumerate((5, 150, 64, 9, 129)):
+        g = torch.Generator().manual_seed(900 + S)
+        base.enc = torch.randn(S, H, generator=g).half()
+        base.att = torch.softmax(torch.randn(S, generator=g), -1).half()
+        print(f"sentence {i}: S={S}", flush=True)
+        want = base.cpu_step(base.x, base.h, base.c)
+        check(base, run_fused(ops, base, plan, base.x, base.h, base.c, n_ctx_outs=2), want)
 
 
 def test_fused_decoder_steps_update_the_state_in_place(ops):
