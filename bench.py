@@ -497,7 +497,6 @@ def main():
         fplan.status()
 
         def reproject():
-            fplan._enc_key = None
             fplan.set_encoder(enc2d)
         other["decoder_step_one_launch"] = {
             "issued_from_python_us": round(fused_eager_us, 2), "hip_graph_replay_us": round(fused_graph_us, 2),

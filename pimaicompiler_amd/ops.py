@@ -626,20 +626,17 @@ class DecoderPlan:
         self._handle = handle
         self._finalizer = weakref.finalize(self, DecoderPlan._destroy, handle.value)
         self._enc = None
-        self._enc_key = None
 
     def set_encoder(self, enc, stream=None):
         """Once per sentence: enc [S, H], the encoder outputs the attention weights of the following steps refer to.
         Multiplies the context columns of every layer's W_ih with enc (pimhip_decoder_plan_set_encoder); the plan keeps
-        enc alive.  A call with the tensor (and version) it already has does nothing."""
+        enc alive.  Every call projects again (three launches): a buffer that is refilled for the next sentence has the
+        same address, and kernels that write it through raw pointers leave no trace a cache could key on."""
         _require_half_cuda(enc)
         if enc.dim() != 2 or enc.size(1) != self.hidden or not enc.is_contiguous():
             raise NNRuntimeException(f"enc must be a contiguous [S, {self.hidden}] tensor")
-        key = (enc.data_ptr(), enc._version, enc.size(0))
-        if key == self._enc_key:
-            return
         _check(L.load().pimhip_decoder_plan_set_encoder(self._handle, enc.data_ptr(), enc.size(0), _stream_handle(stream)))
-        self._enc, self._enc_key = enc, key
+        self._enc = enc
 
     @staticmethod
     def _destroy(handle_value):
@@ -660,8 +657,8 @@ class DecoderPlan:
         """Fixes the buffers of a step (lists of [H] tensors per layer; hn / cn default to h_prev / c_prev, i.e. the state is
         updated in place) and returns a callable step(stream=None) that launches it without touching Python tensors
         again: what a decoder loop or a graph capture calls per step.  The context comes from `att` [S], the attention
-        weights over the encoder outputs (`enc`, handed to set_encoder here unless it is the tensor the plan already has),
-        or from `ctx` [H], a context computed elsewhere."""
+        weights over the encoder outputs (`enc`, handed to set_encoder here; leave it out when set_encoder has been called
+        for this sentence), or from `ctx` [H], a context computed elsewhere."""
         lib = L.load()
         n, H = self.num_layers, self.hidden
         hn = list(h_prev) if hn is None else list(hn)

@@ -20,6 +20,12 @@ one join and hang off one common start are collected into a single `multi_stream
 here where the reference gives each sibling its own stream.  `execute` runs a graph through the operator layer
 (pimaicompiler_amd.ops) on the GPU.
 
+`fuse_decoder_step` has no counterpart in the reference: it collects the per-token chain of the GNMT decoder — the
+seq_len-1 `aten::lstm` cells that read cat(previous output, context), the residual `aten::add`s, the attention `aten::bmm`
+and the classifier — which the reference's interpreter runs operator by operator (executeAtenLSTM1 / executeAtenBmm /
+executeAtenAdd / executeAtenAddmm, runtime/source/executor/op_executor/aten_ops_executor.cpp:2135-2307, 668-747, 43-179,
+181-216), into one `pimhip::decoder_step` op, which `execute` runs as ONE launch (ops.DecoderPlan).
+
 remove_cat_for_addmm is restated for any split point; the reference hard-codes the RNNT joint shapes
 ([1,1024] + [1,320] against a [512,1344] weight, compiler/include/frontend/optimizer/remove_cat_for_addmm.h:77-79).
 """
@@ -248,6 +254,173 @@ def multi_stream_execution(g: Graph, max_search_level: int = 10):
     return g
 
 
+# ---- the decoder's per-token chain into one op -----------------------------------------------------------------------
+_DECODER_MAX_LAYERS = 4
+_DECODER_MAX_HIDDEN = 1024
+
+
+def _lstm_input_form(g: Graph, op: Op):
+    """(in, ctx, [cat op, list op]) when the cell's input is cat([in, ctx]) along the last dim, else (input, None, [])."""
+    cat = g.producer(op.inputs[0])
+    if cat is not None and cat.type == "aten::cat" and cat.attrs.get("dim", -1) in (-1, 2):
+        lst = g.producer(cat.inputs[0])
+        if (lst is not None and lst.type == "prim::ListConstruct" and len(lst.inputs) == 2 and
+                len(g.consumers(cat.outputs[0])) == 1 and len(g.consumers(lst.outputs[0])) == 1 and
+                cat.outputs[0] not in g.outputs and lst.outputs[0] not in g.outputs):
+            return lst.inputs[0], lst.inputs[1], [cat, lst]
+    return op.inputs[0], None, []
+
+
+def _lstm_output_form(g: Graph, op: Op, in_tid):
+    """(out, residual add or None): out = y + in when y feeds exactly one add with the cell's own input, else y."""
+    y = op.outputs[0]
+    users = g.consumers(y)
+    if len(users) == 1 and users[0].type == "aten::add" and y not in g.outputs and sorted(users[0].inputs) == sorted([y, in_tid]) \
+            and y != in_tid and users[0].attrs.get("alpha", 1) == 1:
+        return users[0].outputs[0], users[0]
+    return y, None
+
+
+def _depends_on(g: Graph, tid, ops_):
+    """True if tensor `tid` is computed from an output of one of `ops_`."""
+    seen, todo = set(), [tid]
+    while todo:
+        t = todo.pop()
+        if t in seen:
+            continue
+        seen.add(t)
+        p = g.producer(t)
+        if p is None:
+            continue
+        if any(p is o for o in ops_):
+            return True
+        todo.extend(p.inputs)
+    return False
+
+
+def _single_step_cell(g: Graph, op: Op):
+    """An aten::lstm op this pass may take: one layer, one direction, constant fp16 weights with biases, H within the
+    fused kernel's range."""
+    if op.type != "aten::lstm" or len(op.inputs) != 7 or len(op.outputs) != 3:
+        return False
+    if op.attrs.get("num_layers", 1) != 1 or op.attrs.get("bidirectional", False) or not op.attrs.get("has_biases", True):
+        return False
+    if op.attrs.get("seq_len", 1) != 1:
+        return False
+    if not all(g.is_constant(t) and g.constants[t] is not None for t in op.inputs[3:7]):
+        return False
+    w_ih, w_hh = g.constants[op.inputs[3]], g.constants[op.inputs[4]]
+    H = w_hh.size(1)
+    return (w_ih.dtype == torch.float16 and w_hh.dim() == 2 and w_ih.dim() == 2 and tuple(w_hh.shape) == (4 * H, H) and
+            w_ih.size(0) == 4 * H and H % 8 == 0 and 8 <= H <= _DECODER_MAX_HIDDEN and w_ih.size(1) % 8 == 0)
+
+
+def fuse_decoder_step(g: Graph):
+    """Chains of seq_len-1 cells  lstm_0(x | cat(x, ctx)) -> [add] -> cat(., ctx) -> lstm_1 -> [add] -> ...  (the same ctx in
+    every cat, residual adds from some layer on), optionally with the attention bmm that produces ctx and the linear
+    classifier on the last output, become one `pimhip::decoder_step` op at the position of the chain's first op.
+
+    Left alone: cells whose weights are not constants, a pre-residual y with another consumer (the fused step only
+    stores out_k, hn_k, cn_k), a context that is computed from the chain itself (in GNMT the attention query is layer
+    0's output: the chain then starts at layer 1), chains of fewer than two cells."""
+    taken = []
+    for first in list(g.ops):
+        if all(first is not o for o in g.ops) or any(first is o for o in taken) or not _single_step_cell(g, first):
+            continue
+        # ---- follow the chain upwards from `first`
+        forms, ctx, cur = [], None, first
+        while cur is not None and len(forms) < _DECODER_MAX_LAYERS and _single_step_cell(g, cur) and all(cur is not o for o in taken):
+            in_tid, c_tid, glue = _lstm_input_form(g, cur)
+            H = g.constants[cur.inputs[4]].size(1)
+            own_w = g.constants[cur.inputs[3]].size(1) - (H if c_tid is not None else 0)   # width of the cell's own input
+            if own_w < 8:
+                break
+            if forms:
+                # a later cell reads cat(previous output, the chain's context)
+                if in_tid != forms[-1]["out"] or c_tid is None or (ctx is not None and c_tid != ctx) or H != forms[0]["H"] or own_w != H:
+                    break
+            elif c_tid is not None and own_w != H:
+                break                          # a first cell on cat(x, ctx) needs x as wide as the hidden state
+            if c_tid is not None:
+                ctx = c_tid
+            out, add = _lstm_output_form(g, cur, in_tid)
+            if add is not None and own_w != H:
+                out, add = cur.outputs[0], None  # y + x with x of another width is not this wiring's residual
+            forms.append(dict(cell=cur, in_tid=in_tid, takes_ctx=c_tid is not None, glue=glue, out=out, add=add, H=H))
+            cur = None
+            for u in g.consumers(out):
+                if u.type != "prim::ListConstruct" or len(u.inputs) != 2 or u.inputs[0] != out:
+                    continue
+                cats = g.consumers(u.outputs[0])
+                cells_ = g.consumers(cats[0].outputs[0]) if len(cats) == 1 and cats[0].type == "aten::cat" else []
+                if len(cells_) == 1 and cells_[0].type == "aten::lstm" and cells_[0].inputs[0] == cats[0].outputs[0]:
+                    cur = cells_[0]
+                    break
+        # ---- residual adds must be contiguous from some layer on; cut the chain where they stop being so
+        n = len(forms)
+        for k in range(n):
+            if forms[k]["add"] is None and any(forms[q]["add"] is not None for q in range(k)):
+                n = k
+                break
+        forms = forms[:n]
+        # ---- the context must not be computed from the chain
+        if ctx is not None and forms and _depends_on(g, ctx, [f["cell"] for f in forms]):
+            continue                          # (the chain that starts one cell later is found when the loop reaches that cell)
+        if len(forms) < 2:
+            continue
+        first_res = next((k for k in range(len(forms)) if forms[k]["add"] is not None), len(forms))
+        members = []
+        for f in forms:
+            members += f["glue"] + [f["cell"]] + ([f["add"]] if f["add"] is not None else [])
+        # ---- the attention bmm, when the chain is the context's only consumer
+        att = enc = None
+        bmm = g.producer(ctx) if ctx is not None else None
+        if (bmm is not None and bmm.type == "aten::bmm" and ctx not in g.outputs and
+                all(any(u is m for m in members) for u in g.consumers(ctx))):
+            att, enc = bmm.inputs
+            members.append(bmm)
+        # ---- the classifier on the last output
+        last_out = forms[-1]["out"]
+        cls = next((u for u in g.consumers(last_out)
+                    if u.type in ("aten::linear", "pimhip::gemv") and u.inputs[0] == last_out and g.is_constant(u.inputs[1]) and
+                    g.constants[u.inputs[1]].dim() == 2 and g.constants[u.inputs[1]].size(1) == forms[0]["H"] and
+                    u.attrs.get("act_type", "none") == "none"), None)
+        if cls is not None:
+            members.append(cls)
+        # ---- the fused op goes where the chain starts, or right after the last producer of something it reads if that is
+        # later; no operator before that place may read what the chain computes
+        external = [forms[0]["in_tid"]] + [t for f in forms for t in f["cell"].inputs[1:3]]
+        external += [att, enc] if att is not None else ([ctx] if ctx is not None else [])
+        pos = min(g.ops.index(m) for m in members)
+        for t in external:
+            prod = g.producer(t)
+            if prod is not None:
+                pos = max(pos, g.ops.index(prod) + 1)
+        produced = {t for m in members for t in m.outputs}
+        if any(all(o is not m for m in members) and produced.intersection(o.inputs) for o in g.ops[:pos]):
+            continue
+        pos -= sum(1 for m in members if g.ops.index(m) < pos)     # index after the members have been taken out
+        cls_bias = None
+        if cls is not None and len(cls.inputs) > 2 and (cls.type == "aten::linear" or cls.attrs.get("has_bias")):
+            cls_bias = cls.inputs[2]
+        L = len(forms)
+        fused = Op("pimhip::decoder_step",
+                   [forms[0]["in_tid"]] + ([att, enc] if att is not None else ([ctx] if ctx is not None else [])) +
+                   [f["cell"].inputs[1] for f in forms] + [f["cell"].inputs[2] for f in forms],
+                   [f["out"] for f in forms] + [f["cell"].outputs[1] for f in forms] + [f["cell"].outputs[2] for f in forms] +
+                   ([cls.outputs[0]] if cls is not None else []),
+                   {"num_layers": L, "hidden": forms[0]["H"], "first_takes_context": forms[0]["takes_ctx"],
+                    "first_residual_layer": first_res, "context": "bmm" if att is not None else ("given" if ctx is not None else "none"),
+                    "params": [t for f in forms for t in f["cell"].inputs[3:7]],
+                    "classifier": (cls.inputs[1], cls_bias) if cls is not None else None,
+                    "out_shapes": "as the operators' ([1, 1, H] per layer, classifier as its operator would)"})
+        for m in members:
+            g.ops.remove(m)
+        g.ops.insert(pos, fused)
+        taken.append(fused)
+    return g
+
+
 def _as_row_major_weight(t):
     """For a [..1.., in, out] tensor that is a transposed view of a dense row-major [out, in] matrix: that matrix."""
     if t.dim() < 2 or any(d != 1 for d in t.shape[:-2]) or t.dtype != torch.float16:
@@ -259,8 +432,53 @@ def _as_row_major_weight(t):
 
 
 # ---- execution through the operator layer ----------------------------------------------------------------------------
-def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0"):
-    """Runs the op list with pimaicompiler_amd.ops; returns the graph outputs.  Constants are moved to `device`."""
+def _run_decoder_step(op: Op, env, ops, same_sentence):
+    """One pimhip::decoder_step op: the plan is made on first use and kept on the op; outputs are new tensors shaped as the
+    operators it replaces would shape them."""
+    at = op.attrs
+    L, H = at["num_layers"], at["hidden"]
+    plan = at.get("_plan")
+    if plan is None:
+        cls = None
+        if at["classifier"] is not None:
+            w_t, b_t = at["classifier"]
+            cls = (env[w_t], env[b_t] if b_t is not None else None)
+        plan = ops.DecoderPlan([env[t] for t in at["params"]], True, L, first_takes_context=at["first_takes_context"],
+                               first_residual_layer=at["first_residual_layer"], classifier=cls)
+        at["_plan"] = plan
+    x = env[op.inputs[0]]
+    att = enc = ctx = None
+    i = 1
+    if at["context"] == "bmm":
+        att, enc = env[op.inputs[1]], env[op.inputs[2]]
+        i = 3
+        if not (same_sentence and plan._enc is not None):
+            plan.set_encoder(enc.reshape(-1, H).contiguous())
+    elif at["context"] == "given":
+        ctx = env[op.inputs[1]]
+        i = 2
+    flat = lambda t: t.contiguous().view(-1)  # noqa: E731
+    h_prev = [flat(env[t]) for t in op.inputs[i:i + L]]
+    c_prev = [flat(env[t]) for t in op.inputs[i + L:i + 2 * L]]
+    new = lambda: torch.empty(1, 1, H, dtype=torch.float16, device=x.device)  # noqa: E731
+    outs, hn, cn = [new() for _ in range(L)], [new() for _ in range(L)], [new() for _ in range(L)]
+    logits = None
+    if plan.vocab:
+        logits = torch.empty(list(outs[-1].shape[:-1]) + [plan.vocab], dtype=torch.float16, device=x.device)
+    step = plan.bind(flat(x), h_prev, c_prev, att=flat(att) if att is not None else None, ctx=flat(ctx) if ctx is not None else None,
+                     hn=[t.view(-1) for t in hn], cn=[t.view(-1) for t in cn], outs=[t.view(-1) for t in outs],
+                     logits=logits.view(-1) if logits is not None else None)
+    step()
+    for k in range(L):
+        env[op.outputs[k]], env[op.outputs[L + k]], env[op.outputs[2 * L + k]] = outs[k], hn[k], cn[k]
+    if logits is not None:
+        env[op.outputs[3 * L]] = logits
+
+
+def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0", same_sentence=False):
+    """Runs the op list with pimaicompiler_amd.ops; returns the graph outputs.  Constants are moved to `device`.
+    `same_sentence`: the encoder outputs a fused decoder step attends over are the ones of the previous call (their
+    projection is then not computed again)."""
     from . import ops
 
     env = {k: (v.to(device) if v is not None else None) for k, v in g.constants.items()}
@@ -302,6 +520,15 @@ def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0"):
                     env[m.outputs[0]] = (ops.custom_aten_addmm(m.attrs.get("act_type", "none"), am[0], am[1], am[2])
                                          if m.type == "aten::addmm" else ops.custom_aten_matmul(am[0], am[1]))
             continue
+        elif op.type == "pimhip::decoder_step":
+            _run_decoder_step(op, env, ops, same_sentence)
+            continue
+        elif op.type == "aten::lstm":
+            y, hn, cn = ops.aten_lstm1(a[0], (a[1], a[2]), a[3:7], True, 1, 0.0, False, False, False)
+            env[op.outputs[0]], env[op.outputs[1]], env[op.outputs[2]] = y, hn, cn
+            continue
+        elif op.type == "aten::bmm":
+            r = ops.aten_bmm(a[0], a[1])
         elif op.type == "aten::contiguous":
             r = a[0].contiguous()
         elif op.type == "aten::slice":

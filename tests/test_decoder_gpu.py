@@ -133,6 +133,34 @@ def test_one_plan_serves_sentences_of_different_lengths(ops):
         check(base, run_fused(ops, base, plan, base.x, base.h, base.c, n_ctx_outs=2), want)
 
 
+def test_encoder_buffer_refilled_in_place_is_projected_again(ops):
+    """The next sentence lands in the same buffer, written by one of the path's own kernels through its raw pointer (no
+    tensor version changes): set_encoder must project again, not recognise the buffer."""
+    H, L, S = 256, 2, 11
+    case = Case(5151, H, H, L, True, 0, 0, S)
+    plan = case.plan(ops)
+    enc_buf = torch.zeros(S, H, dtype=torch.float16, device=DEV)
+    zeros = torch.zeros(S, H, dtype=torch.float16, device=DEV)
+    att = case.att.to(DEV)
+    hn = [torch.zeros(H, dtype=torch.float16, device=DEV) for _ in range(L)]
+    cn = [torch.zeros(H, dtype=torch.float16, device=DEV) for _ in range(L)]
+    step = None
+    for i in range(3):
+        g = torch.Generator().manual_seed(7000 + i)
+        case.enc = torch.randn(S, H, generator=g).half()
+        version = enc_buf._version
+        ops.aten_add(case.enc.to(DEV), zeros, out=enc_buf)
+        assert enc_buf._version == version
+        plan.set_encoder(enc_buf)
+        if step is None:
+            step = plan.bind(case.x.to(DEV), [t.to(DEV) for t in case.h], [t.to(DEV) for t in case.c], att=att, hn=hn, cn=cn)
+        step()
+        plan.status()
+        _, _, whn, wcn, _ = case.cpu_step(case.x, case.h, case.c)
+        for k in range(L):
+            assert maxabs(hn[k], whn[k]) <= STATE_TOL and maxabs(cn[k], wcn[k]) <= STATE_TOL, (i, k)
+
+
 def test_fused_decoder_steps_update_the_state_in_place(ops):
     """A decoder loop: hn / cn are the buffers h_prev / c_prev are read from, three steps in a row, against the CPU
     running the same three steps; then the same three steps again into separate buffers give the same bits."""

@@ -198,3 +198,134 @@ def test_multi_stream_graph_matches_the_original_op_list(ops):
         w = x[i:i + 1].float() @ g.constants[100 + i].float().t() + g.constants[200 + i].float()
         assert list(o.shape) == [1, 512] and float((o.float().cpu() - w).abs().max()) <= 4e-3
         assert float((o.float() - r.float()).abs().max()) <= 2e-3
+
+
+# ---- the decoder's per-token chain into one op ----------------------------------------------------------------------
+def decoder_graph(seed=11, H=256, S=9, vocab=500, query_from_layer0=False, in0=None):
+    """One token of a GNMT-style decoder as the interpreter sees it: four seq_len-1 cells, layers 1..3 on cat(previous
+    output, context), residual adds around layers 2 and 3, the attention bmm, the classifier.  With `query_from_layer0`
+    the attention weights are computed from layer 0's output (as in GNMT), otherwise they are a graph input."""
+    from pimaicompiler_amd import workloads
+    g = torch.Generator().manual_seed(seed)
+    in0 = H if in0 is None else in0
+    c, ops = {}, []
+    X, ATT, ENC, KEYS = 0, 1, 2, 3
+    for k in range(4):
+        prm = workloads.lstm_inputs(seed + 10 + k, in0 if k == 0 else 2 * H, H, 1, False, 1)[0]
+        for j, t in enumerate(prm):
+            c[100 + 4 * k + j] = t
+    c[200], c[201] = (0.05 * torch.randn(vocab, H, generator=g)).half(), (0.01 * torch.randn(vocab, generator=g)).half()
+    y, hn, cn, lst, cat, res = (lambda k: 300 + k), (lambda k: 310 + k), (lambda k: 320 + k), (lambda k: 330 + k), (lambda k: 340 + k), (lambda k: 350 + k)
+    CTX = 40
+    ops.append(R.Op("aten::lstm", [X, 10, 20, 100, 101, 102, 103], [y(0), hn(0), cn(0)]))
+    if query_from_layer0:
+        ops.append(R.Op("aten::bmm", [y(0), KEYS], [41]))          # scores [1, 1, S] from layer 0's output
+        ops.append(R.Op("aten::bmm", [41, ENC], [CTX]))
+    else:
+        ops.append(R.Op("aten::bmm", [ATT, ENC], [CTX]))
+    prev = y(0)
+    for k in range(1, 4):
+        ops += [R.Op("prim::ListConstruct", [prev, CTX], [lst(k)]), R.Op("aten::cat", [lst(k)], [cat(k)], {"dim": 2}),
+                R.Op("aten::lstm", [cat(k), 10 + k, 20 + k] + [100 + 4 * k + j for j in range(4)], [y(k), hn(k), cn(k)])]
+        if k >= 2:
+            ops.append(R.Op("aten::add", [y(k), prev], [res(k)]))
+            prev = res(k)
+        else:
+            prev = y(k)
+    ops.append(R.Op("aten::linear", [prev, 200, 201], [400]))
+    inputs = [X, ENC] + ([KEYS] if query_from_layer0 else [ATT]) + [10 + k for k in range(4)] + [20 + k for k in range(4)]
+    outputs = [400] + [hn(k) for k in range(4)] + [cn(k) for k in range(4)]
+    feeds = {X: torch.randn(1, 1, in0, generator=g).half(), ENC: torch.randn(1, S, H, generator=g).half()}
+    if query_from_layer0:
+        feeds[KEYS] = (0.05 * torch.randn(1, H, S, generator=g)).half()
+    else:
+        feeds[ATT] = torch.softmax(torch.randn(1, 1, S, generator=g), -1).half()
+    for k in range(4):
+        feeds[10 + k] = (0.3 * torch.randn(1, 1, H, generator=g)).half()
+        feeds[20 + k] = (0.3 * torch.randn(1, 1, H, generator=g)).half()
+    return R.Graph(ops, inputs, outputs, c, next_id=500), feeds
+
+
+def test_decoder_chain_becomes_one_op():
+    g, _ = decoder_graph()
+    R.fuse_decoder_step(g)
+    assert g.types() == ["pimhip::decoder_step"]
+    op = g.ops[0]
+    assert op.attrs["num_layers"] == 4 and op.attrs["first_takes_context"] is False and op.attrs["first_residual_layer"] == 2
+    assert op.attrs["context"] == "bmm" and op.attrs["classifier"] == (200, 201)
+    assert op.inputs == [0, 1, 2, 10, 11, 12, 13, 20, 21, 22, 23]
+    assert op.outputs == [300, 301, 352, 353, 310, 311, 312, 313, 320, 321, 322, 323, 400]
+    assert op.attrs["params"] == list(range(100, 116))
+
+
+def test_decoder_chain_starts_after_the_cell_the_attention_reads():
+    """In GNMT the attention weights come from layer 0's output: layer 0 and the scores stay operators, the rest of the
+    token (context bmm, three cells, two adds, classifier) is one op whose first cell takes cat(y0, ctx)."""
+    g, _ = decoder_graph(query_from_layer0=True)
+    R.fuse_decoder_step(g)
+    assert g.types() == ["aten::lstm", "aten::bmm", "pimhip::decoder_step"]
+    op = g.ops[2]
+    assert op.attrs["num_layers"] == 3 and op.attrs["first_takes_context"] is True and op.attrs["first_residual_layer"] == 1
+    assert op.attrs["context"] == "bmm" and op.inputs[:3] == [300, 41, 2]
+
+
+def test_decoder_chain_guards():
+    # a pre-residual y with a second consumer cannot be dropped: the chain ends before that cell's add
+    g, _ = decoder_graph()
+    g.ops.append(R.Op("aten::relu", [302], [450]))
+    g.outputs.append(450)
+    R.fuse_decoder_step(g)
+    fused = [o for o in g.ops if o.type == "pimhip::decoder_step"]
+    assert len(fused) == 1 and fused[0].attrs["num_layers"] == 3 and fused[0].attrs["classifier"] is None
+    assert fused[0].attrs["first_residual_layer"] == 3                    # layers 0..2, none of them with a residual add
+    assert [o.type for o in g.ops].count("aten::lstm") == 1 and "aten::linear" in g.types()
+    # the context is used elsewhere too: it stays an operator and is handed to the fused op
+    g, _ = decoder_graph()
+    g.outputs.append(40)
+    R.fuse_decoder_step(g)
+    assert g.types() == ["aten::bmm", "pimhip::decoder_step"] and g.ops[1].attrs["context"] == "given" and g.ops[1].inputs[:2] == [0, 40]
+    # weights that are not constants: nothing to fuse
+    g, _ = decoder_graph()
+    w = g.constants.pop(104)
+    g.inputs.append(104)
+    R.fuse_decoder_step(g)
+    fused = [o for o in g.ops if o.type == "pimhip::decoder_step"]
+    assert len(fused) == 1 and fused[0].attrs["num_layers"] == 2 and fused[0].inputs[0] == 301   # only layers 2 and 3
+    assert w is not None
+    # a single cell is left alone
+    g, _ = decoder_graph()
+    g.ops = g.ops[:1]
+    g.outputs = [300]
+    R.fuse_decoder_step(g)
+    assert g.types() == ["aten::lstm"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("query_from_layer0", [False, True])
+def test_fused_decoder_graph_matches_the_operator_list_and_libtorch(ops, query_from_layer0):
+    H, S = 256, 9
+    g0, feeds = decoder_graph(H=H, S=S, query_from_layer0=query_from_layer0)
+    want_ops = [t.float().cpu() for t in R.execute(g0, feeds, DEV)]
+    g1, _ = decoder_graph(H=H, S=S, query_from_layer0=query_from_layer0)
+    R.fuse_decoder_step(g1)
+    assert "pimhip::decoder_step" in g1.types()
+    for rep in range(2):                      # the second call reuses the op's plan (and, told so, the sentence's projection)
+        got = [t.float().cpu() for t in R.execute(g1, feeds, DEV, same_sentence=rep > 0)]
+        assert [list(t.shape) for t in got] == [list(t.shape) for t in want_ops]
+        for a, b in zip(got, want_ops):
+            assert float((a - b).abs().max()) <= 5e-3
+    # LibTorch CPU on the same op list
+    c = g0.constants
+    f = {k: v for k, v in feeds.items()}
+    cell = lambda k, inp: torch.lstm(inp, (f[10 + k], f[20 + k]), [c[100 + 4 * k + j] for j in range(4)], True, 1, 0.0, False, False, False)  # noqa: E731
+    y0, hn0, cn0 = cell(0, f[0])
+    att = torch.bmm(y0.float(), f[3].float()).half() if query_from_layer0 else f[1]
+    ctx = torch.bmm(att.float(), f[2].float()).half()
+    y1, hn1, cn1 = cell(1, torch.cat([y0, ctx], 2))
+    y2, hn2, cn2 = cell(2, torch.cat([y1, ctx], 2))
+    r2 = y2 + y1
+    y3, hn3, cn3 = cell(3, torch.cat([r2, ctx], 2))
+    r3 = y3 + r2
+    logits = torch.nn.functional.linear(r3.float(), c[200].float(), c[201].float())
+    for a, b in zip(got, [logits, hn0, hn1, hn2, hn3, cn0, cn1, cn2, cn3]):
+        assert float((a - b.float()).abs().max()) <= 5e-3
