@@ -189,8 +189,11 @@ int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limi
 
 /* Selects how pimhip_lstm_forward runs the recurrence: 0 = automatic, 1 = one fused launch per step,
  * 2 = persistent sequence kernel (hidden_size up to 2048; fails with PIMHIP_ERR_UNSUPPORTED otherwise), 3 = as 2 but with
- * four hidden units per block in every launch (2 runs a single unidirectional layer with eight).  A call with
- * seq_len 1 runs the fused step launch in every mode. */
+ * four hidden units per block in every launch (2 runs a single unidirectional layer with eight), 4 = every recurrence
+ * (layer and direction) on one XCD of the part, the two directions of a layer side by side on two (hidden_size up to
+ * 1024 on a device of 8 XCDs x 32 CUs; PIMHIP_ERR_UNSUPPORTED otherwise).  Automatic takes 4 for bidirectional layers
+ * and for a single unidirectional layer when the sequence is long enough to pay for it, 2 for unidirectional stacks
+ * (a wavefront over the layers), 1 where neither fits.  A call with seq_len 1 runs the fused step launch in every mode. */
 int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);
 
 /* The dense input projection of one LSTM layer over all time steps, the only MFMA kernel of the path:
@@ -227,6 +230,11 @@ int pimhip_set_gemv_spin_limit(unsigned int spin_limit);
  * of the GEMV kernels and keeps nothing: what one launch of it takes is the floor for any kernel that has to read
  * those bytes, launch included.  The benchmark reports each GEMV beside it. */
 int pimhip_probe_stream_read(const void* data, int64_t bytes, void* stream);
+
+/* No counterpart in the reference.  Launches `blocks` workgroups of `threads` lanes; workgroup b stores the index of
+ * the XCD it runs on (the hardware's XCC_ID) to out[b] (uint32).  What the per-XCD LSTM kernel (mode 4) relies on can be
+ * looked at with it: consecutive workgroups go to consecutive XCDs. */
+int pimhip_probe_xcc_map(void* out, int blocks, int threads, void* stream);
 
 /* ---- decoder step ---------------------------------------------------------------------------- */
 

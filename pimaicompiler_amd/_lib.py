@@ -27,6 +27,7 @@ SIGNATURES = {
                                                   ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_void_p]),
     "pimhip_probe_stream_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
+    "pimhip_probe_xcc_map": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "pimhip_gemv_status": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
     "pimhip_set_gemv_spin_limit": (ctypes.c_int, [ctypes.c_uint]),
     "pimhip_execute_dot": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,

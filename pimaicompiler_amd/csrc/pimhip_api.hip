@@ -16,6 +16,7 @@
 #include "decoder_kernels.h"
 #include "gemv_kernels.h"
 #include "lstm_kernels.h"
+#include "lstm_xcd_kernels.h"
 #include "shape_logic.h"
 #include "xproj_kernels.h"
 
@@ -459,6 +460,26 @@ extern "C" int pimhip_execute_add(void* c, const void* a, const void* b, int64_t
     return PIMHIP_OK;
 }
 
+namespace
+{
+__global__ void xcc_map_kernel(unsigned int* out)
+{
+    // HW_REG_XCC_ID (hardware register 20), bits 3:0
+    if (threadIdx.x == 0) out[blockIdx.x] = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u;
+}
+}  // namespace
+
+extern "C" int pimhip_probe_xcc_map(void* out, int blocks, int threads, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!out || blocks < 1 || threads < 1 || threads > 1024) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "out must be non-null, blocks >= 1, threads in [1, 1024]");
+    xcc_map_kernel<<<(unsigned)blocks, (unsigned)threads, 0, static_cast<hipStream_t>(stream)>>>(static_cast<unsigned int*>(out));
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
 extern "C" int pimhip_probe_stream_read(const void* data, int64_t bytes, void* stream)
 {
     DeviceState* st = nullptr;
@@ -722,6 +743,11 @@ struct PimHipLstmPlan {
     bool reset_exchange = false;     // the next forward starts from a cleared exchange buffer (layout change)
     bool seq_units8_ok = false;      // a single chain may run with 8 hidden units per block (half as many blocks)
     bool seq_wide = false;           // 1024 < H <= 2048: 32 columns per lane, eight units per block, one layer per launch
+    // Mode 4: every recurrence on one XCD (lstm_xcd_f16_kernel).
+    bool xcd_ok = false;             // H fits one XCD's registers and the device has the eight XCDs of 32 CUs the kernel assumes
+    unsigned int* xcd_hx = nullptr;  // [kXcdMaxChains] regions of kXcdRegionWords, zero when the chain's counter is 2
+    unsigned int* xcd_g_counters = nullptr;  // [kXcdMaxChains]
+    unsigned int* xcd_claims = nullptr;      // [kXcdCount][kXcdMembers], zero when the counters are 2
 };
 
 namespace
@@ -741,6 +767,9 @@ int destroy_plan_locked(PimHipLstmPlan* plan)
     if (plan->c_state) hipFree(plan->c_state);
     if (plan->hx) hipFree(plan->hx);
     if (plan->g_counters) hipFree(plan->g_counters);
+    if (plan->xcd_hx) hipFree(plan->xcd_hx);
+    if (plan->xcd_g_counters) hipFree(plan->xcd_g_counters);
+    if (plan->xcd_claims) hipFree(plan->xcd_claims);
     if (plan->abort_flag) hipFree(plan->abort_flag);
     if (plan->abort_host) hipHostFree(plan->abort_host);
     if (prev >= 0) hipSetDevice(prev);
@@ -873,8 +902,10 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
     PLAN_HIP_CHECK(hipMalloc(&plan->c_state, sizeof(float) * (size_t)D * H));
     PLAN_HIP_CHECK(hipMalloc(&plan->abort_flag, sizeof(unsigned int)));
     PLAN_HIP_CHECK(hipMemsetAsync(plan->abort_flag, 0, sizeof(unsigned int), s));
-    PLAN_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&plan->abort_host), sizeof(unsigned int), hipHostMallocMapped));
-    *plan->abort_host = 0;
+    // word 0: 1 = a wait gave up, 2 = a workgroup of the per-XCD kernel found its rank on its XCD taken (words 1 and 2
+    // then hold that workgroup's index and the XCD it ran on)
+    PLAN_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&plan->abort_host), 4 * sizeof(unsigned int), hipHostMallocMapped));
+    plan->abort_host[0] = plan->abort_host[1] = plan->abort_host[2] = plan->abort_host[3] = 0;
     PLAN_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&plan->abort_host_dev), plan->abort_host, 0));
 
     // Persistent sequence kernel: one block per 4 hidden units (one unit per wavefront, weights in registers),
@@ -906,6 +937,22 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         fill_u32_kernel<<<1, 64, 0, s>>>(plan->g_counters, kSeqMaxChains + 1, 2u);
         PLAN_HIP_CHECK(hipGetLastError());
     }
+    // One recurrence per XCD: the part this is written for has 8 XCDs of 32 CUs, a group is one workgroup per CU of one.
+    if (H <= kXcdMaxH && plan->num_cus == kXcdCount * kXcdMembers) {
+        int per_cu = 0;
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_xcd_f16_kernel, kXcdThreads, 0));
+        plan->xcd_ok = per_cu >= 1;
+    }
+    if (plan->xcd_ok) {
+        const size_t words = (size_t)kXcdRegionWords * kXcdMaxChains;
+        PLAN_HIP_CHECK(hipMalloc(&plan->xcd_hx, words * sizeof(unsigned int)));
+        fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->xcd_hx, words, 0u);
+        PLAN_HIP_CHECK(hipMalloc(&plan->xcd_g_counters, kXcdMaxChains * sizeof(unsigned int)));
+        fill_u32_kernel<<<1, 64, 0, s>>>(plan->xcd_g_counters, kXcdMaxChains, 2u);
+        PLAN_HIP_CHECK(hipMalloc(&plan->xcd_claims, kXcdCount * kXcdMembers * sizeof(unsigned int)));
+        fill_u32_kernel<<<1, 256, 0, s>>>(plan->xcd_claims, kXcdCount * kXcdMembers, 0u);
+        PLAN_HIP_CHECK(hipGetLastError());
+    }
     PLAN_HIP_CHECK(hipStreamSynchronize(s));
 #undef PLAN_HIP_CHECK
     {
@@ -926,12 +973,30 @@ extern "C" int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan)
     return destroy_plan_locked(plan);
 }
 
+namespace
+{
+// Two workgroups of the one-recurrence-per-XCD kernel found themselves with the same rank on the same XCD: that launch's
+// results are undefined, and the plan stops choosing that kernel by itself.
+int xcd_placement_failure(PimHipLstmPlan* plan)
+{
+    plan->xcd_ok = false;
+    if (plan->mode == 4) plan->mode = 0;
+    return fail(PIMHIP_ERR_TIMEOUT, "the workgroups of the per-XCD LSTM kernel were not dealt to the XCDs in rotation (workgroup %u, on "
+                                    "XCD %u, found its rank taken): the results of that forward are undefined; this plan uses the "
+                                    "other kernels from now on",
+                plan->abort_host[1], plan->abort_host[2]);
+}
+}  // namespace
+
 extern "C" int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode)
 {
     if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
-    if (mode < 0 || mode > 3) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "mode %d not in {0, 1, 2, 3}", mode);
-    if (mode >= 2 && !plan->seq_kernel_ok)
+    if (mode < 0 || mode > 4) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "mode %d not in {0, 1, 2, 3, 4}", mode);
+    if ((mode == 2 || mode == 3) && !plan->seq_kernel_ok)
         return fail(PIMHIP_ERR_UNSUPPORTED, "hidden_size %lld does not fit the persistent sequence kernel", (long long)plan->hidden);
+    if (mode == 4 && !plan->xcd_ok)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "hidden_size %lld does not fit one XCD's registers, or this device is not laid out as 8 XCDs of "
+                                            "32 CUs", (long long)plan->hidden);
     // Modes 3 and 0 / 2 lay out a single chain's exchange entries differently: start over from a cleared buffer.
     if ((plan->mode == 3) != (mode == 3)) plan->reset_exchange = true;
     plan->mode = mode;
@@ -951,8 +1016,10 @@ extern "C" int pimhip_lstm_plan_status(PimHipLstmPlan* plan)
     if (*plan->abort_host != 0u) {
         // Reported once, here or by the next pimhip_lstm_forward, whichever comes first.  The caller has synchronised
         // the stream, so the kernel that set the word has ended and nothing sets it again after it is cleared.
+        const bool misplaced = *plan->abort_host == 2u;
         *plan->abort_host = 0u;
         plan->reset_exchange = true;
+        if (misplaced) return xcd_placement_failure(plan);
         return fail(PIMHIP_ERR_TIMEOUT, "a bounded wait of the persistent LSTM kernel gave up: the results of that forward are undefined");
     }
     return PIMHIP_OK;
@@ -1017,7 +1084,15 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     const bool capturing = capture != hipStreamCaptureStatusNone;
     // One step: the fused step kernel in every mode (the persistent kernel's hand-over of its step count to the next
     // launch needs two super-steps).
-    const bool use_seq = T >= 2 && T + kSeqMaxChains <= kSeqMaxT && (plan->mode >= 2 || (plan->mode == 0 && plan->seq_kernel_ok));
+    // Automatic choice: one recurrence per XCD where its groups have something to run side by side or nothing to gain
+    // from a wavefront (the two directions of a layer; a single unidirectional layer), the layer wavefront otherwise.
+    // (Measured on MI355X, whole calls: the per-XCD kernel is 13-30 % faster than the all-CU one for bidirectional layers
+    // from 16 steps on, and 7-17 % for a single unidirectional layer from 16 steps at H <= 512 and from 64 at H = 1024; its
+    // 32 CUs take longer to load the weights, which shorter sequences do not win back.)
+    const bool xcd_pays = (D == 2 && T >= 16) || (D == 1 && L == 1 && T >= (H > 512 ? 64 : 16));
+    const bool use_xcd = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && (plan->mode == 4 || (plan->mode == 0 && xcd_pays));
+    const bool use_seq = !use_xcd && T >= 2 && T + kSeqMaxChains <= kSeqMaxT &&
+                         (plan->mode == 2 || plan->mode == 3 || (plan->mode == 0 && plan->seq_kernel_ok));
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
     if (*plan->abort_host != 0u) {
         // An earlier sequence kernel of this plan gave up a wait and nobody has asked pimhip_lstm_plan_status since:
@@ -1028,21 +1103,31 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             return fail(PIMHIP_ERR_UNSUPPORTED, "an earlier forward of this plan gave up a wait; recovering from that is not for a "
                                                 "graph: call pimhip_lstm_plan_status or one forward outside the capture first");
         PIMHIP_HIP_CHECK(hipStreamSynchronize(s));
+        const bool misplaced = *plan->abort_host == 2u;
         *plan->abort_host = 0u;
         plan->reset_exchange = true;
+        if (misplaced) return xcd_placement_failure(plan);
         return fail(PIMHIP_ERR_TIMEOUT, "an earlier forward of this plan gave up a wait of the persistent LSTM kernel: its results "
                                         "are undefined (this call was not launched; the next one starts from a re-initialised exchange buffer)");
     }
-    if (use_seq && plan->reset_exchange) {
+    if ((use_seq || use_xcd) && plan->reset_exchange) {
         // After a time-out or a change of the entry layout: re-arm the flag and bring the exchange buffer and its step
         // counters back to their initial state.
         if (capturing)
             return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's exchange buffer has to be re-initialised (after a time-out or a change of "
                                                 "mode), which a graph must not record: run one forward outside the capture first");
         fill_u32_kernel<<<1, 1, 0, s>>>(plan->abort_flag, 1, 0u);
-        const size_t words = plan->hx_region_words * kSeqMaxChains;
-        fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->hx, words, 0u);
-        fill_u32_kernel<<<1, 64, 0, s>>>(plan->g_counters, kSeqMaxChains + 1, 2u);
+        if (plan->hx) {
+            const size_t words = plan->hx_region_words * kSeqMaxChains;
+            fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->hx, words, 0u);
+            fill_u32_kernel<<<1, 64, 0, s>>>(plan->g_counters, kSeqMaxChains + 1, 2u);
+        }
+        if (plan->xcd_hx) {
+            const size_t words = (size_t)kXcdRegionWords * kXcdMaxChains;
+            fill_u32_kernel<<<(unsigned)((words + 255) / 256), 256, 0, s>>>(plan->xcd_hx, words, 0u);
+            fill_u32_kernel<<<1, 64, 0, s>>>(plan->xcd_g_counters, kXcdMaxChains, 2u);
+            fill_u32_kernel<<<1, 256, 0, s>>>(plan->xcd_claims, kXcdCount * kXcdMembers, 0u);
+        }
         PIMHIP_HIP_CHECK(hipGetLastError());
         plan->reset_exchange = false;
     }
@@ -1051,7 +1136,57 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
 
     const half_t* layer_in = (const half_t*)x;
     const long y_stride = (long)D * H;
-    if (use_seq) {
+    if (use_xcd) {
+        // The groups of a launch have to be resident together, like the sequence kernel's blocks.
+        if (!capturing) {
+            rc = order_after_previous_sequence_launch(st, s);
+            if (rc != PIMHIP_OK) return rc;
+        }
+        const int members = (int)((H + kXcdUnitsPerBlock - 1) / kXcdUnitsPerBlock);
+        for (int l = 0; l < L; ++l) {
+            half_t* layer_out = (l == L - 1) ? (half_t*)y : plan->ybuf[l & 1];
+            const int64_t in_w = plan->cells[(size_t)l * D].in_w;
+            const PimHipLstmPlan::Cell& c0 = plan->cells[(size_t)l * D];
+            const PimHipLstmPlan::Cell& c1 = plan->cells[(size_t)l * D + (D - 1)];
+            float* outs2[2] = {plan->xproj, plan->xproj + (size_t)plan->max_seq_len * 4 * H};
+            const float* bs2[2] = {c0.bsum, c1.bsum};
+            if (c0.w_ih_packed && c1.w_ih_packed) {
+                const half_t* ws2[2] = {c0.w_ih_packed, c1.w_ih_packed};
+                rc = launch_input_projection_packed(D, outs2, layer_in, ws2, bs2, T, in_w, 4 * H, c0.ksteps, s);
+            } else {
+                const half_t* ws2[2] = {c0.w_ih, c1.w_ih};
+                rc = launch_input_projection(D, outs2, layer_in, ws2, bs2, T, in_w, 4 * H, s);
+            }
+            if (rc != PIMHIP_OK) return rc;
+            LstmXcdArgs a;
+            memset(&a, 0, sizeof(a));
+            for (int d = 0; d < D; ++d) {
+                const int ci = l * D + d;
+                XcdChain& ch = a.chain[d];
+                ch.w_hh = plan->cells[ci].w_hh;
+                ch.xproj = outs2[d];
+                ch.h0 = h0p + (size_t)ci * H;
+                ch.c0 = c0p + (size_t)ci * H;
+                ch.hn = hnp + (size_t)ci * H;
+                ch.cn = cnp + (size_t)ci * H;
+                ch.y = layer_out + (size_t)d * H;
+                ch.reverse = d;
+                a.role[d] = d + 1;  // direction d on XCD d
+            }
+            a.hx = plan->xcd_hx;
+            a.g_counter = plan->xcd_g_counters;
+            a.claims = plan->xcd_claims;
+            a.abort_flag = plan->abort_flag;
+            a.abort_host = plan->abort_host_dev;
+            a.y_stride = y_stride;
+            a.H = (int)H;
+            a.T = (int)T;
+            a.spin_limit = plan->spin_limit;
+            lstm_xcd_f16_kernel<<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+            PIMHIP_HIP_CHECK(hipGetLastError());
+            layer_in = layer_out;
+        }
+    } else if (use_seq) {
         // (Not on a capturing stream, where an event of another stream cannot be waited for: a caller who replays
         // graphs orders them against the device's other sequence launches.)
         if (!capturing) {

@@ -131,10 +131,12 @@ def test_sequence_forward_replays_from_a_graph(ops):
     """The persistent sequence kernel keeps its step count in device memory, so a recorded launch replays: every replay
     equals the eager launch bit for bit, with eager launches of the same plan between the replays.  The one thing a
     graph must not record, the re-initialisation of the exchange buffer after a change of mode, is refused."""
-    T, I, Hs = 7, 64, 256
-    for layers, bidir in ((2, False), (1, True), (1, False)):
-        params, x, h0, c0 = workloads.lstm_inputs(7101 + layers + 2 * bidir, I, Hs, layers, bidir, T)
+    I, Hs = 64, 256
+    # (the last two run one recurrence per XCD: a bidirectional layer of 20 steps in automatic mode, and mode 4 by request)
+    for layers, bidir, T, mode in ((1, True, 20, 0), (1, False, 18, 4), (2, False, 7, 0), (1, True, 7, 0), (1, False, 7, 0)):
+        params, x, h0, c0 = workloads.lstm_inputs(7101 + layers + 2 * bidir + T, I, Hs, layers, bidir, T)
         plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, bidir, T)
+        plan.set_mode(mode)
         xd, hd, cd = x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV)
         x2 = (0.5 * xd + 0.25).contiguous()
         eager = {k: [t.clone() for t in plan.forward(v, hd, cd)] for k, v in (("a", xd), ("b", x2))}

@@ -14,7 +14,9 @@ from pimaicompiler_amd import workloads
 pytestmark = pytest.mark.gpu
 LSTM_TOL = 5e-3
 DEV = "cuda:0"
-MODES = [1, 2, 3]  # 1: one fused launch per step, 2: persistent sequence kernel, 3: the same, four units per block always
+# 1: one fused launch per step, 2: persistent sequence kernel over all CUs, 3: the same, four units per block always,
+# 4: every recurrence on one XCD (hidden sizes up to 1024)
+MODES = [1, 2, 3, 4]
 
 
 def maxabs(a, b):
@@ -71,6 +73,8 @@ CASES = [  # I, H, L, bidirectional, T, biases
 def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
     if mode >= 2 and H > 2048:
         pytest.skip("the persistent kernel takes hidden sizes up to 2048; larger ones run step by step")
+    if mode == 4 and H > 1024:
+        pytest.skip("one XCD's registers hold the recurrent weights of hidden sizes up to 1024")
     params, x, h0, c0 = workloads.lstm_inputs(900 + I + H + T, I, H, L, bidir, T, has_b)
     g = torch.Generator().manual_seed(T)
     h0 = (0.3 * torch.randn(h0.shape, generator=g)).half()
@@ -87,6 +91,11 @@ def test_persistent_kernel_refuses_what_it_cannot_hold(ops):
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 2)
     with pytest.raises(ops.NNRuntimeException):
         plan.set_mode(2)
+    params, x, h0, c0 = workloads.lstm_inputs(1, 16, 1032, 1, False, 2)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 2)
+    plan.set_mode(2)
+    with pytest.raises(ops.NNRuntimeException, match="XCD"):
+        plan.set_mode(4)
 
 
 # ---- benchmark configurations -----------------------------------------------------------------------------------
@@ -234,7 +243,7 @@ def test_switching_the_block_shape_on_one_plan_restarts_the_exchange(ops):
     want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 23)
     outs = []
-    for mode in (2, 3, 3, 2, 0, 3, 1, 2):
+    for mode in (2, 3, 3, 2, 4, 0, 3, 4, 1, 2):
         plan.set_mode(mode)
         y, hn, cn = plan.forward(x.reshape(23, 64).to(DEV), h0.to(DEV), c0.to(DEV))
         plan.status()
@@ -269,13 +278,56 @@ def test_sequence_kernels_issued_on_two_streams_do_not_starve_each_other(ops):
         assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
 
 
+def test_automatic_mode_takes_the_per_xcd_kernel_where_it_pays(ops):
+    """Bidirectional layers from 16 steps on and single unidirectional layers from 64 (16 at H <= 512) run one recurrence
+    per XCD in automatic mode: the same bits as mode 4, which sums in another order than mode 2."""
+    for I, H, L, bidir, T, same_as in [(32, 256, 2, True, 40, 4), (32, 1024, 1, False, 70, 4), (32, 1024, 1, False, 20, 2),
+                                        (32, 256, 1, False, 20, 4), (32, 256, 3, False, 40, 2), (32, 256, 1, True, 9, 2)]:
+        params, x, h0, c0 = workloads.lstm_inputs(800 + T, I, H, L, bidir, T)
+        y0, _, c0n = run_plan(ops, params, x, h0, c0, True, L, bidir, 0)
+        ym, _, cmn = run_plan(ops, params, x, h0, c0, True, L, bidir, same_as)
+        assert torch.equal(y0, ym) and torch.equal(c0n, cmn), (I, H, L, bidir, T)
+        want = oracle.torch_lstm(x, h0, c0, params, True, L, bidir)
+        assert maxabs(y0, want[0]) <= 2e-3 and maxabs(c0n, want[2]) <= 2e-3
+
+
+def test_per_xcd_kernel_finds_its_groups_on_any_queue(ops):
+    """Workgroup b of a launch runs on XCD (b + o) % 8, with a start o that belongs to the hardware queue and moves over a
+    process's life (this test is placed after ones that use several streams for that reason): the kernel takes its
+    groups from the hardware's XCC_ID, so it is right on every stream, whatever o is there."""
+    from pimaicompiler_amd import _lib as L
+    lib = L.load()
+    params, x, h0, c0 = workloads.lstm_inputs(611, 48, 512, 1, True, 24)
+    want = oracle.torch_lstm(x, h0, c0, params, True, 1, True)
+    pd = [p.to(DEV) for p in params]
+    xd, hd, cd = x.reshape(24, 48).to(DEV), h0.to(DEV), c0.to(DEV)
+    starts = []
+    for st in [torch.cuda.current_stream()] + [torch.cuda.Stream() for _ in range(5)]:
+        where = torch.full((64,), -1, dtype=torch.int32, device=DEV)
+        torch.cuda.synchronize()
+        assert lib.pimhip_probe_xcc_map(where.data_ptr(), 64, 512, st.cuda_stream) == 0
+        st.synchronize()
+        m = where.cpu().tolist()
+        assert all(0 <= v < 8 for v in m) and all(m[b] == (m[0] + b) % 8 for b in range(64)), m     # a rotation
+        starts.append(m[0])
+        plan = ops.LstmPlan(pd, True, 1, True, 24)
+        plan.set_mode(4)
+        with torch.cuda.stream(st):
+            y, hn, cn = plan.forward(xd, hd, cd, stream=st)
+        st.synchronize()
+        plan.status()
+        assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
+    print("first workgroup's XCD per stream:", starts, flush=True)
+
+
 # ---- the bounded wait ---------------------------------------------------------------------------------------------
-def test_persistent_kernel_wait_gives_up_and_reports(ops):
+@pytest.mark.parametrize("mode", [2, 4])
+def test_persistent_kernel_wait_gives_up_and_reports(ops, mode):
     """Forced from the host: with a spin limit of 0 every wait gives up at its first unsuccessful poll, the kernel
     still runs to its end, and the plan reports the time-out.  A later forward with the default limit works."""
     params, x, h0, c0 = workloads.lstm_inputs(123, 64, 1024, 1, False, 30)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 30)
-    plan.set_mode(2)
+    plan.set_mode(mode)
     plan.set_spin_limit(0)
     plan.forward(x.reshape(30, 64).to(DEV), h0.to(DEV), c0.to(DEV))
     with pytest.raises(ops.NNRuntimeException, match="gave up"):
@@ -340,7 +392,7 @@ def test_plan_cache_follows_weight_updates_and_is_bounded(ops):
     assert ops.invalidate_lstm_plans() == O.PLAN_CACHE_MAX
 
 
-@pytest.mark.parametrize("mode", [2, 3])
+@pytest.mark.parametrize("mode", [2, 3, 4])
 def test_persistent_kernel_survives_a_nan_input(ops, mode):
     """A NaN cannot carry the exchange's flag bit, so it is exchanged as 0; the cell state keeps it, and y is NaN from
     that step on exactly as in LibTorch.  No wait times out."""
