@@ -24,6 +24,16 @@
 // that cache behaviour: a stale piece fails its flag check and is polled again; only the time a poll takes does.
 // Every wait is bounded (spin_limit polls, then the abort flag, as in lstm_seq_f16_kernel).
 //
+// A stack of unidirectional layers runs as a pipeline over the XCDs: layer k's recurrence (group R_k) on one XCD, and for
+// k >= 1 a second group P_k on another XCD that holds W_ih of layer k and turns every h of layer k - 1 into layer k's
+// input-projection row as soon as it exists.  R_{k-1} hands its h_t to P_k, and P_k its row to R_k, through buffers in
+// memory with one slot per time step (device-scope stores and loads; a slot is written once per launch, so there is no
+// flow control): the host fills them with all-ones bytes before the launch, a pattern that neither an fp16 h (a NaN is
+// stored in its canonical form there) nor an fp32 sum can be, and a reader polls a slot until none of its elements is
+// that pattern.  Those hand-overs cross XCDs and take about a microsecond, but they are not on the recurrences' critical
+// path: P_k looks one step ahead while it multiplies, R_k starts a few steps late and from then on finds its rows
+// waiting.  All groups then advance at the rate of one group, L layers in about the time of one.
+//
 // A workgroup has eight wavefronts; wavefront w owns hidden units 32 * rank + 4 * w .. + 3, one per row of 16 lanes:
 // lane l keeps, of the four gate rows of unit l >> 4, the 8-wide column pieces 16 c + (l & 15), c = 0..7, in 128 registers
 // for the whole sequence.  Per step: lanes 0..15 of every wavefront fetch one 16-byte piece of the group's entries into
@@ -49,19 +59,32 @@ static constexpr int kXcdRegionWords = 2 * kXcdMembers * kXcdEntryWords;  // one
 
 struct XcdChain {
     const half_t* w_hh;   // [4H, H]
-    const float* xproj;   // [T, 4H] fp32 with biases
+    const float* xproj;   // [T, 4H] fp32 with biases: computed before the launch, or filled during it by the layer's P group
     const half_t* h0;     // [H]
     const half_t* c0;     // [H]
-    half_t* y;            // row t at y + t * y_stride
+    half_t* y;            // row t at y + t * y_stride; null for an inner layer of a pipeline
     half_t* hn;           // [H]
     half_t* cn;           // [H]
+    half_t* seq_out;      // [T][H], one slot per step, read by the P group of the layer above; null for the last layer
     int reverse;          // 1: t = T-1 .. 0
+    int xproj_polled;     // 1: the rows of xproj are written during this launch (all-ones bytes = not yet)
 };
+
+struct XcdProj {
+    const half_t* w_ih;    // [4H, H] of the layer this group feeds
+    const float* bsum;     // [4H] fp32 b_ih + b_hh
+    const half_t* seq_in;  // [T][H]: the h of the layer below, slot t filled during this launch
+    float* xp_out;         // [T][4H]: the xproj of the layer this group feeds
+};
+
+static constexpr int kXcdRoleProj = 9;  // role values: 0 none, 1 + k recurrence of chain k, kXcdRoleProj + j projection j
+static constexpr int kXcdLag = 2;       // steps a recurrence fed by a P group lets that group get ahead before it starts
 
 struct LstmXcdArgs {
     XcdChain chain[kXcdMaxChains];
-    int role[kXcdCount];       // chain index + 1 of the group that runs on the XCD with this hardware index, 0: none
-    unsigned int* claims;      // [kXcdCount][kXcdMembers]: the launch (its chain's counter value) that last took (XCD, rank)
+    XcdProj proj[kXcdMaxChains - 1];  // proj[j] feeds chain[j + 1]
+    int role[kXcdCount];       // what the group on the XCD with this hardware index runs
+    unsigned int* claims;      // [kXcdCount][kXcdMembers]: the launch (a counter value of the plan) that last took (XCD, rank)
     unsigned int* hx;          // [kXcdMaxChains] regions of kXcdRegionWords; zero when the chain's counter is 2
     unsigned int* g_counter;   // [kXcdMaxChains] device words: super-steps a chain's region has seen so far, plus 2
     unsigned int* abort_flag;
@@ -71,6 +94,11 @@ struct LstmXcdArgs {
     int T;
     unsigned int spin_limit;
 };
+
+// The barrier of a step: LDS traffic of this wavefront done, then s_barrier.  __syncthreads() would also wait for every
+// global store and load the wavefront has in flight (its release semantics cover global memory), and some of those cross
+// to another XCD and back; nothing that passes between the wavefronts of a workgroup here goes through global memory.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __device__ __forceinline__ void load16_nt(const void* p, unsigned long long& lo, unsigned long long& hi)
 {
@@ -107,6 +135,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
 {
     __shared__ __align__(16) half_t hbuf[2][kXcdMaxH];  // h of the previous step, double buffered by step parity
     __shared__ __align__(16) float xring[kXcdWaves][32][4][4];  // per wavefront: [step & 31][gate][unit] projection terms
+    __shared__ __align__(16) unsigned long long hout[2][kXcdWaves];  // the workgroup's 32 new h values, for the layer above
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -119,8 +148,10 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     const int T = p.T;
     const int members = (H + kXcdUnitsPerBlock - 1) / kXcdUnitsPerBlock;
     if (role == 0 || rank >= members) return;  // whole workgroups, before any barrier
-    const int k = role - 1;
+    const bool is_proj = role >= kXcdRoleProj;
+    const int k = is_proj ? role - kXcdRoleProj + 1 : role - 1;  // the chain this group runs or feeds
     const XcdChain& ch = p.chain[k];
+    const XcdProj& pj = p.proj[is_proj ? k - 1 : 0];
 
     bool gave_up = false;
     const unsigned int g_base = __builtin_amdgcn_readfirstlane(
@@ -136,6 +167,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     const int u0 = rank * kXcdUnitsPerBlock + wave * kXcdUnitsPerWave;
     const bool units_ok = u0 < H;  // H % 8 == 0: the four units of a wavefront are all inside or all outside
     const int cl = lane & 15;
+    const half_t* wsrc = is_proj ? pj.w_ih : ch.w_hh;
     half8_t w[4][8];
     {
         half8_t zero;
@@ -148,7 +180,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
                 const int col = (16 * c + cl) * 8;
                 const bool ok = units_ok && col < H;
                 const long off = ((long)g * H + (u0 + (lane >> 4))) * H + col;
-                w[g][c] = ok ? *reinterpret_cast<const half8_t*>(ch.w_hh + off) : zero;
+                w[g][c] = ok ? *reinterpret_cast<const half8_t*>(wsrc + off) : zero;
             }
         }
         for (int i = tid; i < 2 * kXcdMaxH / 8; i += kXcdThreads) reinterpret_cast<half8_t*>(&hbuf[0][0])[i] = zero;
@@ -165,14 +197,92 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     const int my_unit = u0 + (lane >> 4);
     const int my_gate = (lane >> 2) & 3;
     const int uc = units_ok ? my_unit : H - 1;
+    // Lanes 0..31 of wavefronts 0..3 fetch piece 32 w + lane of an h vector: 8 fp16 = columns 8 q .. 8 q + 7.  (The other
+    // wavefronts never poll: they are the ones that talk to other XCDs, and a wavefront's loads come back in order.)
+    const int piece = wave * 32 + lane;
+    const bool polls = wave < 4 && lane < 32 && piece * 8 < H;
+
+    // One bounded wait: `again` loads and tests; gives up like every wait of this kernel.
+    auto bounded_wait = [&](auto again) __attribute__((always_inline)) {
+        unsigned int spins = 0;
+        while (!again() && !gave_up) {
+            ++spins;
+            if ((spins & 255u) == 0u) {
+                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
+            }
+            if (spins >= p.spin_limit) {
+                __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                gave_up = true;
+            }
+        }
+    };
+    // true if none of the four fp16 of the word is the all-ones pattern
+    auto filled16 = [](unsigned long long v) {
+        const unsigned long long x = ~v;  // an all-ones fp16 becomes zero
+        return ((x & 0xffffull) != 0ull) && ((x & 0xffff0000ull) != 0ull) && ((x & 0xffff00000000ull) != 0ull) && ((x >> 48) != 0ull);
+    };
+
+    if (is_proj) {
+        // ================= P group: xproj rows of layer k from the h of layer k - 1, step by step =================
+        const float bias = pj.bsum[(long)my_gate * H + uc];
+        float* dst = pj.xp_out + (long)my_gate * H + uc;
+        unsigned long long lo = 0ull, hi = 0ull;  // this lane's piece of the step ahead
+        if (polls) {
+            lo = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(pj.seq_in + piece * 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            hi = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(pj.seq_in + piece * 8) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        for (int t = 0; t < T; ++t) {
+            half_t* hb = hbuf[t & 1];
+            if (polls) {
+                const unsigned long long* src = reinterpret_cast<const unsigned long long*>(pj.seq_in + (long)t * H + piece * 8);
+                if (!(filled16(lo) && filled16(hi))) {
+                    bounded_wait([&]() {
+                        load16_device_scope(src, lo, hi);
+                        return filled16(lo) && filled16(hi);
+                    });
+                }
+                typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+                const u64x2 both = {lo, hi};
+                *reinterpret_cast<half8_t*>(hb + piece * 8) = __builtin_bit_cast(half8_t, both);
+            }
+            lds_barrier();
+            if (polls && t + 1 < T) {
+                // the step ahead, in flight while this one is multiplied (tested at the top of the next iteration)
+                const unsigned long long* nxt = reinterpret_cast<const unsigned long long*>(pj.seq_in + (long)(t + 1) * H + piece * 8);
+                lo = __hip_atomic_load(nxt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                hi = __hip_atomic_load(nxt + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                if (c * 128 >= H) break;
+                const half8_t hv = *reinterpret_cast<const half8_t*>(hb + (16 * c + cl) * 8);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) acc[g] = dot8(w[g][c], hv, acc[g]);
+            }
+            const float v = row16_transpose_sum4(acc, lane) + bias;
+            if (units_ok && (lane & 3) == 0)
+                __hip_atomic_store(reinterpret_cast<unsigned int*>(dst + (long)t * 4 * H), __builtin_bit_cast(unsigned int, v), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+
+    // ================= R group: the recurrence of chain k =================
     float c_reg = (float)ch.c0[uc];
     const bool rev = ch.reverse != 0;
+    const bool polled = ch.xproj_polled != 0;
+    const bool feeds = ch.seq_out != nullptr;
 
     // The input-projection term does not depend on h and must stay off the step's critical path: a wavefront's loads
     // return in order, so a poll issued behind a load that misses the L2 would wait for it.  Each wavefront keeps the
-    // terms of its 16 rows for 32 steps in LDS (two halves of 16 steps) and refills the half it has used up with ONE
-    // 16-byte load per lane every 16 steps: lane l fetches gate l & 3 of the wavefront's four units (adjacent in a row of
-    // xproj) for step offset l >> 2.
+    // terms of its 16 rows for up to 32 steps in LDS.  Rows that exist before the launch are fetched 16 steps at a time,
+    // ONE 16-byte load per lane every 16 steps (lane l: gate l & 3 of the wavefront's four units, adjacent in a row of
+    // xproj, for step offset l >> 2).  Rows that a P group writes during the launch are fetched one element per lane two
+    // steps ahead, right after the step's barrier so that the load travels while the step is computed, and tested when
+    // they are used; the wavefronts that poll for h leave that to wavefronts 4..7, which fetch the elements of wavefront
+    // w - 4 beside their own (a poll would have to wait for such a load to come back from the other XCD first).
     const int u0c = units_ok ? u0 : H - 4;
     auto fetch_xp = [&](int s0) {
         const int sx = min(s0 + (lane >> 2), T - 1);
@@ -182,20 +292,43 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     auto deposit_xp = [&](int half, const float4_t v) {
         *reinterpret_cast<float4_t*>(&xring[wave][half * 16 + (lane >> 2)][lane & 3][0]) = v;
     };
-    deposit_xp(0, fetch_xp(0));
-    deposit_xp(1, fetch_xp(16));
+    const unsigned int* xp_mine = reinterpret_cast<const unsigned int*>(ch.xproj + (long)my_gate * H + uc);  // + t * 4H
+    const bool fetcher = wave >= 4;
+    const unsigned int* xp_other =
+        reinterpret_cast<const unsigned int*>(ch.xproj + (long)my_gate * H + min(max(u0 - 16, 0) + (lane >> 4), H - 1));  // wavefront w - 4's
+    auto xp_bits_at = [&](int t) { return __hip_atomic_load(xp_mine + (long)t * 4 * H, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    auto wait_xp = [&](int t) {
+        unsigned int bits = 0xffffffffu;
+        bounded_wait([&]() {
+            bits = xp_bits_at(t);
+            return bits != 0xffffffffu;
+        });
+        return bits;
+    };
     float4_t xp_next = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-
-    // Lanes 0..15 of wavefront w fetch piece 16 w + lane of the group's entries: 8 fp16 = columns 8 q .. 8 q + 7 of h.
-    const int piece = wave * 16 + lane;
-    const bool polls = lane < 16 && piece * 8 < H;
+    unsigned int xp_ahead = 0xffffffffu, xp_ahead_other = 0xffffffffu;  // polled rows: the elements of step s + 2, loaded during step s
+    if (!polled) {
+        deposit_xp(0, fetch_xp(0));
+        deposit_xp(1, fetch_xp(16));
+    } else {
+        // Let the P group get kXcdLag steps ahead, then take the first two rows.
+        (void)wait_xp(min(kXcdLag, T - 1));
+        reinterpret_cast<unsigned int&>(xring[wave][0][my_gate][lane >> 4]) = wait_xp(0);
+        reinterpret_cast<unsigned int&>(xring[wave][1][my_gate][lane >> 4]) = wait_xp(min(1, T - 1));
+    }
 
     for (int s = 0; s < T; ++s) {
         half_t* hb = hbuf[s & 1];
-        // Refill of the projection terms: steps s + 16 .. s + 31 are fetched when step s starts a half, and written over
-        // the half that has just been used up one step later (this wavefront's poll in between has waited for them).
-        if ((s & 15) == 0 && s > 0) xp_next = fetch_xp(s + 16);
-        if ((s & 15) == 1 && s > 1) deposit_xp(((s >> 4) & 1) ^ 1, xp_next);
+        if (!polled) {
+            // steps s + 16 .. s + 31 are fetched when step s starts a half, and written over the half that has just been
+            // used up one step later (this wavefront's poll in between has waited for them)
+            if ((s & 15) == 0 && s > 0) xp_next = fetch_xp(s + 16);
+            if ((s & 15) == 1 && s > 1) deposit_xp(((s >> 4) & 1) ^ 1, xp_next);
+        } else if (fetcher && s >= 1 && s + 1 < T) {
+            // loaded during step s - 1; read (by this wavefront and by wavefront w - 4) after the barrier of step s + 1
+            reinterpret_cast<unsigned int&>(xring[wave][(s + 1) & 31][my_gate][lane >> 4]) = xp_ahead;
+            reinterpret_cast<unsigned int&>(xring[wave - 4][(s + 1) & 31][my_gate][lane >> 4]) = xp_ahead_other;
+        }
         // ---- 1. h of the previous step into LDS
         if (polls) {
             half8_t hv;
@@ -206,20 +339,10 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
                 const unsigned long long want = ((gp >> 1) & 1u) ? 0x4000400040004000ull : 0ull;
                 const unsigned char* src = reinterpret_cast<const unsigned char*>(region + (long)(gp & 1u) * kXcdMembers * kXcdEntryWords) + piece * 16;
                 unsigned long long lo = 0ull, hi = 0ull;
-                unsigned int spins = 0;
-                while (true) {
+                bounded_wait([&]() {
                     load16_nt(src, lo, hi);
-                    if (((lo & 0x4000400040004000ull) == want && (hi & 0x4000400040004000ull) == want) || gave_up) break;
-                    ++spins;
-                    if ((spins & 255u) == 0u) {
-                        if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
-                    }
-                    if (spins >= p.spin_limit) {
-                        __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                        gave_up = true;
-                    }
-                }
+                    return (lo & 0x4000400040004000ull) == want && (hi & 0x4000400040004000ull) == want;
+                });
                 lo &= 0xbfffbfffbfffbfffull;
                 hi &= 0xbfffbfffbfffbfffull;
                 typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
@@ -228,7 +351,17 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
             }
             *reinterpret_cast<half8_t*>(hb + piece * 8) = hv;
         }
-        __syncthreads();
+        lds_barrier();
+        if (polled && fetcher && s + 2 < T) {
+            xp_ahead = xp_bits_at(s + 2);
+            xp_ahead_other = __hip_atomic_load(xp_other + (long)(s + 2) * 4 * H, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // The previous step's h of the whole workgroup (gathered in LDS before the barrier) goes to the layer above, from a
+        // wavefront that does not poll.
+        if (feeds && s > 0 && wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) {
+            const unsigned long long* src = &hout[(s - 1) & 1][2 * lane];
+            store16_device_scope(ch.seq_out + (long)(s - 1) * H + rank * kXcdUnitsPerBlock + lane * 8, src[0], src[1]);
+        }
 
         // ---- 2. the four gate rows of this row of lanes' unit
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -239,7 +372,9 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
 #pragma unroll
             for (int g = 0; g < 4; ++g) acc[g] = dot8(w[g][c], hv, acc[g]);
         }
-        const float a = row16_transpose_sum4(acc, lane) + xring[wave][s & 31][my_gate][lane >> 4];
+        unsigned int xp_bits = reinterpret_cast<const unsigned int&>(xring[wave][s & 31][my_gate][lane >> 4]);
+        if (polled && xp_bits == 0xffffffffu) xp_bits = wait_xp(s);  // the P group had not got there when it was fetched
+        const float a = row16_transpose_sum4(acc, lane) + __builtin_bit_cast(float, xp_bits);
         const int t = rev ? (T - 1 - s) : s;
 
         // Every lane activates its own gate; a lane of gate 0 then finds gate f in its mirror within half the row (l ^ 7),
@@ -259,12 +394,14 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
 
         // ---- 3. the wavefront's four h values: lanes 0, 16, 32, 48 hold them; lane 0 stores y and publishes
         const unsigned int hb16 = (unsigned int)__builtin_bit_cast(unsigned short, h);
-        const unsigned int pb16 = h_is_number ? hb16 : 0u;  // a NaN cannot carry the flag: it is exchanged as 0, y keeps it
-        unsigned long long yw = 0ull, pw = 0ull;
+        const unsigned int pb16 = h_is_number ? hb16 : 0u;       // a NaN cannot carry the flag: it is exchanged as 0, y keeps it
+        const unsigned int sb16 = h_is_number ? hb16 : 0x7e00u;  // and goes to the layer above in its canonical form
+        unsigned long long yw = 0ull, pw = 0ull, sw = 0ull;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             yw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)hb16, 16 * i) << (16 * i);
             pw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)pb16, 16 * i) << (16 * i);
+            sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
         }
         if (lane == 0) {
             const unsigned int g = g_base + (unsigned int)s;
@@ -272,11 +409,19 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
             // units past H publish zeros with the flag, so that every piece of a member's entry validates
             unsigned char* dst = reinterpret_cast<unsigned char*>(region + ((long)(g & 1u) * kXcdMembers + rank) * kXcdEntryWords) + wave * 8;
             store8_plain(dst, (units_ok ? pw : 0ull) | flag);
-            if (units_ok) *reinterpret_cast<unsigned long long*>(ch.y + (long)t * p.y_stride + u0) = yw;
+            if (units_ok && ch.y) *reinterpret_cast<unsigned long long*>(ch.y + (long)t * p.y_stride + u0) = yw;
+            if (feeds) hout[s & 1][wave] = sw;
         }
         if (s == T - 1 && units_ok && (lane & 15) == 0) {
             ch.hn[my_unit] = h;
             ch.cn[my_unit] = (half_t)c_new;
+        }
+    }
+    if (feeds) {
+        lds_barrier();
+        if (wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) {
+            const unsigned long long* src = &hout[(T - 1) & 1][2 * lane];
+            store16_device_scope(ch.seq_out + (long)(T - 1) * H + rank * kXcdUnitsPerBlock + lane * 8, src[0], src[1]);
         }
     }
     // Rank 0 has finished its last step, for which (T >= 2) it needed what every member published one step earlier:

@@ -45,6 +45,18 @@ int fail(int status, const char* fmt, ...)
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Up to six ranges of 32-bit words set to one value in one launch (blockIdx.y = range).
+struct FillSegments {
+    unsigned int* ptr[6];
+    size_t words[6];
+};
+__global__ void fill_segments_kernel(FillSegments seg, unsigned int v)
+{
+    unsigned int* p = seg.ptr[blockIdx.y];
+    const size_t n = seg.words[blockIdx.y];
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
 __global__ void fill_u32_kernel(unsigned int* p, size_t n, unsigned int v)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -748,6 +760,10 @@ struct PimHipLstmPlan {
     unsigned int* xcd_hx = nullptr;  // [kXcdMaxChains] regions of kXcdRegionWords, zero when the chain's counter is 2
     unsigned int* xcd_g_counters = nullptr;  // [kXcdMaxChains]
     unsigned int* xcd_claims = nullptr;      // [kXcdCount][kXcdMembers], zero when the counters are 2
+    // Unidirectional stacks in mode 4 run as a pipeline over the XCDs: per boundary between two layers of a launch, the
+    // lower layer's h per step ([max_seq_len][H] fp16) and the upper layer's projection rows ([max_seq_len][4H] fp32).
+    unsigned char* xcd_pipe = nullptr;
+    size_t xcd_pipe_boundary_bytes = 0;
 };
 
 namespace
@@ -770,6 +786,7 @@ int destroy_plan_locked(PimHipLstmPlan* plan)
     if (plan->xcd_hx) hipFree(plan->xcd_hx);
     if (plan->xcd_g_counters) hipFree(plan->xcd_g_counters);
     if (plan->xcd_claims) hipFree(plan->xcd_claims);
+    if (plan->xcd_pipe) hipFree(plan->xcd_pipe);
     if (plan->abort_flag) hipFree(plan->abort_flag);
     if (plan->abort_host) hipHostFree(plan->abort_host);
     if (prev >= 0) hipSetDevice(prev);
@@ -952,6 +969,11 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         PLAN_HIP_CHECK(hipMalloc(&plan->xcd_claims, kXcdCount * kXcdMembers * sizeof(unsigned int)));
         fill_u32_kernel<<<1, 256, 0, s>>>(plan->xcd_claims, kXcdCount * kXcdMembers, 0u);
         PLAN_HIP_CHECK(hipGetLastError());
+        if (D == 1 && num_layers >= 2) {
+            plan->xcd_pipe_boundary_bytes = (size_t)max_seq_len * H * (sizeof(half_t) + 4 * sizeof(float));
+            const int boundaries = (num_layers < kXcdMaxChains ? num_layers : kXcdMaxChains) - 1;
+            PLAN_HIP_CHECK(hipMalloc(&plan->xcd_pipe, plan->xcd_pipe_boundary_bytes * boundaries));
+        }
     }
     PLAN_HIP_CHECK(hipStreamSynchronize(s));
 #undef PLAN_HIP_CHECK
@@ -1143,7 +1165,74 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             if (rc != PIMHIP_OK) return rc;
         }
         const int members = (int)((H + kXcdUnitsPerBlock - 1) / kXcdUnitsPerBlock);
-        for (int l = 0; l < L; ++l) {
+        // A unidirectional stack: up to kXcdMaxChains layers per launch as a pipeline over the XCDs (recurrence of layer
+        // j of the launch on XCD 2 j, the group that makes its projection rows from the layer below on XCD 2 j - 1).
+        for (int l = 0; D == 1 && L >= 2 && l < L;) {
+            const int n = (L - l) < kXcdMaxChains ? (L - l) : kXcdMaxChains;
+            const int last = l + n - 1;
+            half_t* group_out = (last == L - 1) ? (half_t*)y : plan->ybuf[last & 1];
+            const PimHipLstmPlan::Cell& cf = plan->cells[(size_t)l];
+            if (cf.w_ih_packed) {
+                float* outs1[1] = {plan->xproj};
+                const half_t* ws1[1] = {cf.w_ih_packed};
+                const float* bs1[1] = {cf.bsum};
+                rc = launch_input_projection_packed(1, outs1, layer_in, ws1, bs1, T, cf.in_w, 4 * H, cf.ksteps, s);
+            } else {
+                rc = launch_input_projection(plan->xproj, layer_in, cf.w_ih, cf.bsum, T, cf.in_w, 4 * H, s);
+            }
+            if (rc != PIMHIP_OK) return rc;
+            LstmXcdArgs a;
+            memset(&a, 0, sizeof(a));
+            FillSegments seg;
+            memset(&seg, 0, sizeof(seg));
+            for (int j = 0; j < n; ++j) {
+                const int ci = l + j;
+                XcdChain& ch = a.chain[j];
+                ch.w_hh = plan->cells[ci].w_hh;
+                ch.h0 = h0p + (size_t)ci * H;
+                ch.c0 = c0p + (size_t)ci * H;
+                ch.hn = hnp + (size_t)ci * H;
+                ch.cn = cnp + (size_t)ci * H;
+                ch.y = (j == n - 1) ? group_out : nullptr;
+                a.role[2 * j] = j + 1;
+                if (j == 0) {
+                    ch.xproj = plan->xproj;
+                } else {
+                    unsigned char* boundary = plan->xcd_pipe + plan->xcd_pipe_boundary_bytes * (size_t)(j - 1);
+                    half_t* seq = reinterpret_cast<half_t*>(boundary);
+                    float* xp = reinterpret_cast<float*>(boundary + (size_t)plan->max_seq_len * H * sizeof(half_t));
+                    a.chain[j - 1].seq_out = seq;
+                    ch.xproj = xp;
+                    ch.xproj_polled = 1;
+                    XcdProj& pj = a.proj[j - 1];
+                    pj.w_ih = plan->cells[ci].w_ih;
+                    pj.bsum = plan->cells[ci].bsum;
+                    pj.seq_in = seq;
+                    pj.xp_out = xp;
+                    a.role[2 * j - 1] = kXcdRoleProj + (j - 1);
+                    // this launch's slots start out as "not written yet": all-ones bytes
+                    seg.ptr[2 * (j - 1)] = reinterpret_cast<unsigned int*>(seq);
+                    seg.words[2 * (j - 1)] = (size_t)T * H / 2;
+                    seg.ptr[2 * (j - 1) + 1] = reinterpret_cast<unsigned int*>(xp);
+                    seg.words[2 * (j - 1) + 1] = (size_t)T * 4 * H;
+                }
+            }
+            if (n > 1) fill_segments_kernel<<<dim3(64, 2 * (n - 1)), 256, 0, s>>>(seg, 0xffffffffu);
+            a.hx = plan->xcd_hx;
+            a.g_counter = plan->xcd_g_counters;
+            a.claims = plan->xcd_claims;
+            a.abort_flag = plan->abort_flag;
+            a.abort_host = plan->abort_host_dev;
+            a.y_stride = y_stride;
+            a.H = (int)H;
+            a.T = (int)T;
+            a.spin_limit = plan->spin_limit;
+            lstm_xcd_f16_kernel<<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+            PIMHIP_HIP_CHECK(hipGetLastError());
+            layer_in = group_out;
+            l += n;
+        }
+        for (int l = 0; (D == 2 || L == 1) && l < L; ++l) {
             half_t* layer_out = (l == L - 1) ? (half_t*)y : plan->ybuf[l & 1];
             const int64_t in_w = plan->cells[(size_t)l * D].in_w;
             const PimHipLstmPlan::Cell& c0 = plan->cells[(size_t)l * D];
