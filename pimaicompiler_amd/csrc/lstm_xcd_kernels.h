@@ -131,6 +131,9 @@ __device__ __forceinline__ float row16_transpose_sum4(const float (&acc)[4], int
     return v;
 }
 
+// PIPE = false: groups that neither feed nor are fed across XCDs (a single layer, the two directions of one); everything
+// that concerns P groups and the hand-overs is compiled out, which is worth 10 % of a step.
+template <bool PIPE>
 __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p)
 {
     __shared__ __align__(16) half_t hbuf[2][kXcdMaxH];  // h of the previous step, double buffered by step parity
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     const int T = p.T;
     const int members = (H + kXcdUnitsPerBlock - 1) / kXcdUnitsPerBlock;
     if (role == 0 || rank >= members) return;  // whole workgroups, before any barrier
-    const bool is_proj = role >= kXcdRoleProj;
+    const bool is_proj = PIPE && role >= kXcdRoleProj;
     const int k = is_proj ? role - kXcdRoleProj + 1 : role - 1;  // the chain this group runs or feeds
     const XcdChain& ch = p.chain[k];
     const XcdProj& pj = p.proj[is_proj ? k - 1 : 0];
@@ -199,8 +202,10 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     const int uc = units_ok ? my_unit : H - 1;
     // Lanes 0..31 of wavefronts 0..3 fetch piece 32 w + lane of an h vector: 8 fp16 = columns 8 q .. 8 q + 7.  (The other
     // wavefronts never poll: they are the ones that talk to other XCDs, and a wavefront's loads come back in order.)
-    const int piece = wave * 32 + lane;
-    const bool polls = wave < 4 && lane < 32 && piece * 8 < H;
+    // A group that neither feeds nor is fed across XCDs spreads the polls over all eight wavefronts, 16 lanes each.
+    const bool crosses = PIPE && (is_proj || ch.xproj_polled != 0 || ch.seq_out != nullptr);
+    const int piece = crosses ? wave * 32 + lane : wave * 16 + lane;
+    const bool polls = (crosses ? (wave < 4 && lane < 32) : lane < 16) && piece * 8 < H;
 
     // One bounded wait: `again` loads and tests; gives up like every wait of this kernel.
     auto bounded_wait = [&](auto again) __attribute__((always_inline)) {
@@ -272,8 +277,8 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     // ================= R group: the recurrence of chain k =================
     float c_reg = (float)ch.c0[uc];
     const bool rev = ch.reverse != 0;
-    const bool polled = ch.xproj_polled != 0;
-    const bool feeds = ch.seq_out != nullptr;
+    const bool polled = PIPE && ch.xproj_polled != 0;
+    const bool feeds = PIPE && ch.seq_out != nullptr;
 
     // The input-projection term does not depend on h and must stay off the step's critical path: a wavefront's loads
     // return in order, so a poll issued behind a load that misses the L2 would wait for it.  Each wavefront keeps the
@@ -401,7 +406,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
         for (int i = 0; i < 4; ++i) {
             yw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)hb16, 16 * i) << (16 * i);
             pw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)pb16, 16 * i) << (16 * i);
-            sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
+            if (PIPE) sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
         }
         if (lane == 0) {
             const unsigned int g = g_base + (unsigned int)s;

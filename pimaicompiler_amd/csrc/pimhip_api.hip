@@ -957,8 +957,10 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
     // One recurrence per XCD: the part this is written for has 8 XCDs of 32 CUs, a group is one workgroup per CU of one.
     if (H <= kXcdMaxH && plan->num_cus == kXcdCount * kXcdMembers) {
         int per_cu = 0;
-        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_xcd_f16_kernel, kXcdThreads, 0));
-        plan->xcd_ok = per_cu >= 1;
+        int per_cu_pipe = 0;
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_xcd_f16_kernel<false>, kXcdThreads, 0));
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_pipe, lstm_xcd_f16_kernel<true>, kXcdThreads, 0));
+        plan->xcd_ok = per_cu >= 1 && per_cu_pipe >= 1;
     }
     if (plan->xcd_ok) {
         const size_t words = (size_t)kXcdRegionWords * kXcdMaxChains;
@@ -1227,7 +1229,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             a.H = (int)H;
             a.T = (int)T;
             a.spin_limit = plan->spin_limit;
-            lstm_xcd_f16_kernel<<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+            lstm_xcd_f16_kernel<true><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
             PIMHIP_HIP_CHECK(hipGetLastError());
             layer_in = group_out;
             l += n;
@@ -1271,7 +1273,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             a.H = (int)H;
             a.T = (int)T;
             a.spin_limit = plan->spin_limit;
-            lstm_xcd_f16_kernel<<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+            lstm_xcd_f16_kernel<false><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
             PIMHIP_HIP_CHECK(hipGetLastError());
             layer_in = layer_out;
         }
