@@ -1110,10 +1110,12 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     // launch needs two super-steps).
     // Automatic choice: one recurrence per XCD where its groups have something to run side by side or nothing to gain
     // from a wavefront (the two directions of a layer; a single unidirectional layer), the layer wavefront otherwise.
-    // (Measured on MI355X, whole calls: the per-XCD kernel is 13-30 % faster than the all-CU one for bidirectional layers
-    // from 16 steps on, and 7-17 % for a single unidirectional layer from 16 steps at H <= 512 and from 64 at H = 1024; its
-    // 32 CUs take longer to load the weights, which shorter sequences do not win back.)
-    const bool xcd_pays = (D == 2 && T >= 16) || (D == 1 && L == 1 && T >= (H > 512 ? 64 : 16));
+    // (Measured on MI355X, whole calls against the all-CU kernel: bidirectional layers 13-30 % faster from 16 steps on; a
+    // single unidirectional layer 7-17 % from 16 steps at H <= 512 and from 64 at H = 1024; a unidirectional stack as a
+    // pipeline over the XCDs 6-25 % for two layers from 32 steps, 12-60 % for three and more from 16.  Its 32 CUs per group
+    // take longer to load the weights and the pipeline has to fill, which shorter sequences do not win back.)
+    const bool xcd_pays = (D == 2 && T >= 16) || (D == 1 && L == 1 && T >= (H > 512 ? 64 : 16)) ||
+                          (D == 1 && L >= 2 && T >= (L >= 3 ? 16 : 32));
     const bool use_xcd = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && (plan->mode == 4 || (plan->mode == 0 && xcd_pays));
     const bool use_seq = !use_xcd && T >= 2 && T + kSeqMaxChains <= kSeqMaxT &&
                          (plan->mode == 2 || plan->mode == 3 || (plan->mode == 0 && plan->seq_kernel_ok));

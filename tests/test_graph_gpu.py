@@ -132,8 +132,9 @@ def test_sequence_forward_replays_from_a_graph(ops):
     equals the eager launch bit for bit, with eager launches of the same plan between the replays.  The one thing a
     graph must not record, the re-initialisation of the exchange buffer after a change of mode, is refused."""
     I, Hs = 64, 256
-    # (the last two run one recurrence per XCD: a bidirectional layer of 20 steps in automatic mode, and mode 4 by request)
-    for layers, bidir, T, mode in ((1, True, 20, 0), (1, False, 18, 4), (2, False, 7, 0), (1, True, 7, 0), (1, False, 7, 0)):
+    # (the first three run one recurrence per XCD: a bidirectional layer of 20 steps in automatic mode, mode 4 by request,
+    # and a stack of three layers as a pipeline over the XCDs)
+    for layers, bidir, T, mode in ((1, True, 20, 0), (1, False, 18, 4), (3, False, 21, 0), (2, False, 7, 0), (1, True, 7, 0), (1, False, 7, 0)):
         params, x, h0, c0 = workloads.lstm_inputs(7101 + layers + 2 * bidir + T, I, Hs, layers, bidir, T)
         plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, bidir, T)
         plan.set_mode(mode)

@@ -65,6 +65,9 @@ CASES = [  # I, H, L, bidirectional, T, biases
     # layer 1 of a bidirectional stack at 65 <= T <= 256 with a 2048-wide input: the packed projection with
     # eight wavefronts per block and 32-column tiles
     (64, 1024, 2, True, 70, True),
+    # unidirectional stacks long enough for the pipeline over the XCDs to fill and for its LDS rings to wrap (mode 4 and,
+    # from 32 / 16 steps, automatic mode): two, four (one launch), five and nine layers (two and three launches)
+    (40, 264, 2, False, 45, True), (24, 520, 4, False, 37, False), (16, 72, 5, False, 35, True), (8, 136, 9, False, 18, True),
 ]
 
 
@@ -279,10 +282,12 @@ def test_sequence_kernels_issued_on_two_streams_do_not_starve_each_other(ops):
 
 
 def test_automatic_mode_takes_the_per_xcd_kernel_where_it_pays(ops):
-    """Bidirectional layers from 16 steps on and single unidirectional layers from 64 (16 at H <= 512) run one recurrence
-    per XCD in automatic mode: the same bits as mode 4, which sums in another order than mode 2."""
+    """Bidirectional layers from 16 steps on, single unidirectional layers from 64 (16 at H <= 512) and unidirectional
+    stacks from 32 (16 with three layers and more) run one recurrence per XCD in automatic mode: the same bits as mode 4,
+    which sums in another order than mode 2."""
     for I, H, L, bidir, T, same_as in [(32, 256, 2, True, 40, 4), (32, 1024, 1, False, 70, 4), (32, 1024, 1, False, 20, 2),
-                                        (32, 256, 1, False, 20, 4), (32, 256, 3, False, 40, 2), (32, 256, 1, True, 9, 2)]:
+                                        (32, 256, 1, False, 20, 4), (32, 256, 3, False, 40, 4), (32, 256, 1, True, 9, 2),
+                                        (32, 256, 2, False, 20, 2), (32, 256, 2, False, 33, 4), (32, 256, 3, False, 12, 2)]:
         params, x, h0, c0 = workloads.lstm_inputs(800 + T, I, H, L, bidir, T)
         y0, _, c0n = run_plan(ops, params, x, h0, c0, True, L, bidir, 0)
         ym, _, cmn = run_plan(ops, params, x, h0, c0, True, L, bidir, same_as)
@@ -321,12 +326,13 @@ def test_per_xcd_kernel_finds_its_groups_on_any_queue(ops):
 
 
 # ---- the bounded wait ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("mode", [2, 4])
-def test_persistent_kernel_wait_gives_up_and_reports(ops, mode):
+@pytest.mark.parametrize("mode,layers", [(2, 1), (4, 1), (4, 3)])
+def test_persistent_kernel_wait_gives_up_and_reports(ops, mode, layers):
     """Forced from the host: with a spin limit of 0 every wait gives up at its first unsuccessful poll, the kernel
-    still runs to its end, and the plan reports the time-out.  A later forward with the default limit works."""
-    params, x, h0, c0 = workloads.lstm_inputs(123, 64, 1024, 1, False, 30)
-    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 30)
+    still runs to its end, and the plan reports the time-out.  A later forward with the default limit works.  (Mode 4
+    with three layers: the recurrence groups and the projection groups of the pipeline all give up.)"""
+    params, x, h0, c0 = workloads.lstm_inputs(123, 64, 1024, layers, False, 30)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, False, 30)
     plan.set_mode(mode)
     plan.set_spin_limit(0)
     plan.forward(x.reshape(30, 64).to(DEV), h0.to(DEV), c0.to(DEV))
@@ -335,8 +341,8 @@ def test_persistent_kernel_wait_gives_up_and_reports(ops, mode):
     plan.set_spin_limit(1 << 22)
     y, hn, cn = plan.forward(x.reshape(30, 64).to(DEV), h0.to(DEV), c0.to(DEV))
     plan.status()
-    want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)
-    assert maxabs(y, want[0]) <= 2e-3
+    want = oracle.torch_lstm(x, h0, c0, params, True, layers, False)
+    assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
 
 
 def test_a_timeout_nobody_asked_about_is_raised_by_the_next_call(ops):
@@ -406,6 +412,21 @@ def test_persistent_kernel_survives_a_nan_input(ops, mode):
     want = oracle.torch_lstm(x, h0, c0, params, True, 1, False)[0]
     assert maxabs(y[:7], want[:7]) <= 2e-3
     assert bool(torch.isnan(want[7:]).all()) and bool(torch.isnan(y[7:]).all()) and bool(torch.isnan(cn).all())
+
+
+def test_a_nan_travels_through_the_pipeline_of_layers(ops):
+    """Mode 4 hands h from layer to layer through slots whose "not written yet" mark is the all-ones pattern, itself a NaN:
+    a NaN h is stored there in its canonical form, so it arrives, and nobody waits for a slot that looks empty."""
+    params, x, h0, c0 = workloads.lstm_inputs(6, 64, 256, 3, False, 20)
+    x = x.clone()
+    x[11, 0, 5] = float("nan")
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 3, False, 20)
+    plan.set_mode(4)
+    y, hn, cn = plan.forward(x.reshape(20, 64).to(DEV), h0.to(DEV), c0.to(DEV))
+    plan.status()
+    want = oracle.torch_lstm(x, h0, c0, params, True, 3, False)
+    assert maxabs(y[:11], want[0][:11]) <= 2e-3
+    assert bool(torch.isnan(want[0][11:]).all()) and bool(torch.isnan(y[11:]).all()) and bool(torch.isnan(cn).all())
 
 
 # ---- input projection (the MFMA kernel) against fp32 torch on the host ---------------------------------------------
