@@ -78,6 +78,7 @@ struct XcdProj {
 };
 
 static constexpr int kXcdRoleProj = 9;  // role values: 0 none, 1 + k recurrence of chain k, kXcdRoleProj + j projection j
+static constexpr unsigned long long kXcdWaitTicks = 100000000ull;  // one second of the 100 MHz clock
 static constexpr int kXcdLag = 2;       // steps a recurrence fed by a P group lets that group get ahead before it starts
 
 struct LstmXcdArgs {
@@ -207,13 +208,19 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     const int piece = crosses ? wave * 32 + lane : wave * 16 + lane;
     const bool polls = (crosses ? (wave < 4 && lane < 32) : lane < 16) && piece * 8 < H;
 
-    // One bounded wait: `again` loads and tests; gives up like every wait of this kernel.
+    // One bounded wait: `again` loads and tests; gives up like every wait of this kernel, after spin_limit polls, and
+    // also after kXcdWaitTicks of the constant 100 MHz clock, however long a poll takes in the environment the kernel
+    // finds itself in (a wait that succeeds does so within microseconds).
     auto bounded_wait = [&](auto again) __attribute__((always_inline)) {
         unsigned int spins = 0;
+        unsigned long long t_first = 0ull;
         while (!again() && !gave_up) {
             ++spins;
             if ((spins & 255u) == 0u) {
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
+                const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+                if (spins == 256u) t_first = now;
+                else if (now - t_first > kXcdWaitTicks) spins = 0xffffffffu;  // gives up below
             }
             if (spins >= p.spin_limit) {
                 __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
