@@ -528,6 +528,8 @@ class LstmPlan:
             pass
 
     def set_mode(self, mode):
+        """0 automatic, 1 one launch per step, 2 / 3 the persistent kernel over all CUs (3: four units per block always),
+        4 one recurrence per XCD (pimhip_lstm_plan_set_mode)."""
         _check(L.load().pimhip_lstm_plan_set_mode(self._handle, mode))
 
     def set_spin_limit(self, limit):
