@@ -42,6 +42,8 @@
 // 8-byte store of the wavefront's four new h values into the workgroup's entry.
 #pragma once
 
+#include <type_traits>
+
 #include "lstm_kernels.h"
 
 namespace pimhip
@@ -282,10 +284,13 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     }
 
     // ================= R group: the recurrence of chain k =================
+    // Compiled once per combination of "its projection rows arrive during the launch" and "its h goes to a layer above":
+    // a step is sensitive to every instruction on its path, and the plain combination should not carry the others'.
+    auto recurrence = [&](auto polled_c, auto feeds_c) __attribute__((always_inline)) {
+    constexpr bool polled = decltype(polled_c)::value;
+    constexpr bool feeds = decltype(feeds_c)::value;
     float c_reg = (float)ch.c0[uc];
     const bool rev = ch.reverse != 0;
-    const bool polled = PIPE && ch.xproj_polled != 0;
-    const bool feeds = PIPE && ch.seq_out != nullptr;
 
     // The input-projection term does not depend on h and must stay off the step's critical path: a wavefront's loads
     // return in order, so a poll issued behind a load that misses the L2 would wait for it.  Each wavefront keeps the
@@ -413,7 +418,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
         for (int i = 0; i < 4; ++i) {
             yw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)hb16, 16 * i) << (16 * i);
             pw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)pb16, 16 * i) << (16 * i);
-            if (PIPE) sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
+            if (feeds) sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
         }
         if (lane == 0) {
             const unsigned int g = g_base + (unsigned int)s;
@@ -436,6 +441,13 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
             store16_device_scope(ch.seq_out + (long)(T - 1) * H + rank * kXcdUnitsPerBlock + lane * 8, src[0], src[1]);
         }
     }
+    };
+    const bool polled_rt = PIPE && ch.xproj_polled != 0;
+    const bool feeds_rt = PIPE && ch.seq_out != nullptr;
+    if (!PIPE || (!polled_rt && !feeds_rt)) recurrence(std::false_type{}, std::false_type{});
+    else if (!polled_rt) recurrence(std::false_type{}, std::true_type{});
+    else if (!feeds_rt) recurrence(std::true_type{}, std::false_type{});
+    else recurrence(std::true_type{}, std::true_type{});
     // Rank 0 has finished its last step, for which (T >= 2) it needed what every member published one step earlier:
     // every member has read the counter by now.
     if (rank == 0 && tid == 0)
