@@ -349,8 +349,14 @@ def main():
             lib.pimhip_lstm_forward(plan_d._handle, xd1.data_ptr(), h0d.data_ptr(), c0d.data_ptr(), yd1.data_ptr(),
                                     hnd.data_ptr(), cnd.data_ptr(), 1, s_h)
         us = graph_timed_us(decode_launch, 32)
+        # the floor beside it: a launch that only reads as many (warm) bytes as the step's two weight matrices
+        probe_buf = torch.empty(2 * 4096 * 1024, dtype=torch.float16, device=dev).normal_()
+
+        def decode_floor(s_h=sh):
+            lib.pimhip_probe_stream_read(probe_buf.data_ptr(), probe_buf.numel() * 2, s_h)
         other["lstm_decode_step"] = {"us": round(us, 3), "gbs": round((2 * 4096 * 2048 + 8 * 4096) / us / 1e3, 1),
-                                     "issued_from_python_us": round(timed_us(decode_launch, 200), 3)}
+                                     "issued_from_python_us": round(timed_us(decode_launch, 200), 3),
+                                     "read_only_kernel_us": round(graph_timed_us(decode_floor, 32), 3)}
         # the same sweep as ONE grouped launch (executeMultiStream's siblings in one grid), cold
         def grouped():
             ws = []

@@ -54,6 +54,7 @@ class LayerType(enum.Enum):
     ATENLSTM2 = "aten::lstm2"
     ATENMATMUL = "aten::matmul"
     MULTISTREAM = "multi_stream"
+    DECODERSTEP = "pimhip::decoder_step"    # no counterpart in ir/include/types.h: see DecoderStepLayer
 
 
 class DataType(enum.Enum):
@@ -142,6 +143,25 @@ class AtenBmmLayer(NNLayer):            # ir/include/layers/aten_bmm_layer.h
 
 
 @dataclass
+class DecoderStepLayer(NNLayer):
+    """No counterpart in the reference's IR: the per-token chain of its GNMT decoder, which its interpreter runs as
+    separate layers (executeAtenLSTM1 per cell with the state in the buffer blob, executeAtenBmm for the context,
+    executeAtenAdd for the residual sums, executeAtenAddmm for the classifier), as ONE record that runs as one launch.
+
+    cells: the AtenLSTM1Layer records of the chain, bottom to top, as the model builder leaves them (param_vector set,
+    custom_opt_number = k and custom_cat_mem_id = the state buffer blob: rows 2k, 2k+1 hold (h, c) of cell k and are
+    updated in place).  in_stensor_ids: [x, attention weights, encoder outputs], or [x, context] when the context is
+    computed elsewhere.  out_stensor_ids: one id per cell for its output (y, or y + input from first_residual_layer on),
+    then the id of the logits when classifier ids are given.  The encoder outputs are projected once per sentence: set
+    StreamExecutor.same_sentence while the blob keeps the sentence it had at the previous token."""
+    cells: List[AtenLSTM1Layer] = field(default_factory=list)
+    first_takes_context: bool = False
+    first_residual_layer: int = 2
+    classifier_weight_id: int = -1      # blob ids of W [vocab, H] and b [vocab] (or -1)
+    classifier_bias_id: int = -1
+
+
+@dataclass
 class MultiStreamLayer(NNLayer):        # ir/include/layers/multi_stream_layer.h
     layers: List[NNLayer] = field(default_factory=list)
 
@@ -162,6 +182,9 @@ class StreamExecutor:
         self.streams: List[torch.cuda.Stream] = []
         # True: sibling GEMVs of a MULTISTREAM layer go out as one grouped launch instead of one stream each.
         self.grouped_multi_stream = grouped_multi_stream
+        # True while the encoder outputs a DecoderStepLayer attends over are those of its previous call (their projection
+        # is then not computed again); a driver sets it after the first token of a sentence and clears it for the next one.
+        self.same_sentence = False
         ops.initialize(device)
         width = max([l.layer_num for l in self.layers if isinstance(l, MultiStreamLayer)], default=0)
         self.set_streams(width)
@@ -554,8 +577,56 @@ def execute_aten_bmm(layer, executor):
     executor.update_blob(layer.out_stensor_ids[0], DataType.TENSOR, out)
 
 
+def execute_decoder_step(layer, executor):
+    """One decoder token as one launch (ops.DecoderPlan / pimhip_decoder_step).  The plan is made on the first call and kept
+    on the record; the cells' states are read from and written to their rows of the state buffer blob."""
+    cells = layer.cells
+    n = len(cells)
+    if n < 1 or any(len(c.param_vector) != 4 for c in cells):
+        raise NNRuntimeException("a decoder step needs its cells' parameter vectors (w_ih, w_hh, b_ih, b_hh per cell)")
+    ids = layer.in_stensor_ids
+    x = _tensor(executor, ids[0], "decoder step input")
+    H = cells[0].param_vector[1].size(1)
+    plan = getattr(layer, "_plan", None)
+    if plan is None:
+        cls = None
+        if layer.classifier_weight_id >= 0:
+            cls = (_tensor(executor, layer.classifier_weight_id, "classifier weight"),
+                   _tensor(executor, layer.classifier_bias_id, "classifier bias") if layer.classifier_bias_id >= 0 else None)
+        plan = ops.DecoderPlan([t for c in cells for t in c.param_vector], True, n, first_takes_context=layer.first_takes_context,
+                               first_residual_layer=layer.first_residual_layer, classifier=cls)
+        layer._plan = plan
+    att = enc = ctx = None
+    if len(ids) >= 3:
+        att, enc = _tensor(executor, ids[1], "attention weights"), _tensor(executor, ids[2], "encoder outputs")
+        if not (getattr(executor, "same_sentence", False) and plan._enc is not None):
+            plan.set_encoder(enc.reshape(-1, H).contiguous())
+    elif len(ids) == 2:
+        ctx = _tensor(executor, ids[1], "context")
+    h_prev, c_prev = [], []
+    for c in cells:
+        state = _tensor(executor, c.custom_cat_mem_id, "decoder state buffer")
+        k = c.custom_opt_number
+        if not state.is_contiguous() or state.numel() < (2 * k + 2) * H:
+            raise NNRuntimeException(f"blob {c.custom_cat_mem_id} cannot hold the state of decoder cell {k}")
+        flat = state.view(-1)
+        h_prev.append(flat[2 * k * H:(2 * k + 1) * H])
+        c_prev.append(flat[(2 * k + 1) * H:(2 * k + 2) * H])
+    outs = [torch.empty(1, 1, H, dtype=torch.float16, device=x.device) for _ in range(n)]
+    logits = torch.empty(1, plan.vocab, dtype=torch.float16, device=x.device) if plan.vocab else None
+    flat1 = lambda t: t.contiguous().view(-1)  # noqa: E731
+    step = plan.bind(flat1(x), h_prev, c_prev, att=flat1(att) if att is not None else None, ctx=flat1(ctx) if ctx is not None else None,
+                     outs=[o.view(-1) for o in outs], logits=logits.view(-1) if logits is not None else None)   # state in place
+    step()
+    for k in range(n):
+        executor.update_blob(layer.out_stensor_ids[k], DataType.TENSOR, outs[k])
+    if logits is not None:
+        executor.update_blob(layer.out_stensor_ids[n], DataType.TENSOR, logits)
+
+
 # registerOp (stream_executor.cpp:433-576) for the layer types of this path
 OP_EXECUTORS = {
+    LayerType.DECODERSTEP: execute_decoder_step,
     LayerType.ATENADD: execute_aten_add,
     LayerType.ATENADDMM: execute_aten_addmm,
     LayerType.ATENBMM: execute_aten_bmm,

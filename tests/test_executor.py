@@ -475,6 +475,51 @@ def test_gnmt_decoder_steps_write_into_the_state_and_attention_buffers(ops):
 
 
 @pytest.mark.gpu
+def test_decoder_step_record_runs_the_token_as_one_launch(ops):
+    """The same four cells as one DecoderStepLayer (layers 1..3 on cat(previous output, context), residual sums from layer
+    2 on, the classifier): three tokens of two sentences through the dispatch loop, state updated in place in the state
+    buffer blob, against LibTorch CPU running the chain operator by operator."""
+    H, S, V = 256, 11, 300
+    g = torch.Generator().manual_seed(41)
+    params = [workloads.lstm_inputs(60 + k, H if k == 0 else 2 * H, H, 1, False, 1)[0] for k in range(4)]
+    Wc, bc = (0.05 * torch.randn(V, H, generator=g)).half(), (0.01 * torch.randn(V, generator=g)).half()
+    state = (0.2 * torch.randn(8, 1, H, generator=g)).half()
+    cells = [E.AtenLSTM1Layer(LayerType.ATENLSTM1, k, [], [], has_biases=1, num_layers=1, dropout=0.0, train=0, bidirectional=0,
+                              batch_first=0, param_vector=[p.to(DEV) for p in params[k]], match_custom_opt=True,
+                              custom_opt_number=k, custom_cat_mem_id=100) for k in range(4)]
+    layer = E.DecoderStepLayer(LayerType.DECODERSTEP, 0, [1, 2, 3], [30, 31, 32, 33, 40], cells=cells, first_takes_context=False,
+                               first_residual_layer=2, classifier_weight_id=50, classifier_bias_id=51)
+    ex = E.StreamExecutor([layer], model_type="GNMT", device=0)
+    state_d = state.to(DEV)
+    _blobs(ex, b100=state_d, b50=Wc.to(DEV), b51=bc.to(DEV))
+    ref = state.clone()
+    enc_buf = torch.zeros(1, S, H, dtype=torch.float16, device=DEV)     # the same blob is refilled for the next sentence
+    ex.update_blob(3, DataType.TENSOR, enc_buf)
+    for sentence in range(2):
+        enc = torch.randn(1, S, H, generator=g).half()
+        enc_buf.copy_(enc.to(DEV))
+        ex.same_sentence = False
+        for token in range(3):
+            x = torch.randn(1, 1, H, generator=g).half()
+            att = torch.softmax(torch.randn(1, 1, S, generator=g), -1).half()
+            _blobs(ex, b1=x.to(DEV), b2=att.to(DEV))
+            ex.inference()
+            ex.same_sentence = True
+            ctx = torch.bmm(att.float(), enc.float()).half()
+            inp = x
+            for k in range(4):
+                full = inp if k == 0 else torch.cat([inp, ctx], 2)
+                y, hn, cn = torch.lstm(full, (ref[2 * k:2 * k + 1], ref[2 * k + 1:2 * k + 2]), params[k], True, 1, 0.0, False, False, False)
+                ref[2 * k], ref[2 * k + 1] = hn[0], cn[0]
+                inp = y + inp if k >= 2 else y
+                assert maxabs(ex.find_blob(30 + k)[1], inp) <= TOL_LSTM, (sentence, token, k)
+            logits = torch.addmm(bc, inp.view(1, H), Wc.t())
+            got = ex.find_blob(40)[1]
+            assert list(got.shape) == [1, V] and maxabs(got, logits) <= TOL_LSTM
+            assert maxabs(state_d, ref) <= TOL_LSTM
+
+
+@pytest.mark.gpu
 def test_gnmt_attention_context_lands_in_three_concatenation_buffers(ops):
     """aten_ops_executor.cpp:680-737: y[1,1,1024] = p[1,1,50] . enc[1,50,1024] at offset 1024 of three buffers."""
     g = torch.Generator().manual_seed(8)
