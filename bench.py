@@ -50,6 +50,9 @@ def main():
                     help="comma list of what to run: sweep (the timed steps, always run), lstm (LSTM and input projection "
                          "figures), other (the other kernels of the path), decoder (the one-launch decoder step alone, "
                          "issued eagerly; not in the default set); counter runs use one of sweep, lstm, decoder at a time")
+    ap.add_argument("--lstm-modes", default="",
+                    help="comma list of LSTM plan modes to time in the lstm section (0 automatic, 4 per-XCD, 2 all-CU wavefront, "
+                         "1 per-step launches); default: all four, under a counter run 2 and 1 only")
     args = ap.parse_args()
     sections = set(args.sections.split(","))
 
@@ -194,10 +197,13 @@ def main():
     # 1 are forced beside it: the same pipeline, the two layers as a wavefront over all CUs, one launch per step
     lstm = {"automatic": None, "per_xcd_pipeline": None, "all_cu_wavefront": None, "per_step_launches": None}
     lstm_modes = ((0, "automatic"), (4, "per_xcd_pipeline"), (2, "all_cu_wavefront"), (1, "per_step_launches"))
-    if counter_run:
+    if args.lstm_modes:
+        wanted = [int(m) for m in args.lstm_modes.split(",")]
+        lstm_modes = tuple(mn for mn in lstm_modes if mn[0] in wanted)
+    elif counter_run:
         # The per-XCD kernel keeps groups of workgroups on particular XCDs waiting for one another; a counter run of it
         # stopped making progress (the all-CU kernel and the per-step kernel have been collected under --pmc), so under
-        # counters only those two run.
+        # counters only those two run unless --lstm-modes asks otherwise.
         lstm_modes = ((2, "all_cu_wavefront"), (1, "per_step_launches"))
         progress("counter run detected: the per-XCD LSTM modes are left out")
     for mode, name in lstm_modes if "lstm" in sections else ():
