@@ -59,9 +59,10 @@ def main():
     def progress(msg):
         print(f"[bench] {msg}", file=sys.stderr, flush=True)
     # Under rocprofv3 --pmc (it exports ROCPROF_COUNTER_COLLECTION) every dispatch is serialised and bracketed by counter
-    # reads.  The `other` section captures and replays HIP graphs and issues kernels that wait for each other's partial
-    # results back to back; the one counter run that included it stopped making progress.  Counter runs therefore never
-    # run that section (the sweep and the LSTM section have been collected under --pmc and are all the counters serve).
+    # reads.  Counter runs that dispatched kernels whose workgroups wait for one another (the persistent LSTM kernels, the
+    # sliced I_X_W reducers) or replayed HIP graphs have now and then stopped making progress.  A counter run therefore never
+    # runs the `other` section, runs the per-XCD LSTM modes only on request, and bounds every LSTM wait tightly; the
+    # sweep, the LSTM section and the decoder section have all been collected under --pmc this way.
     counter_run = bool(os.environ.get("ROCPROF_COUNTER_COLLECTION"))
     if counter_run and "other" in sections:
         sections.discard("other")
