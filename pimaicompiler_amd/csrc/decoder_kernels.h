@@ -132,6 +132,19 @@ __device__ __forceinline__ unsigned int readlane_u32(unsigned int v, int l)
 // L = p.n_layers and CLS = "there is a classifier" are template parameters so that the order of loads and uses is fixed
 // at compile time: the lifetime of every register, and the number of later loads that may still be in flight when an
 // earlier one is waited for (a load issued under a run-time condition would make every such wait a wait for all).
+// How many groups of classifier rows (four rows per streaming wavefront each; a wavefront's registers hold four groups)
+// are asked for right after layer k's output has been stored.  One group stands in front of each exchange's polls: the
+// 16 MB stream while the output travels.  (Measured on MI355X, four layers, 32000 rows: {1, 1, 1, 1} 26.7 us per step;
+// {2, 0, 0, 2} 30.3 us; {0, 2, 0, 2} 30.3 us; {0, 1, 1, 2} 27.3 us; {0, 1, 2, 1} 27.3 us; {1, 1, 2, 0} 31.0 us.)
+template <int L>
+__device__ constexpr int cls_groups_after(int k)
+{
+    if (k + 1 == L) return 4;  // whatever is left
+    if (L == 2) return 2;
+    if (L == 3) return k == 0 ? 1 : 2;
+    return k <= 2 ? 1 : 0;
+}
+
 template <int L, bool CLS>
 __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderStepArgs p)
 {
@@ -268,6 +281,18 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
         // Layer 0 waits for nothing but its own weights: its h_prev comes straight from memory, ahead of them.
         const half8_t hv0 = active ? reinterpret_cast<const half8_t*>(p.layer[0].h_prev)[chunk] : zero8;
         issue_a(0);
+        // the bias of this wavefront's first sixteen classifier rows, long before the end of the step needs it
+        // (every lane loads, from a clamped row: a load under a run-time condition would blur the count of loads in flight)
+        float cls_bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (has_cls) {
+            const half_t* bias_src = p.cls_b ? p.cls_b : p.cls_w;
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const long row = min(cls_row0(it) + gate_of_slot[lane & 3], (long)V - 1);
+                const float b = (float)bias_src[row];
+                cls_bias[it] = p.cls_b ? b : 0.0f;
+            }
+        }
         DEC_TRACE(1);
         if (staged_ctx_first) __syncthreads();  // B0: a given context is in LDS (a first layer that takes it)
         DEC_TRACE(2);
@@ -289,18 +314,18 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
             }
         }
         deliver(0);
+        // B2: the block's output is on its way before anything else is asked for.  A store, and the polls behind it, wait in
+        // the CU's memory pipeline for every load issued before them; without this barrier layer 0's output left some
+        // blocks 5 us late (behind 24 MB of the later layers' rows) and every block waited for it.
+        if (L > 1 || has_cls) __syncthreads();
         // everything else that needs no other layer goes out now and is consumed as it arrives, while layer 0's output travels
 #pragma unroll
         for (int k = 1; k < L; ++k) issue_a(k);
         // (after B1 of layer 0: every later layer's h_prev and a given context are in LDS)
         if (p.ctx_in && active) cvec = *reinterpret_cast<const half8_t*>(&ctx_vec[chunk * 8]);
         auto hv_of = [&](int k) { return active ? *reinterpret_cast<const half8_t*>(&hprev[k][chunk * 8]) : zero8; };
-        // The registers freed by each consumed group take the next loads: D(1..), then classifier rows.  A wavefront's first
-        // four groups of classifier rows go out at fixed points: kPre of them behind the layers' weights, then kPer after
-        // each later layer's gate sums, the rest after the last layer.  (Measured on MI355X with four layers and 32000
-        // rows: 2 / 0 is fastest, 31.6 us per step; groups issued during the later layers' exchanges stand in front of
-        // the polls in the CU's memory pipeline and lengthen each exchange by what they save afterwards: 32.6 to 36.8 us.)
-        constexpr int kPre = 2, kPer = 0;
+        // The registers freed by each consumed group take the next loads: D(1..), then classifier rows, of which a
+        // wavefront's first four groups go out at fixed points (cls_groups_after).
         int cls_next = 0;  // (a compile-time value at every use: the code below is straight-line in L)
         auto cls_prefetch = [&](int n) __attribute__((always_inline)) {
 #pragma unroll
@@ -324,7 +349,7 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
             if (L >= 4) issue_d(3);
         }
         if (L >= 4) consume_a(3, cvec, hv_of(3));
-        cls_prefetch(L == 1 ? 4 : kPre);
+        cls_prefetch(cls_groups_after<L>(0));
         if (L > 1 || has_cls) {
             __syncthreads();  // B3 of layer 0: its whole output (the next input) is in LDS
             DEC_TRACE(10);
@@ -335,7 +360,9 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
 #pragma unroll
             for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_in[k][v], pv, acc[k][v]);
             deliver(k);
-            cls_prefetch(k + 1 == L ? 4 : kPer);
+            // B2 again, then the next classifier rows: they stream while this layer's output travels
+            if (has_cls && cls_groups_after<L>(k) > 0) __syncthreads();
+            cls_prefetch(cls_groups_after<L>(k));
             if (k + 1 < L || has_cls) {
                 __syncthreads();  // B3: the layer's whole output (the next input) is in LDS
                 DEC_TRACE(10 + 4 * k);
@@ -347,7 +374,7 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
             half8_t vv[CH];
 #pragma unroll
             for (int c = 0; c < CH; ++c) vv[c] = (c * 64 + lane < nchunks) ? *reinterpret_cast<const half8_t*>(&in_vec[(c * 64 + lane) * 8]) : zero8;
-            auto cls_finish = [&](const half8_t (&src)[4][CH], int it) __attribute__((always_inline)) {
+            auto cls_finish = [&](const half8_t (&src)[4][CH], int it, float bias, bool bias_given) __attribute__((always_inline)) {
                 const long r0 = cls_row0(it);
                 float s[4];
 #pragma unroll
@@ -360,21 +387,21 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                 if (lane < 4) {
                     const long row = r0 + gate_of_slot[lane];  // lane l holds slot {0, 2, 1, 3}[l]
                     if (row < V) {
-                        float r = tot;
-                        if (p.cls_b) r += (float)p.cls_b[row];
+                        float r = tot + bias;
+                        if (!bias_given && p.cls_b) r += (float)p.cls_b[row];
                         p.logits[row] = (half_t)r;
                     }
                 }
             };
-            cls_finish(cbuf[0], 0);
-            cls_finish(cbuf[1], 1);
-            cls_finish(cbuf[2], 2);
-            cls_finish(cbuf[3], 3);
+            cls_finish(cbuf[0], 0, cls_bias[0], true);
+            cls_finish(cbuf[1], 1, cls_bias[1], true);
+            cls_finish(cbuf[2], 2, cls_bias[2], true);
+            cls_finish(cbuf[3], 3, cls_bias[3], true);
             for (int it = 4; cls_row0(it) < V; it += 2) {  // vocabularies beyond 16 rows per wavefront: two groups at a time
                 cls_issue(cbuf[0], it);
                 cls_issue(cbuf[1], it + 1);
-                cls_finish(cbuf[0], it);
-                cls_finish(cbuf[1], it + 1);
+                cls_finish(cbuf[0], it, 0.0f, false);
+                cls_finish(cbuf[1], it + 1, 0.0f, false);
             }
         }
         DEC_TRACE(25);
@@ -500,6 +527,7 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                         __hip_atomic_store(slot + (long)blockIdx.x * (kDecEntryWords / 2), word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
+            if (k == 0 ? (L > 1 || has_cls) : (has_cls && cls_groups_after<L>(k) > 0)) __syncthreads();  // B2: this block's output has been stored
             if (exchange) {
                 const unsigned long long* slot = reinterpret_cast<const unsigned long long*>(p.hx + ((long)k * nb) * kDecEntryWords);
                 const unsigned long long want = flag ? 0x4000400040004000ull : 0ull;
