@@ -33,9 +33,10 @@
 //     applies the gates (lanes 4u .. 4u+3 = the gates of unit u), stores the state and publishes the block's four
 //     outputs with one 8-byte store; all of them poll the other blocks' entries and put the layer's whole output into
 //     LDS for the streamers.
-// Two barriers per layer: gate sums ready, next input ready.  (All wavefronts of a CU share its path to memory, and a
-// load is served after every load issued before it: polls that are issued while weights are still queued are slow.  So
-// the layers' chain after layer 0 runs with the weights already in registers and little else in flight.)
+// Three barriers per layer: gate sums ready (B1), the block's output stored (B2), next input ready (B3).  All wavefronts
+// of a CU share its path to memory, and a request is served after every request issued before it: a store or a poll
+// issued while weights are still queued is slow.  B2 lets the store and the first polls go out in front; what the
+// streaming wavefronts ask for after it (one group of classifier rows per layer) streams while the output travels.
 //
 // Exchange: hx[stage][NB] entries of 64 bytes: a block's four fp16 outputs of layer `stage` in the first 8 bytes.
 // |y| <= 1, so bit 14 of each fp16 carries a flag, the parity of the launch count g (a device word read at the start and
