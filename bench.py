@@ -343,6 +343,17 @@ def main():
                 cur, _, _ = plan_g.forward(cur, hg, cg)
 
         other["gnmt_lstm_stack_us_per_layer_step"] = round(timed_us(gnmt_stack, 30) / 250, 3)
+        # the same stack after rewrite.fuse_lstm_stack: the three one-direction layers as ONE aten::lstm with num_layers = 3
+        # (a pipeline over the XCDs in one launch), behind the bidirectional layer's call
+        plan_123 = P.LstmPlan([q for pl, _, _ in gn[1:] for q in pl.params], True, 3, False, 50)
+        h_123 = torch.cat([hg for _, hg, _ in gn[1:]], 0).contiguous()
+        c_123 = torch.cat([cg for _, _, cg in gn[1:]], 0).contiguous()
+
+        def gnmt_stack_two_calls():
+            cur, _, _ = gn[0][0].forward(seq, gn[0][1], gn[0][2])
+            plan_123.forward(cur, h_123, c_123)
+
+        other["gnmt_lstm_stack_us_per_layer_step_layers_1_to_3_as_one_call"] = round(timed_us(gnmt_stack_two_calls, 30) / 250, 3)
         # the same four calls (eight launches) replayed from a HIP graph
         other["gnmt_lstm_stack_us_per_layer_step_hip_graph"] = round(graph_timed_us(lambda _s: gnmt_stack(), 1) / 250, 3)
         # one decoder step (seq_len 1, I = H = 1024): the fused step kernel, W_ih and W_hh streamed once (16.8 MB)

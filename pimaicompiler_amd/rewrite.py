@@ -26,6 +26,12 @@ and the classifier — which the reference's interpreter runs operator by operat
 executeAtenAdd / executeAtenAddmm, runtime/source/executor/op_executor/aten_ops_executor.cpp:2135-2307, 668-747, 43-179,
 181-216), into one `pimhip::decoder_step` op, which `execute` runs as ONE launch (ops.DecoderPlan).
 
+`fuse_lstm_stack` has no counterpart either: consecutive one-layer `aten::lstm` ops over a whole sequence, each reading
+only the sequence the one before wrote (the GNMT encoder's layers above the bidirectional one, which the reference runs
+as one executeAtenLSTM1 call each), become ONE `aten::lstm` with `num_layers = n`, LibTorch's own multi-layer form, so
+that the layers run as a pipeline in one launch (layer k starts step t as soon as layer k - 1 has finished it) instead
+of one after the other.
+
 remove_cat_for_addmm is restated for any split point; the reference hard-codes the RNNT joint shapes
 ([1,1024] + [1,320] against a [512,1344] weight, compiler/include/frontend/optimizer/remove_cat_for_addmm.h:77-79).
 """
@@ -421,6 +427,98 @@ def fuse_decoder_step(g: Graph):
     return g
 
 
+# ---- consecutive sequence layers into one multi-layer op -------------------------------------------------------------
+def _sequence_layer(g: Graph, op: Op):
+    """A one-layer, one-direction aten::lstm over a padded sequence with constant fp16 weights and biases (seq_len-1 cells
+    are fuse_decoder_step's)."""
+    if op.type != "aten::lstm" or len(op.inputs) != 7 or len(op.outputs) != 3:
+        return False
+    a = op.attrs
+    if a.get("num_layers", 1) != 1 or a.get("bidirectional", False) or not a.get("has_biases", True) or a.get("batch_first", False):
+        return False
+    if a.get("seq_len", 0) == 1:
+        return False
+    if not all(g.is_constant(t) and g.constants[t] is not None for t in op.inputs[3:7]):
+        return False
+    w_ih, w_hh = g.constants[op.inputs[3]], g.constants[op.inputs[4]]
+    return (w_ih.dtype == torch.float16 and w_hh.dtype == torch.float16 and w_ih.dim() == 2 and w_hh.dim() == 2 and
+            w_hh.size(0) == 4 * w_hh.size(1) and w_ih.size(0) == w_hh.size(0))
+
+
+def fuse_lstm_stack(g: Graph):
+    """lstm_a(x, h0_a, c0_a) -> lstm_b(y_a, h0_b, c0_b) -> ...  becomes  lstm(x, cat(h0_a, h0_b, ..), cat(c0_a, c0_b, ..))
+    with num_layers = n and the parameters of the layers in order, placed where the chain's last op was.  The stacked
+    hn / cn are sliced back into the tensors the single ops produced, for whoever reads them.
+
+    A layer joins the chain when it is the only reader of the sequence before it, that sequence is not a graph output,
+    its input width is the hidden size of the layer before (as in a multi-layer aten::lstm) and its hidden size is the
+    same.  Left alone: layers with a residual sum around them (their input has a second reader), layers whose initial
+    state is computed from the chain itself, chains whose intermediate hn / cn are read before the chain's end."""
+    taken = set()
+    for first in list(g.ops):
+        if id(first) in taken or all(first is not o for o in g.ops) or not _sequence_layer(g, first):
+            continue
+        chain = [first]
+        while True:
+            last = chain[-1]
+            y = last.outputs[0]
+            users = g.consumers(y)
+            if len(users) != 1 or y in g.outputs or users[0].inputs.count(y) != 1 or users[0].inputs[0] != y:
+                break
+            nxt = users[0]
+            H = g.constants[last.inputs[4]].size(1)
+            if not _sequence_layer(g, nxt) or g.constants[nxt.inputs[4]].size(1) != H or g.constants[nxt.inputs[3]].size(1) != H:
+                break
+            if any(_depends_on(g, t, chain) for t in nxt.inputs[1:3]):
+                break
+            if nxt.attrs.get("seq_len", 0) != last.attrs.get("seq_len", 0):
+                break
+            chain.append(nxt)
+        # the intermediate hn / cn must not be read before the place the fused op takes (the last op's)
+        while len(chain) >= 2:
+            end = next(i for i, o in enumerate(g.ops) if o is chain[-1])
+            early = False
+            for o in chain[:-1]:
+                for t in o.outputs[1:3]:
+                    for user in g.consumers(t):
+                        if next(i for i, q in enumerate(g.ops) if q is user) < end:
+                            early = True
+            if not early:
+                break
+            chain.pop()
+        if len(chain) < 2:
+            continue
+        n = len(chain)
+        state = []
+        pre = []
+        for slot in (1, 2):
+            ids = [o.inputs[slot] for o in chain]
+            if all(g.is_constant(t) and g.constants[t] is not None for t in ids):
+                tid = g.new_id()
+                g.constants[tid] = torch.cat([g.constants[t].reshape(1, 1, -1) for t in ids], 0)
+            else:
+                lst, tid = g.new_id(), None
+                pre.append(Op("prim::ListConstruct", ids, [lst]))
+                tid = g.new_id()
+                pre.append(Op("aten::cat", [lst], [tid], {"dim": 0}))
+            state.append(tid)
+        hn_all, cn_all = g.new_id(), g.new_id()
+        params = [t for o in chain for t in o.inputs[3:7]]
+        attrs = dict(chain[0].attrs)
+        attrs["num_layers"] = n
+        fused = Op("aten::lstm", [chain[0].inputs[0]] + state + params, [chain[-1].outputs[0], hn_all, cn_all], attrs)
+        post = []
+        for k, o in enumerate(chain):
+            for t, src in ((o.outputs[1], hn_all), (o.outputs[2], cn_all)):
+                if g.consumers(t) or t in g.outputs:
+                    post.append(Op("aten::slice", [src], [t], {"dim": 0, "start": k, "end": k + 1}))
+        end = next(i for i, o in enumerate(g.ops) if o is chain[-1])
+        g.ops[end:end + 1] = pre + [fused] + post
+        g.ops = [o for o in g.ops if all(o is not c for c in chain)]
+        taken.update(id(o) for o in chain)
+    return g
+
+
 def _as_row_major_weight(t):
     """For a [..1.., in, out] tensor that is a transposed view of a dense row-major [out, in] matrix: that matrix."""
     if t.dim() < 2 or any(d != 1 for d in t.shape[:-2]) or t.dtype != torch.float16:
@@ -524,7 +622,10 @@ def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0", same_sent
             _run_decoder_step(op, env, ops, same_sentence)
             continue
         elif op.type == "aten::lstm":
-            y, hn, cn = ops.aten_lstm1(a[0], (a[1], a[2]), a[3:7], True, 1, 0.0, False, False, False)
+            n = op.attrs.get("num_layers", 1)
+            bidir = bool(op.attrs.get("bidirectional", False))
+            y, hn, cn = ops.aten_lstm1(a[0], (a[1], a[2]), a[3:3 + 4 * n * (2 if bidir else 1)], True, n, 0.0, False, bidir,
+                                       bool(op.attrs.get("batch_first", False)))
             env[op.outputs[0]], env[op.outputs[1]], env[op.outputs[2]] = y, hn, cn
             continue
         elif op.type == "aten::bmm":

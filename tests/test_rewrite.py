@@ -329,3 +329,115 @@ def test_fused_decoder_graph_matches_the_operator_list_and_libtorch(ops, query_f
     logits = torch.nn.functional.linear(r3.float(), c[200].float(), c[201].float())
     for a, b in zip(got, [logits, hn0, hn1, hn2, hn3, cn0, cn1, cn2, cn3]):
         assert float((a - b.float()).abs().max()) <= 5e-3
+
+
+# ---- consecutive sequence layers into one multi-layer op --------------------------------------------------------------
+def encoder_graph(seed=21, H=128, T=12, residual_last=False, constant_state=False):
+    """The GNMT encoder as the interpreter sees it: a bidirectional layer, then three one-direction layers, each an
+    aten::lstm of its own reading the sequence before it (the first of them 2H wide); optionally a residual sum around
+    the last one."""
+    from pimaicompiler_amd import workloads
+    g = torch.Generator().manual_seed(seed)
+    c, ops, feeds = {}, [], {}
+    X = 0
+    p0 = workloads.lstm_inputs(seed + 10, H, H, 1, True, T)[0]
+    for j, t in enumerate(p0):
+        c[100 + j] = t
+    ops.append(R.Op("aten::lstm", [X, 10, 20] + [100 + j for j in range(8)], [300, 310, 320], {"bidirectional": True, "seq_len": T}))
+    prev = 300
+    for k in range(1, 4):
+        prm = workloads.lstm_inputs(seed + 10 + k, 2 * H if k == 1 else H, H, 1, False, T)[0]
+        for j, t in enumerate(prm):
+            c[100 + 8 * k + j] = t
+        ops.append(R.Op("aten::lstm", [prev, 10 + k, 20 + k] + [100 + 8 * k + j for j in range(4)], [300 + k, 310 + k, 320 + k], {"seq_len": T}))
+        if k == 3 and residual_last:
+            ops.append(R.Op("aten::add", [303, prev], [353]))
+            prev = 353
+        else:
+            prev = 300 + k
+    feeds[X] = torch.randn(T, 1, H, generator=g).half()
+    feeds[10], feeds[20] = (0.3 * torch.randn(2, 1, H, generator=g)).half(), (0.3 * torch.randn(2, 1, H, generator=g)).half()
+    inputs = [X, 10, 20]
+    for k in range(1, 4):
+        h, cc = (0.3 * torch.randn(1, 1, H, generator=g)).half(), (0.3 * torch.randn(1, 1, H, generator=g)).half()
+        if constant_state:
+            c[10 + k], c[20 + k] = h, cc
+        else:
+            feeds[10 + k], feeds[20 + k] = h, cc
+            inputs += [10 + k, 20 + k]
+    outputs = [prev, 312, 322, 313]
+    return R.Graph(ops, inputs, outputs, c, next_id=500), feeds
+
+
+def test_sequence_layers_become_one_multi_layer_op():
+    g, _ = encoder_graph()
+    R.fuse_lstm_stack(g)
+    assert g.types() == ["aten::lstm", "prim::ListConstruct", "aten::cat", "prim::ListConstruct", "aten::cat", "aten::lstm",
+                         "aten::slice", "aten::slice", "aten::slice"]
+    fused = g.ops[5]
+    assert fused.attrs["num_layers"] == 3 and fused.inputs[0] == 300 and fused.outputs[0] == 303
+    assert fused.inputs[3:] == [108 + j for j in range(4)] + [116 + j for j in range(4)] + [124 + j for j in range(4)]
+    assert g.ops[1].inputs == [11, 12, 13] and g.ops[3].inputs == [21, 22, 23]
+    assert [(o.outputs[0], o.inputs[0] == fused.outputs[1 if o.outputs[0] < 320 else 2], o.attrs["start"]) for o in g.ops[6:]] == \
+        [(312, True, 1), (322, True, 1), (313, True, 2)]
+    # an initial state of constants is stacked at rewrite time
+    g, _ = encoder_graph(constant_state=True)
+    R.fuse_lstm_stack(g)
+    assert g.types() == ["aten::lstm", "aten::lstm", "aten::slice", "aten::slice", "aten::slice"]
+    h_all = g.constants[g.ops[1].inputs[1]]
+    assert list(h_all.shape) == [3, 1, 128] and torch.equal(h_all[1:2], g.constants[12])
+
+
+def test_sequence_layer_chain_guards():
+    # a residual sum around the last layer: its input has a second reader, the chain ends before it
+    g, _ = encoder_graph(residual_last=True)
+    R.fuse_lstm_stack(g)
+    fused = [o for o in g.ops if o.type == "aten::lstm" and o.attrs.get("num_layers", 1) > 1]
+    assert len(fused) == 1 and fused[0].attrs["num_layers"] == 2 and fused[0].outputs[0] == 302
+    assert [o.type for o in g.ops].count("aten::lstm") == 3 and "aten::add" in g.types()
+    # a sequence in between that is a graph output stays a tensor of its own
+    g, _ = encoder_graph()
+    g.outputs.append(302)
+    R.fuse_lstm_stack(g)
+    fused = [o for o in g.ops if o.type == "aten::lstm" and o.attrs.get("num_layers", 1) > 1]
+    assert len(fused) == 1 and fused[0].attrs["num_layers"] == 2 and fused[0].outputs[0] == 302
+    # a final state that is read before the chain ends: the chain ends at that reader
+    g, _ = encoder_graph()
+    g.ops.insert(2, R.Op("aten::relu", [311], [450]))
+    g.outputs.append(450)
+    R.fuse_lstm_stack(g)
+    fused = [o for o in g.ops if o.type == "aten::lstm" and o.attrs.get("num_layers", 1) > 1]
+    assert len(fused) == 1 and fused[0].attrs["num_layers"] == 2 and fused[0].inputs[0] == 301 and fused[0].outputs[0] == 303
+    # weights that are graph inputs, single-step cells and bidirectional layers are not taken
+    g, _ = encoder_graph()
+    g.constants.pop(117)
+    g.inputs.append(117)
+    R.fuse_lstm_stack(g)
+    assert all(o.attrs.get("num_layers", 1) == 1 for o in g.ops)
+    g, _ = decoder_graph()
+    before = g.types()
+    R.fuse_lstm_stack(g)
+    assert g.types() == before
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,T", [(128, 12), (1024, 24)])
+def test_fused_sequence_layers_match_the_operator_list_and_libtorch(ops, H, T):
+    g0, feeds = encoder_graph(H=H, T=T)
+    want_ops = [t.float().cpu() for t in R.execute(g0, feeds, DEV)]
+    g1, _ = encoder_graph(H=H, T=T)
+    R.fuse_lstm_stack(g1)
+    assert [o.attrs.get("num_layers", 1) for o in g1.ops if o.type == "aten::lstm"] == [1, 3]
+    got = [t.float().cpu() for t in R.execute(g1, feeds, DEV)]
+    assert [list(t.shape) for t in got] == [list(t.shape) for t in want_ops]
+    for a, b in zip(got, want_ops):
+        assert float((a - b).abs().max()) <= 5e-3
+    # LibTorch CPU on the original op list
+    c, f = g0.constants, feeds
+    y, _, _ = torch.lstm(f[0], (f[10], f[20]), [c[100 + j] for j in range(8)], True, 1, 0.0, False, True, False)
+    finals = {}
+    for k in range(1, 4):
+        y, hn, cn = torch.lstm(y, (f[10 + k], f[20 + k]), [c[100 + 8 * k + j] for j in range(4)], True, 1, 0.0, False, False, False)
+        finals[310 + k], finals[320 + k] = hn, cn
+    for a, b in zip(got, [y, finals[312], finals[322], finals[313]]):
+        assert list(a.shape) == list(b.shape) and float((a - b.float()).abs().max()) <= 5e-3
