@@ -447,6 +447,30 @@ def main():
             lib.pimhip_execute_gemv(yo.data_ptr(), hid.data_ptr(), w2.data_ptr(), None, 3072, 768, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, s_h)
         other["moe_ffn_step_three_gemvs_us"] = round(graph_timed_us(moe_step, 32), 3)
         other["moe_ffn_step_issued_from_python_us"] = round(timed_us(moe_step, 200), 3)
+        # the same block as ONE launch that also picks the expert (router, argmax on the GPU, W1[e], W2[e]; eight experts),
+        # and as the reference's interpreter has to run it: the argmax read back on the host between the launches
+        w1s = [w1] + [(0.02 * torch.randn(3072, 768, device=dev)).half() for _ in range(7)]
+        w2s = [w2] + [(0.02 * torch.randn(768, 3072, device=dev)).half() for _ in range(7)]
+        moe_plan = P.MoePlan((wr, None), w1s, w2s)
+        y_one, e_one = torch.empty(768, dtype=torch.float16, device=dev), torch.empty(1, dtype=torch.int32, device=dev)
+        moe_one = moe_plan.bind(tok, y_one, logits, e_one)
+        moe_one()
+        torch.cuda.synchronize()
+
+        def moe_host_routed():
+            lib.pimhip_execute_gemv(logits.data_ptr(), tok.data_ptr(), wr.data_ptr(), None, 768, 8, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+            e = int(torch.argmax(logits))
+            lib.pimhip_execute_gemv(hid.data_ptr(), tok.data_ptr(), w1s[e].data_ptr(), None, 768, 3072, 0, L.PIMHIP_ACT_RELU, L.PIMHIP_W_X_I, sh)
+            lib.pimhip_execute_gemv(yo.data_ptr(), hid.data_ptr(), w2s[e].data_ptr(), None, 3072, 768, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, sh)
+        moe_host_routed()
+        torch.cuda.synchronize()
+        other["moe_ffn_step_one_launch"] = {
+            "us": round(graph_timed_us(lambda s_: moe_one(s_), 32), 3),
+            "issued_from_python_us": round(timed_us(moe_one, 200), 3),
+            "three_gemvs_with_the_expert_chosen_on_the_host_us": round(timed_us(moe_host_routed, 100), 3),
+            "max_abs_diff_to_the_three_gemvs": round(float((y_one.float() - yo.float()).abs().max()), 6),
+            "expert": int(e_one.item())}
+        moe_plan.status()
         # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
         big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
         big_c = torch.empty_like(big_a)

@@ -295,6 +295,38 @@ int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const void* att,
 int pimhip_decoder_plan_status(PimHipDecoderPlan* plan);
 int pimhip_decoder_plan_set_spin_limit(PimHipDecoderPlan* plan, unsigned int spin_limit);
 
+/* ---- mixture-of-experts feed-forward step ----------------------------------------------------- */
+
+typedef struct PimHipMoePlan PimHipMoePlan;
+
+/* One launch for a token's pass through a top-1 mixture-of-experts feed-forward block (the Switch Transformer's):
+ *
+ *     logits = router_w[E, d_model] . x (+ router_b)      e = argmax(logits)   (first maximum, logits rounded to fp16)
+ *     hidden = act(w1[e][d_ff, d_model] . x + b1[e])                           (rounded to fp16)
+ *     y      = w2[e][d_model, d_ff] . hidden + b2[e]      (times softmax(logits)[e] when scale_by_router_prob)
+ *
+ * Replaces three customAtenAddmm / atenLinear calls (aten_ops.cpp:609-758, :304-307) and the host's choice of the
+ * expert between them, which costs the reference's interpreter a stream synchronisation and a read-back per token; here
+ * the choice is made on the GPU and only expert e's weights are read.
+ *   w1, b1, w2, b2: host arrays of E device pointers (b1 / b2 may be null arrays: no bias); all weights row-major, dense,
+ *   fp16, 16-byte aligned.  E <= 64; d_model <= 2048 and d_ff <= 4096, multiples of 8 (PIMHIP_ERR_UNSUPPORTED
+ *   otherwise: three pimhip_execute_gemv calls serve any size); act as in pimhip_execute_gemv.
+ * The plan keeps the pointers (the weights must outlive it) and owns a 32 KiB exchange buffer.  Needs a device whose
+ * 256 blocks are resident together; the library orders it against its other such launches (pimhip_lstm_forward,
+ * pimhip_decoder_step), and steps sharing a plan must be ordered on one stream. */
+int pimhip_moe_plan_create(PimHipMoePlan** plan, const void* router_w, const void* router_b, const void* const* w1,
+                           const void* const* b1, const void* const* w2, const void* const* b2, int num_experts,
+                           int64_t d_model, int64_t d_ff, int act, int scale_by_router_prob, void* stream);
+int pimhip_moe_plan_destroy(PimHipMoePlan* plan);
+
+/* x [d_model] (16-byte aligned), y [d_model]; router_logits [E] fp16 and expert [1] int32 are device pointers or null.
+ * Records one kernel.  Every wait inside is bounded: see pimhip_moe_plan_status. */
+int pimhip_moe_ffn_step(PimHipMoePlan* plan, const void* x, void* y, void* router_logits, int* expert, void* stream);
+
+/* As pimhip_decoder_plan_status / pimhip_decoder_plan_set_spin_limit. */
+int pimhip_moe_plan_status(PimHipMoePlan* plan);
+int pimhip_moe_plan_set_spin_limit(PimHipMoePlan* plan, unsigned int spin_limit);
+
 #ifdef __cplusplus
 }
 #endif

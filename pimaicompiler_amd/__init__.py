@@ -26,6 +26,7 @@ from .ops import (  # noqa: F401
     pack_projection_weight,
     LstmPlan,
     DecoderPlan,
+    MoePlan,
     prepare_lstm,
     invalidate_lstm_plans,
     gemv_status,

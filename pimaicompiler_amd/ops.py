@@ -700,6 +700,94 @@ class DecoderPlan:
         return step
 
 
+class MoePlan:
+    """One launch per token for a top-1 mixture-of-experts feed-forward block (pimhip_moe_ffn_step): router, choice of the
+    expert on the GPU, the chosen expert's two products.  The reference runs three customAtenAddmm / atenLinear calls
+    (aten_ops.cpp:609-758, :304-307) with the argmax read back on the host in between.
+
+    router = (W_r [E, d_model], b_r [E] or None); w1[e] [d_ff, d_model], w2[e] [d_model, d_ff]; b1 / b2: lists of E biases
+    or None; act_type "none" | "aten::relu" (as customAtenAddmm's); scale_by_router_prob multiplies y by softmax(logits)[e] (the Switch Transformer's
+    gating)."""
+
+    def __init__(self, router, w1, w2, b1=None, b2=None, act_type="aten::relu", scale_by_router_prob=False, stream=None):
+        lib = L.load()
+        wr, br = router
+        E = len(w1)
+        ts = [wr] + list(w1) + list(w2) + ([br] if br is not None else []) + (list(b1) if b1 is not None else []) + \
+            (list(b2) if b2 is not None else [])
+        _require_half_cuda(*ts)
+        _ensure_init(wr)
+        if wr.dim() != 2 or wr.size(0) != E or len(w2) != E or (b1 is not None and len(b1) != E) or (b2 is not None and len(b2) != E):
+            raise NNRuntimeException("router_w must be [E, d_model] with E experts in w1, w2 (and b1, b2)")
+        self.d_model, self.d_ff, self.num_experts = wr.size(1), w1[0].size(0), E
+        for e in range(E):
+            if tuple(w1[e].shape) != (self.d_ff, self.d_model) or tuple(w2[e].shape) != (self.d_model, self.d_ff):
+                raise NNRuntimeException(f"expert {e}: w1 must be [{self.d_ff}, {self.d_model}] and w2 [{self.d_model}, {self.d_ff}]")
+            if (b1 is not None and b1[e].numel() != self.d_ff) or (b2 is not None and b2[e].numel() != self.d_model):
+                raise NNRuntimeException(f"expert {e}: b1 must have {self.d_ff} and b2 {self.d_model} elements")
+        if br is not None and br.numel() != E:
+            raise NNRuntimeException(f"router bias must have {E} elements")
+        self.device = wr.device
+        self._keep = [t.contiguous() for t in ts]   # the plan reads the weights where they lie: keep them alive
+        k = iter(self._keep)
+        wr_c = next(k)
+        w1_c, w2_c = [next(k) for _ in range(E)], [next(k) for _ in range(E)]
+        br_c = next(k) if br is not None else None
+        b1_c = [next(k) for _ in range(E)] if b1 is not None else None
+        b2_c = [next(k) for _ in range(E)] if b2 is not None else None
+        mk = lambda lst: (ctypes.c_void_p * E)(*[t.data_ptr() for t in lst]) if lst is not None else None  # noqa: E731
+        handle = ctypes.c_void_p()
+        _check(lib.pimhip_moe_plan_create(ctypes.byref(handle), wr_c.data_ptr(), br_c.data_ptr() if br_c is not None else None,
+                                          mk(w1_c), mk(b1_c), mk(w2_c), mk(b2_c), E, self.d_model, self.d_ff, _act_code(act_type),
+                                          int(bool(scale_by_router_prob)), _stream_handle(stream)))
+        self._handle = handle
+        self._finalizer = weakref.finalize(self, MoePlan._destroy, handle.value)
+
+    @staticmethod
+    def _destroy(handle_value):
+        try:
+            L.load().pimhip_moe_plan_destroy(ctypes.c_void_p(handle_value))
+        except Exception:  # interpreter shutdown
+            pass
+
+    def set_spin_limit(self, limit):
+        _check(L.load().pimhip_moe_plan_set_spin_limit(self._handle, limit))
+
+    def status(self):
+        """Raises NNRuntimeException if a step's kernel gave up a wait since the last report.  Synchronises."""
+        torch.cuda.synchronize(self.device)
+        _check(L.load().pimhip_moe_plan_status(self._handle))
+
+    def bind(self, x, y, router_logits=None, expert=None):
+        """Fixes the buffers of a step (x, y [d_model] fp16; router_logits [E] fp16 and expert [1] int32 optional) and returns
+        a callable step(stream=None): what a serving loop or a graph capture calls per token."""
+        lib = L.load()
+        _require_half_cuda(x, y, *([router_logits] if router_logits is not None else []))
+        for t in (x, y, router_logits, expert):
+            if t is not None and not t.is_contiguous():
+                raise NNRuntimeException("step buffers must be contiguous")
+        if x.numel() != self.d_model or y.numel() != self.d_model:
+            raise NNRuntimeException(f"x and y must have {self.d_model} elements")
+        if router_logits is not None and router_logits.numel() != self.num_experts:
+            raise NNRuntimeException(f"router_logits must have {self.num_experts} elements")
+        if expert is not None and (expert.dtype != torch.int32 or expert.numel() != 1 or expert.device != x.device):
+            raise NNRuntimeException("expert must be one int32 on the device")
+        ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+        args = (self._handle, ptr(x), ptr(y), ptr(router_logits), ptr(expert))
+
+        def step(stream=None, _keep=(x, y, router_logits, expert)):
+            _check(lib.pimhip_moe_ffn_step(*args, _stream_handle(stream)))
+        return step
+
+    def forward(self, x, stream=None):
+        """y, router_logits, expert (device tensors; nothing is read back) for one token x [.., d_model]."""
+        y = torch.empty(self.d_model, dtype=torch.float16, device=self.device)
+        logits = torch.empty(self.num_experts, dtype=torch.float16, device=self.device)
+        expert = torch.empty(1, dtype=torch.int32, device=self.device)
+        self.bind(x.contiguous(), y, logits, expert)(stream)
+        return y.view(x.shape), logits, expert
+
+
 def _overlap(a, b):
     """True if the two tensors' storage ranges intersect (both are dense here)."""
     a0, b0 = a.data_ptr(), b.data_ptr()
