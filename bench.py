@@ -354,6 +354,21 @@ def main():
             plan_123.forward(cur, h_123, c_123)
 
         other["gnmt_lstm_stack_us_per_layer_step_layers_1_to_3_as_one_call"] = round(timed_us(gnmt_stack_two_calls, 30) / 250, 3)
+        # the encoder as GNMT wires it, with residual sums around its two upper layers: one aten::lstm and one aten::add per
+        # layer as the reference runs them, against the one call rewrite.fuse_lstm_stack makes of them
+        def gnmt_upper_layers_op_by_op():
+            cur = l0_out
+            for li, (plan_g, hg, cg) in enumerate(gn[1:]):
+                yl, _, _ = plan_g.forward(cur, hg, cg)
+                cur = P.aten_add(yl, cur) if li >= 1 else yl
+
+        l0_out = gn[0][0].forward(seq, gn[0][1], gn[0][2])[0]
+        op_by_op_us = timed_us(gnmt_upper_layers_op_by_op, 30)
+        plan_123.set_residual(1)
+        other["gnmt_encoder_upper_layers_with_residual_sums"] = {
+            "three_lstm_calls_and_two_adds_us": round(op_by_op_us, 2),
+            "one_call_us": round(timed_us(lambda: plan_123.forward(l0_out, h_123, c_123), 30), 2), "steps": 50}
+        plan_123.set_residual(None)
         # the same four calls (eight launches) replayed from a HIP graph
         other["gnmt_lstm_stack_us_per_layer_step_hip_graph"] = round(graph_timed_us(lambda _s: gnmt_stack(), 1) / 250, 3)
         # one decoder step (seq_len 1, I = H = 1024): the fused step kernel, W_ih and W_hh streamed once (16.8 MB)

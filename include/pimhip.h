@@ -196,6 +196,14 @@ int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limi
  * (a wavefront over the layers), 1 where neither fits.  A call with seq_len 1 runs the fused step launch in every mode. */
 int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);
 
+/* No counterpart in aten::lstm.  Layers first_residual_layer .. num_layers - 1 of a unidirectional stack hand up and
+ * return out_t = h_t + in_t (fp16, one rounding) instead of h_t, in_t being the layer's own input: the wiring of the GNMT
+ * encoder and decoder, which the reference runs as one executeAtenLSTM1 and one executeAtenAdd per layer
+ * (aten_ops_executor.cpp:2135-2307, :43-179).  hn / cn stay the layers' own h and c.  Such a layer's input width must equal
+ * hidden_size.  first_residual_layer >= num_layers switches it off (the default).  A stack then still runs as one
+ * pipeline launch where pimhip_lstm_forward would use one without the sums. */
+int pimhip_lstm_plan_set_residual(PimHipLstmPlan* plan, int first_residual_layer);
+
 /* The dense input projection of one LSTM layer over all time steps, the only MFMA kernel of the path:
  * out[T, n_out] (fp32) = x[T, in] (fp16) . w[n_out, in]^T (fp16) + bias[n_out] (fp32, may be NULL). */
 int pimhip_input_projection(void* out, const void* x, const void* w, const void* bias, int64_t seq_len,

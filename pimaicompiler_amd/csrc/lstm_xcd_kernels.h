@@ -70,6 +70,8 @@ struct XcdChain {
     half_t* seq_out;      // [T][H], one slot per step, read by the P group of the layer above; null for the last layer
     int reverse;          // 1: t = T-1 .. 0
     int xproj_polled;     // 1: the rows of xproj are written during this launch (all-ones bytes = not yet)
+    const half_t* res_in; // [T][H]: the layer's own input, added to its output (y and seq_out get h + in); null: no residual sum
+    int res_polled;       // 1: res_in is the seq_out of the layer below, written during this launch (all-ones fp16 = not yet)
 };
 
 struct XcdProj {
@@ -136,12 +138,17 @@ __device__ __forceinline__ float row16_transpose_sum4(const float (&acc)[4], int
 
 // PIPE = false: groups that neither feed nor are fed across XCDs (a single layer, the two directions of one); everything
 // that concerns P groups and the hand-overs is compiled out, which is worth 10 % of a step.
-template <bool PIPE>
+// RES = true: layers with a residual sum (out_t = h_t + in_t).  The sum is made where h leaves the workgroup: the wavefront
+// that hands the previous step's 32 h values to the layer above adds the layer's own input of that step, which it asked
+// for a step earlier, and stores y from there too (one step late; hn stays h).  Compiled in only for stacks that have such
+// layers.
+template <bool PIPE, bool RES = false>
 __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p)
 {
     __shared__ __align__(16) half_t hbuf[2][kXcdMaxH];  // h of the previous step, double buffered by step parity
     __shared__ __align__(16) float xring[kXcdWaves][32][4][4];  // per wavefront: [step & 31][gate][unit] projection terms
     __shared__ __align__(16) unsigned long long hout[2][kXcdWaves];  // the workgroup's 32 new h values, for the layer above
+    __shared__ unsigned short in_ring[2][kXcdUnitsPerBlock];        // RES: the layer's own input of the last two steps, for the sums
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -206,7 +213,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     // Lanes 0..31 of wavefronts 0..3 fetch piece 32 w + lane of an h vector: 8 fp16 = columns 8 q .. 8 q + 7.  (The other
     // wavefronts never poll: they are the ones that talk to other XCDs, and a wavefront's loads come back in order.)
     // A group that neither feeds nor is fed across XCDs spreads the polls over all eight wavefronts, 16 lanes each.
-    const bool crosses = PIPE && (is_proj || ch.xproj_polled != 0 || ch.seq_out != nullptr);
+    const bool crosses = PIPE && (is_proj || ch.xproj_polled != 0 || ch.seq_out != nullptr || (RES && ch.res_in != nullptr));
     const int piece = crosses ? wave * 32 + lane : wave * 16 + lane;
     const bool polls = (crosses ? (wave < 4 && lane < 32) : lane < 16) && piece * 8 < H;
 
@@ -286,9 +293,41 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     // ================= R group: the recurrence of chain k =================
     // Compiled once per combination of "its projection rows arrive during the launch" and "its h goes to a layer above":
     // a step is sensitive to every instruction on its path, and the plain combination should not carry the others'.
-    auto recurrence = [&](auto polled_c, auto feeds_c) __attribute__((always_inline)) {
+    auto recurrence = [&](auto polled_c, auto feeds_c, auto res_c) __attribute__((always_inline)) {
     constexpr bool polled = decltype(polled_c)::value;
     constexpr bool feeds = decltype(feeds_c)::value;
+    constexpr bool res = decltype(res_c)::value;
+    constexpr bool emits = feeds || res;  // the workgroup's h values leave through hout, one step late
+    // Without a residual sum: lanes 0..3 of wavefront 4 hand step se's 32 h values to the layer above, 16 bytes each.
+    auto emit = [&](int se) __attribute__((always_inline)) {
+        const unsigned long long* src = &hout[se & 1][2 * lane];
+        store16_device_scope(ch.seq_out + (long)se * H + rank * kXcdUnitsPerBlock + lane * 8, src[0], src[1]);
+    };
+    // With one: lanes 0..31 of wavefront 4, one value each: a handful of instructions per step (eight values in each of
+    // four lanes took 0.1 us per step more).
+    const int eu = rank * kXcdUnitsPerBlock + (lane & 31);  // the unit an emitting lane handles
+    const bool sums = res && wave == 4 && lane < 32 && eu < H;
+    // The input of step s is asked for right after that step's barrier, together with the projection rows two steps ahead
+    // (it exists: the projection row made from it is in use), parked in LDS at the top of step s + 1 and added after
+    // that step's barrier.  Every wavefront drains its loads once per step, so what matters is that the load leaves
+    // early in the step: issued behind the sum of the step before, it cost 0.23 us per step.
+    unsigned short in_ahead = 0xffffu;
+    auto emit_sum = [&](int se) __attribute__((always_inline)) {
+        unsigned short in_bits = in_ring[se & 1][lane & 31];
+        if (ch.res_polled && in_bits == 0xffffu) {
+            const unsigned short* rin = reinterpret_cast<const unsigned short*>(ch.res_in) + (long)se * H + eu;
+            bounded_wait([&]() {
+                in_bits = __hip_atomic_load(rin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return in_bits != 0xffffu;
+            });
+        }
+        const unsigned short hbits = reinterpret_cast<const unsigned short*>(&hout[se & 1][0])[lane & 31];
+        const float v = (float)__builtin_bit_cast(half_t, hbits) + (float)__builtin_bit_cast(half_t, in_bits);
+        const unsigned short ob = (v == v) ? __builtin_bit_cast(unsigned short, (half_t)v) : (unsigned short)0x7e00u;
+        if (ch.y) reinterpret_cast<unsigned short*>(ch.y)[(long)se * p.y_stride + eu] = ob;
+        if (feeds)
+            __hip_atomic_store(reinterpret_cast<unsigned short*>(ch.seq_out) + (long)se * H + eu, ob, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
     float c_reg = (float)ch.c0[uc];
     const bool rev = ch.reverse != 0;
 
@@ -346,6 +385,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
             reinterpret_cast<unsigned int&>(xring[wave][(s + 1) & 31][my_gate][lane >> 4]) = xp_ahead;
             reinterpret_cast<unsigned int&>(xring[wave - 4][(s + 1) & 31][my_gate][lane >> 4]) = xp_ahead_other;
         }
+        if (sums && s > 0) in_ring[(s - 1) & 1][lane & 31] = in_ahead;  // read after this step's barrier
         // ---- 1. h of the previous step into LDS
         if (polls) {
             half8_t hv;
@@ -375,9 +415,11 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
         }
         // The previous step's h of the whole workgroup (gathered in LDS before the barrier) goes to the layer above, from a
         // wavefront that does not poll.
-        if (feeds && s > 0 && wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) {
-            const unsigned long long* src = &hout[(s - 1) & 1][2 * lane];
-            store16_device_scope(ch.seq_out + (long)(s - 1) * H + rank * kXcdUnitsPerBlock + lane * 8, src[0], src[1]);
+        if (!res && feeds && s > 0 && wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) emit(s - 1);
+        if (sums) {
+            in_ahead = __hip_atomic_load(reinterpret_cast<const unsigned short*>(ch.res_in) + (long)s * H + eu, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+            if (s > 0) emit_sum(s - 1);
         }
 
         // ---- 2. the four gate rows of this row of lanes' unit
@@ -418,7 +460,7 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
         for (int i = 0; i < 4; ++i) {
             yw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)hb16, 16 * i) << (16 * i);
             pw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)pb16, 16 * i) << (16 * i);
-            if (feeds) sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
+            if (emits) sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
         }
         if (lane == 0) {
             const unsigned int g = g_base + (unsigned int)s;
@@ -426,28 +468,33 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
             // units past H publish zeros with the flag, so that every piece of a member's entry validates
             unsigned char* dst = reinterpret_cast<unsigned char*>(region + ((long)(g & 1u) * kXcdMembers + rank) * kXcdEntryWords) + wave * 8;
             store8_plain(dst, (units_ok ? pw : 0ull) | flag);
-            if (units_ok && ch.y) *reinterpret_cast<unsigned long long*>(ch.y + (long)t * p.y_stride + u0) = yw;
-            if (feeds) hout[s & 1][wave] = sw;
+            if (!res && units_ok && ch.y) *reinterpret_cast<unsigned long long*>(ch.y + (long)t * p.y_stride + u0) = yw;
+            if (emits) hout[s & 1][wave] = sw;
         }
         if (s == T - 1 && units_ok && (lane & 15) == 0) {
             ch.hn[my_unit] = h;
             ch.cn[my_unit] = (half_t)c_new;
         }
     }
-    if (feeds) {
+    if (emits) {
+        if (sums) in_ring[(T - 1) & 1][lane & 31] = in_ahead;
         lds_barrier();
-        if (wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) {
-            const unsigned long long* src = &hout[(T - 1) & 1][2 * lane];
-            store16_device_scope(ch.seq_out + (long)(T - 1) * H + rank * kXcdUnitsPerBlock + lane * 8, src[0], src[1]);
-        }
+        if (!res && wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) emit(T - 1);
+        if (sums) emit_sum(T - 1);
     }
     };
     const bool polled_rt = PIPE && ch.xproj_polled != 0;
     const bool feeds_rt = PIPE && ch.seq_out != nullptr;
-    if (!PIPE || (!polled_rt && !feeds_rt)) recurrence(std::false_type{}, std::false_type{});
-    else if (!polled_rt) recurrence(std::false_type{}, std::true_type{});
-    else if (!feeds_rt) recurrence(std::true_type{}, std::false_type{});
-    else recurrence(std::true_type{}, std::true_type{});
+    const bool res_rt = RES && ch.res_in != nullptr;
+    if (RES && res_rt) {
+        if (!polled_rt && !feeds_rt) recurrence(std::false_type{}, std::false_type{}, std::true_type{});
+        else if (!polled_rt) recurrence(std::false_type{}, std::true_type{}, std::true_type{});
+        else if (!feeds_rt) recurrence(std::true_type{}, std::false_type{}, std::true_type{});
+        else recurrence(std::true_type{}, std::true_type{}, std::true_type{});
+    } else if (!PIPE || (!polled_rt && !feeds_rt)) recurrence(std::false_type{}, std::false_type{}, std::false_type{});
+    else if (!polled_rt) recurrence(std::false_type{}, std::true_type{}, std::false_type{});
+    else if (!feeds_rt) recurrence(std::true_type{}, std::false_type{}, std::false_type{});
+    else recurrence(std::true_type{}, std::true_type{}, std::false_type{});
     // Rank 0 has finished its last step, for which (T >= 2) it needed what every member published one step earlier:
     // every member has read the counter by now.
     if (rank == 0 && tid == 0)

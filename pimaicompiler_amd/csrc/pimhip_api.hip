@@ -733,6 +733,8 @@ struct PimHipLstmPlan {
     unsigned int* g_counters = nullptr;  // device, [kSeqMaxChains + 1]: per chain count, super-steps its region of hx has seen, plus 2
     size_t hx_region_words = 0;      // 32-bit words of one region of hx (one region per chain count)
     int max_wavefront = kSeqMaxChains;  // layers of a unidirectional stack advanced by one persistent launch
+    int first_residual_layer = 1 << 30;  // layers from this one on give out_t = h_t + in_t (pimhip_lstm_plan_set_residual)
+    bool xcd_res_ok = false;         // the pipeline kernel with residual sums is resident on this device
 
     struct Cell {
         const half_t* w_ih = nullptr;
@@ -966,6 +968,9 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_xcd_f16_kernel<false>, kXcdThreads, 0));
         PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_pipe, lstm_xcd_f16_kernel<true>, kXcdThreads, 0));
         plan->xcd_ok = per_cu >= 1 && per_cu_pipe >= 1;
+        int per_cu_res = 0;
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_res, lstm_xcd_f16_kernel<true, true>, kXcdThreads, 0));
+        plan->xcd_res_ok = plan->xcd_ok && per_cu_res >= 1;
     }
     if (plan->xcd_ok) {
         const size_t words = (size_t)kXcdRegionWords * kXcdMaxChains;
@@ -1029,6 +1034,21 @@ extern "C" int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode)
     // Modes 3 and 0 / 2 lay out a single chain's exchange entries differently: start over from a cleared buffer.
     if ((plan->mode == 3) != (mode == 3)) plan->reset_exchange = true;
     plan->mode = mode;
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_lstm_plan_set_residual(PimHipLstmPlan* plan, int first_residual_layer)
+{
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    if (first_residual_layer < 0) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "first_residual_layer=%d is negative", first_residual_layer);
+    if (first_residual_layer < plan->num_layers) {
+        if (plan->num_dirs != 1) return fail(PIMHIP_ERR_UNSUPPORTED, "residual sums are for unidirectional stacks");
+        for (int l = first_residual_layer; l < plan->num_layers; ++l)
+            if (plan->cells[(size_t)l].in_w != plan->hidden)
+                return fail(PIMHIP_ERR_INVALID_ARGUMENT, "layer %d has input width %lld and hidden size %lld: its input cannot be added to its output",
+                            l, (long long)plan->cells[(size_t)l].in_w, (long long)plan->hidden);
+    }
+    plan->first_residual_layer = first_residual_layer;
     return PIMHIP_OK;
 }
 
@@ -1167,6 +1187,14 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
 
     const half_t* layer_in = (const half_t*)x;
     const long y_stride = (long)D * H;
+    auto residual = [&](int l) { return D == 1 && l >= plan->first_residual_layer; };
+    // out = out + in over a whole sequence, for the paths that run a layer with a residual sum as a launch of its own
+    auto add_input = [&](half_t* out, const half_t* in) {
+        const long total8 = (long)T * H / 8;
+        long grid = (total8 + 255) / 256;
+        if (grid > 8L * st->num_cus) grid = 8L * st->num_cus;
+        add_f16_vec_kernel<<<(unsigned)grid, 256, 0, s>>>(out, in, out, total8, (long)(H / 8), 0);
+    };
     if (use_xcd) {
         // The groups of a launch have to be resident together, like the sequence kernel's blocks.
         if (!capturing) {
@@ -1178,6 +1206,9 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         // j of the launch on XCD 2 j, the group that makes its projection rows from the layer below on XCD 2 j - 1).
         for (int l = 0; D == 1 && L >= 2 && l < L;) {
             const int n = (L - l) < kXcdMaxChains ? (L - l) : kXcdMaxChains;
+            bool any_res = false;
+            for (int j = 0; j < n; ++j) any_res = any_res || residual(l + j);
+            if (any_res && !plan->xcd_res_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "the pipeline kernel with residual sums is not resident on this device");
             const int last = l + n - 1;
             half_t* group_out = (last == L - 1) ? (half_t*)y : plan->ybuf[last & 1];
             const PimHipLstmPlan::Cell& cf = plan->cells[(size_t)l];
@@ -1206,6 +1237,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                 a.role[2 * j] = j + 1;
                 if (j == 0) {
                     ch.xproj = plan->xproj;
+                    if (residual(ci)) ch.res_in = layer_in;
                 } else {
                     unsigned char* boundary = plan->xcd_pipe + plan->xcd_pipe_boundary_bytes * (size_t)(j - 1);
                     half_t* seq = reinterpret_cast<half_t*>(boundary);
@@ -1213,6 +1245,10 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                     a.chain[j - 1].seq_out = seq;
                     ch.xproj = xp;
                     ch.xproj_polled = 1;
+                    if (residual(ci)) {
+                        ch.res_in = seq;  // what the layer below hands up (its own residual sum included) is this layer's input
+                        ch.res_polled = 1;
+                    }
                     XcdProj& pj = a.proj[j - 1];
                     pj.w_ih = plan->cells[ci].w_ih;
                     pj.bsum = plan->cells[ci].bsum;
@@ -1236,7 +1272,10 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             a.H = (int)H;
             a.T = (int)T;
             a.spin_limit = plan->spin_limit;
-            lstm_xcd_f16_kernel<true><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+            if (any_res)
+                lstm_xcd_f16_kernel<true, true><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+            else
+                lstm_xcd_f16_kernel<true><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
             PIMHIP_HIP_CHECK(hipGetLastError());
             layer_in = group_out;
             l += n;
@@ -1281,6 +1320,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             a.T = (int)T;
             a.spin_limit = plan->spin_limit;
             lstm_xcd_f16_kernel<false><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+            if (residual(l)) add_input(layer_out, layer_in);
             PIMHIP_HIP_CHECK(hipGetLastError());
             layer_in = layer_out;
         }
@@ -1295,7 +1335,13 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         // bidirectional layer, or up to kSeqMaxChains consecutive layers of a unidirectional stack as a wavefront.
         int l = 0;
         while (l < L) {
-            const int group_layers = (D == 2) ? 1 : ((L - l) < plan->max_wavefront ? (L - l) : plan->max_wavefront);
+            int group_layers = (D == 2) ? 1 : ((L - l) < plan->max_wavefront ? (L - l) : plan->max_wavefront);
+            if (D == 1) {
+                // a layer with a residual sum runs alone: its input and its output both have to exist as sequences
+                int gl = 1;
+                while (!residual(l) && gl < group_layers && !residual(l + gl)) ++gl;
+                group_layers = gl;
+            }
             const int nc = (D == 2) ? 2 : group_layers;
             const int last = l + group_layers - 1;
             half_t* group_out = (last == L - 1) ? (half_t*)y : plan->ybuf[last & 1];
@@ -1367,6 +1413,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                     default: lstm_seq_f16_kernel<4, true><<<grid, block, 0, s>>>(a); break;
                 }
             }
+            if (residual(l)) add_input(group_out, layer_in);
             PIMHIP_HIP_CHECK(hipGetLastError());
             layer_in = group_out;
             l += group_layers;
@@ -1400,6 +1447,10 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                         (step == 0) ? c0c : nullptr, cst, yd + t * y_stride, last ? hnc : nullptr, last ? cnc : nullptr,
                         (int)in_w, (int)H);
                 }
+                PIMHIP_HIP_CHECK(hipGetLastError());
+            }
+            if (residual(l)) {
+                add_input(layer_out, layer_in);
                 PIMHIP_HIP_CHECK(hipGetLastError());
             }
             layer_in = layer_out;

@@ -532,6 +532,11 @@ class LstmPlan:
         4 one recurrence per XCD (pimhip_lstm_plan_set_mode)."""
         _check(L.load().pimhip_lstm_plan_set_mode(self._handle, mode))
 
+    def set_residual(self, first_residual_layer):
+        """Layers from `first_residual_layer` on return and hand up h + their own input (the GNMT wiring: an aten::lstm and an
+        aten::add per layer in the reference); None or >= num_layers switches it off (pimhip_lstm_plan_set_residual)."""
+        _check(L.load().pimhip_lstm_plan_set_residual(self._handle, self.num_layers if first_residual_layer is None else int(first_residual_layer)))
+
     def set_spin_limit(self, limit):
         _check(L.load().pimhip_lstm_plan_set_spin_limit(self._handle, limit))
 

@@ -450,33 +450,57 @@ def fuse_lstm_stack(g: Graph):
     with num_layers = n and the parameters of the layers in order, placed where the chain's last op was.  The stacked
     hn / cn are sliced back into the tensors the single ops produced, for whoever reads them.
 
-    A layer joins the chain when it is the only reader of the sequence before it, that sequence is not a graph output,
-    its input width is the hidden size of the layer before (as in a multi-layer aten::lstm) and its hidden size is the
-    same.  Left alone: layers with a residual sum around them (their input has a second reader), layers whose initial
-    state is computed from the chain itself, chains whose intermediate hn / cn are read before the chain's end."""
+    A layer may carry a residual sum, out = lstm(in) + in (the GNMT encoder's upper layers): from the first such layer on
+    every layer of the chain has to, and the fused op is then a `pimhip::lstm_stack` with `first_residual_layer` (an
+    aten::lstm has no such wiring; ops.LstmPlan.set_residual runs it as the same one-launch pipeline).
+
+    A layer joins the chain when the sequence before it is read by nothing but that layer (and its own residual sum) and
+    is not a graph output, its input width is the hidden size of the layer before (as in a multi-layer aten::lstm) and its
+    hidden size is the same.  Left alone: layers whose y is read before the sum, layers whose initial state is computed
+    from the chain itself, chains whose intermediate hn / cn are read before the chain's end, a plain layer above one with
+    a residual sum."""
     taken = set()
     for first in list(g.ops):
         if id(first) in taken or all(first is not o for o in g.ops) or not _sequence_layer(g, first):
             continue
-        chain = [first]
+
+        def form(op):
+            """(out, add op or None) of a layer: its residual sum when y feeds exactly one add with the layer's own input."""
+            out, add = _lstm_output_form(g, op, op.inputs[0])
+            if add is not None and g.constants[op.inputs[3]].size(1) != g.constants[op.inputs[4]].size(1):
+                return op.outputs[0], None
+            return out, add
+
+        chain, adds = [first], [form(first)[1]]
+        cur = form(first)[0]
         while True:
             last = chain[-1]
-            y = last.outputs[0]
-            users = g.consumers(y)
-            if len(users) != 1 or y in g.outputs or users[0].inputs.count(y) != 1 or users[0].inputs[0] != y:
+            users = g.consumers(cur)
+            cand = [u for u in users if u.type == "aten::lstm" and u.inputs[0] == cur]
+            if len(cand) != 1 or cur in g.outputs:
                 break
-            nxt = users[0]
+            nxt = cand[0]
             H = g.constants[last.inputs[4]].size(1)
             if not _sequence_layer(g, nxt) or g.constants[nxt.inputs[4]].size(1) != H or g.constants[nxt.inputs[3]].size(1) != H:
                 break
+            n_out, n_add = form(nxt)
+            allowed = [nxt] + ([n_add] if n_add is not None else [])
+            if any(all(u is not a for a in allowed) for u in users) or sum(u.inputs.count(cur) for u in users) != len(allowed):
+                break  # somebody else reads the sequence in between
+            if n_add is None and any(a is not None for a in adds):
+                break  # a plain layer above one with a residual sum
             if any(_depends_on(g, t, chain) for t in nxt.inputs[1:3]):
                 break
             if nxt.attrs.get("seq_len", 0) != last.attrs.get("seq_len", 0):
                 break
             chain.append(nxt)
-        # the intermediate hn / cn must not be read before the place the fused op takes (the last op's)
+            adds.append(n_add)
+            cur = n_out
+        # a first layer with a residual sum whose y has another reader was refused by form(); nothing else to check there.
+        # The intermediate hn / cn must not be read before the place the fused op takes (the last op's).
         while len(chain) >= 2:
-            end = next(i for i, o in enumerate(g.ops) if o is chain[-1])
+            tail = adds[-1] if adds[-1] is not None else chain[-1]
+            end = next(i for i, o in enumerate(g.ops) if o is tail)
             early = False
             for o in chain[:-1]:
                 for t in o.outputs[1:3]:
@@ -486,18 +510,20 @@ def fuse_lstm_stack(g: Graph):
             if not early:
                 break
             chain.pop()
+            adds.pop()
         if len(chain) < 2:
             continue
         n = len(chain)
-        state = []
-        pre = []
+        first_res = next((k for k, a in enumerate(adds) if a is not None), n)
+        out_tid = adds[-1].outputs[0] if adds[-1] is not None else chain[-1].outputs[0]
+        state, pre = [], []
         for slot in (1, 2):
             ids = [o.inputs[slot] for o in chain]
             if all(g.is_constant(t) and g.constants[t] is not None for t in ids):
                 tid = g.new_id()
                 g.constants[tid] = torch.cat([g.constants[t].reshape(1, 1, -1) for t in ids], 0)
             else:
-                lst, tid = g.new_id(), None
+                lst = g.new_id()
                 pre.append(Op("prim::ListConstruct", ids, [lst]))
                 tid = g.new_id()
                 pre.append(Op("aten::cat", [lst], [tid], {"dim": 0}))
@@ -506,17 +532,32 @@ def fuse_lstm_stack(g: Graph):
         params = [t for o in chain for t in o.inputs[3:7]]
         attrs = dict(chain[0].attrs)
         attrs["num_layers"] = n
-        fused = Op("aten::lstm", [chain[0].inputs[0]] + state + params, [chain[-1].outputs[0], hn_all, cn_all], attrs)
+        if first_res < n:
+            attrs["first_residual_layer"] = first_res
+        fused = Op("aten::lstm" if first_res == n else "pimhip::lstm_stack", [chain[0].inputs[0]] + state + params,
+                   [out_tid, hn_all, cn_all], attrs)
         post = []
         for k, o in enumerate(chain):
             for t, src in ((o.outputs[1], hn_all), (o.outputs[2], cn_all)):
                 if g.consumers(t) or t in g.outputs:
                     post.append(Op("aten::slice", [src], [t], {"dim": 0, "start": k, "end": k + 1}))
-        end = next(i for i, o in enumerate(g.ops) if o is chain[-1])
+        gone = chain + [a for a in adds if a is not None]
+        tail = adds[-1] if adds[-1] is not None else chain[-1]
+        end = next(i for i, o in enumerate(g.ops) if o is tail)
         g.ops[end:end + 1] = pre + [fused] + post
-        g.ops = [o for o in g.ops if all(o is not c for c in chain)]
-        taken.update(id(o) for o in chain)
+        g.ops = [o for o in g.ops if all(o is not c for c in gone)]
+        taken.update(id(o) for o in gone)
     return g
+
+
+def _stack_plan(op: Op, ops, params, n, T):
+    """The plan of a pimhip::lstm_stack op, kept on the op (its weights are constants of the graph)."""
+    plan = op.attrs.get("_plan")
+    if plan is None or plan.max_seq_len < T or any(p.data_ptr() != q.data_ptr() for p, q in zip(plan.params, params)):
+        plan = ops.LstmPlan(list(params), True, n, False, max(T, 16))
+        plan.set_residual(op.attrs["first_residual_layer"])
+        op.attrs["_plan"] = plan
+    return plan
 
 
 def _as_row_major_weight(t):
@@ -620,6 +661,13 @@ def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0", same_sent
             continue
         elif op.type == "pimhip::decoder_step":
             _run_decoder_step(op, env, ops, same_sentence)
+            continue
+        elif op.type == "pimhip::lstm_stack":
+            n = op.attrs["num_layers"]
+            T = a[0].size(0)
+            plan = _stack_plan(op, ops, a[3:3 + 4 * n], n, T)
+            y, hn, cn = plan.forward(a[0].reshape(T, a[0].size(2)), a[1], a[2])
+            env[op.outputs[0]], env[op.outputs[1]], env[op.outputs[2]] = y.view(T, 1, -1), hn.view(n, 1, -1), cn.view(n, 1, -1)
             continue
         elif op.type == "aten::lstm":
             n = op.attrs.get("num_layers", 1)

@@ -89,6 +89,66 @@ def test_lstm_matches_oracle(ops, I, H, L, bidir, T, has_b, mode):
     assert maxabs(y, wy) <= 2e-3 and maxabs(hn, whn) <= 2e-3 and maxabs(cn, wcn) <= 2e-3
 
 
+# ---- stacks with residual sums (the GNMT wiring): layer by layer on LibTorch CPU ----------------------------------
+RESIDUAL_CASES = [  # I, H, L, first residual layer, T, biases
+    (2048, 1024, 3, 1, 50, True),    # the GNMT encoder above its bidirectional layer
+    (64, 64, 4, 2, 20, True),
+    (128, 128, 2, 0, 9, False),      # the first layer too (its input is the call's)
+    (40, 40, 5, 1, 33, True),        # a last pipeline launch of one layer
+    (1024, 1024, 1, 0, 70, True),    # a single layer
+    (72, 72, 3, 2, 1, True),         # one step
+    (24, 136, 6, 3, 5, True),
+]
+
+
+def libtorch_residual_stack(params, x, h0, c0, has_b, L, first_res):
+    """One at::lstm and one at::add per layer, fp16 on the CPU: what the reference's interpreter runs."""
+    per = 4 if has_b else 2
+    cur, hs, cs = x, [], []
+    for l in range(L):
+        y, hn, cn = torch.lstm(cur, (h0[l:l + 1], c0[l:l + 1]), params[l * per:(l + 1) * per], has_b, 1, 0.0, False, False, False)
+        hs.append(hn)
+        cs.append(cn)
+        cur = y + cur if l >= first_res else y
+    return cur, torch.cat(hs, 0), torch.cat(cs, 0)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 4])
+@pytest.mark.parametrize("I,H,L,first_res,T,has_b", RESIDUAL_CASES)
+def test_residual_stack_matches_libtorch_layer_by_layer(ops, I, H, L, first_res, T, has_b, mode):
+    params, x, h0, c0 = workloads.lstm_inputs(700 + H + T, I, H, L, False, T, has_b)
+    g = torch.Generator().manual_seed(T)
+    h0 = (0.3 * torch.randn(h0.shape, generator=g)).half()
+    c0 = (0.3 * torch.randn(c0.shape, generator=g)).half()
+    want_y, want_hn, want_cn = libtorch_residual_stack(params, x, h0, c0, has_b, L, first_res)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], has_b, L, False, T)
+    if mode:
+        plan.set_mode(mode)
+    plan.set_residual(first_res)
+    for rep in range(2):                              # a second call finds the hand-over slots of the first
+        y, hn, cn = plan.forward(x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV))
+        plan.status()
+        assert maxabs(y, want_y) <= LSTM_TOL and maxabs(hn, want_hn) <= LSTM_TOL and maxabs(cn, want_cn) <= LSTM_TOL
+    # switched off again, the plan is a plain stack
+    plan.set_residual(None)
+    y, hn, cn = plan.forward(x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV))
+    plan.status()
+    wy, whn, wcn = torch.lstm(x, (h0, c0), params, has_b, L, 0.0, False, False, False)
+    assert maxabs(y, wy) <= LSTM_TOL and maxabs(hn, whn) <= LSTM_TOL
+
+
+def test_residual_needs_equal_widths_and_one_direction(ops):
+    params, x, h0, c0 = workloads.lstm_inputs(1, 64, 32, 2, False, 4)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 2, False, 4)
+    with pytest.raises(ops.NNRuntimeException):
+        plan.set_residual(0)                          # layer 0 is 64 wide, its output 32
+    plan.set_residual(1)
+    params, x, h0, c0 = workloads.lstm_inputs(1, 32, 32, 2, True, 4)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 2, True, 4)
+    with pytest.raises(ops.NNRuntimeException):
+        plan.set_residual(1)
+
+
 def test_persistent_kernel_refuses_what_it_cannot_hold(ops):
     params, x, h0, c0 = workloads.lstm_inputs(1, 16, 2056, 1, False, 2)
     plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 2)

@@ -332,10 +332,10 @@ def test_fused_decoder_graph_matches_the_operator_list_and_libtorch(ops, query_f
 
 
 # ---- consecutive sequence layers into one multi-layer op --------------------------------------------------------------
-def encoder_graph(seed=21, H=128, T=12, residual_last=False, constant_state=False):
+def encoder_graph(seed=21, H=128, T=12, residual_from=4, constant_state=False):
     """The GNMT encoder as the interpreter sees it: a bidirectional layer, then three one-direction layers, each an
-    aten::lstm of its own reading the sequence before it (the first of them 2H wide); optionally a residual sum around
-    the last one."""
+    aten::lstm of its own reading the sequence before it (the first of them 2H wide); layers from `residual_from` on
+    (2 in GNMT) with a residual sum around them."""
     from pimaicompiler_amd import workloads
     g = torch.Generator().manual_seed(seed)
     c, ops, feeds = {}, [], {}
@@ -350,9 +350,9 @@ def encoder_graph(seed=21, H=128, T=12, residual_last=False, constant_state=Fals
         for j, t in enumerate(prm):
             c[100 + 8 * k + j] = t
         ops.append(R.Op("aten::lstm", [prev, 10 + k, 20 + k] + [100 + 8 * k + j for j in range(4)], [300 + k, 310 + k, 320 + k], {"seq_len": T}))
-        if k == 3 and residual_last:
-            ops.append(R.Op("aten::add", [303, prev], [353]))
-            prev = 353
+        if k >= residual_from:
+            ops.append(R.Op("aten::add", [300 + k, prev], [350 + k]))
+            prev = 350 + k
         else:
             prev = 300 + k
     feeds[X] = torch.randn(T, 1, H, generator=g).half()
@@ -389,12 +389,33 @@ def test_sequence_layers_become_one_multi_layer_op():
 
 
 def test_sequence_layer_chain_guards():
-    # a residual sum around the last layer: its input has a second reader, the chain ends before it
-    g, _ = encoder_graph(residual_last=True)
+    # residual sums (GNMT: around the two upper layers) go into the fused op
+    g, _ = encoder_graph(residual_from=2)
     R.fuse_lstm_stack(g)
-    fused = [o for o in g.ops if o.type == "aten::lstm" and o.attrs.get("num_layers", 1) > 1]
-    assert len(fused) == 1 and fused[0].attrs["num_layers"] == 2 and fused[0].outputs[0] == 302
-    assert [o.type for o in g.ops].count("aten::lstm") == 3 and "aten::add" in g.types()
+    assert g.types()[:5] == ["aten::lstm", "prim::ListConstruct", "aten::cat", "prim::ListConstruct", "aten::cat"]
+    fused = g.ops[5]
+    assert fused.type == "pimhip::lstm_stack" and fused.attrs["num_layers"] == 3 and fused.attrs["first_residual_layer"] == 1
+    assert fused.inputs[0] == 300 and fused.outputs[0] == 353 and "aten::add" not in g.types()
+    # ... unless the sum is not of the layer's own input, or y is read before the sum, or a plain layer follows
+    g, _ = encoder_graph(residual_from=3)
+    g.ops[4].inputs = [303, 301]                    # add(y3, y1): not a residual sum of layer 3
+    R.fuse_lstm_stack(g)
+    fused = [o for o in g.ops if o.attrs.get("num_layers", 1) > 1]
+    assert len(fused) == 1 and fused[0].type == "aten::lstm" and fused[0].attrs["num_layers"] == 2 and "aten::add" in g.types()
+    g, _ = encoder_graph(residual_from=3)
+    g.ops.append(R.Op("aten::relu", [303], [450]))  # y3 itself is read
+    g.outputs.append(450)
+    R.fuse_lstm_stack(g)
+    fused = [o for o in g.ops if o.attrs.get("num_layers", 1) > 1]
+    assert len(fused) == 1 and fused[0].type == "aten::lstm" and fused[0].attrs["num_layers"] == 2 and "aten::add" in g.types()
+    g, _ = encoder_graph(residual_from=2)
+    g.ops = [o for o in g.ops if not (o.type == "aten::add" and o.outputs[0] == 353)]   # layer 3 plain above layer 2 with a sum
+    g.ops[-1].inputs[0] = 352
+    g.outputs[0] = 303
+    R.fuse_lstm_stack(g)
+    fused = [o for o in g.ops if o.attrs.get("num_layers", 1) > 1]
+    assert len(fused) == 1 and fused[0].type == "pimhip::lstm_stack" and fused[0].attrs["num_layers"] == 2 and fused[0].outputs[0] == 352
+    assert [o.type for o in g.ops].count("aten::lstm") == 2
     # a sequence in between that is a graph output stays a tensor of its own
     g, _ = encoder_graph()
     g.outputs.append(302)
@@ -421,13 +442,13 @@ def test_sequence_layer_chain_guards():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,T", [(128, 12), (1024, 24)])
-def test_fused_sequence_layers_match_the_operator_list_and_libtorch(ops, H, T):
-    g0, feeds = encoder_graph(H=H, T=T)
+@pytest.mark.parametrize("H,T,residual_from", [(128, 12, 4), (1024, 24, 4), (128, 12, 2), (1024, 50, 2), (256, 20, 3)])
+def test_fused_sequence_layers_match_the_operator_list_and_libtorch(ops, H, T, residual_from):
+    g0, feeds = encoder_graph(H=H, T=T, residual_from=residual_from)
     want_ops = [t.float().cpu() for t in R.execute(g0, feeds, DEV)]
-    g1, _ = encoder_graph(H=H, T=T)
+    g1, _ = encoder_graph(H=H, T=T, residual_from=residual_from)
     R.fuse_lstm_stack(g1)
-    assert [o.attrs.get("num_layers", 1) for o in g1.ops if o.type == "aten::lstm"] == [1, 3]
+    assert [o.attrs.get("num_layers", 1) for o in g1.ops if o.type in ("aten::lstm", "pimhip::lstm_stack")] == [1, 3]
     got = [t.float().cpu() for t in R.execute(g1, feeds, DEV)]
     assert [list(t.shape) for t in got] == [list(t.shape) for t in want_ops]
     for a, b in zip(got, want_ops):
@@ -437,7 +458,8 @@ def test_fused_sequence_layers_match_the_operator_list_and_libtorch(ops, H, T):
     y, _, _ = torch.lstm(f[0], (f[10], f[20]), [c[100 + j] for j in range(8)], True, 1, 0.0, False, True, False)
     finals = {}
     for k in range(1, 4):
-        y, hn, cn = torch.lstm(y, (f[10 + k], f[20 + k]), [c[100 + 8 * k + j] for j in range(4)], True, 1, 0.0, False, False, False)
+        yk, hn, cn = torch.lstm(y, (f[10 + k], f[20 + k]), [c[100 + 8 * k + j] for j in range(4)], True, 1, 0.0, False, False, False)
         finals[310 + k], finals[320 + k] = hn, cn
+        y = yk + y if k >= residual_from else yk
     for a, b in zip(got, [y, finals[312], finals[322], finals[313]]):
         assert list(a.shape) == list(b.shape) and float((a - b.float()).abs().max()) <= 5e-3
