@@ -134,10 +134,13 @@ def test_sequence_forward_replays_from_a_graph(ops):
     I, Hs = 64, 256
     # (the first three run one recurrence per XCD: a bidirectional layer of 20 steps in automatic mode, mode 4 by request,
     # and a stack of three layers as a pipeline over the XCDs)
-    for layers, bidir, T, mode in ((1, True, 20, 0), (1, False, 18, 4), (3, False, 21, 0), (2, False, 7, 0), (1, True, 7, 0), (1, False, 7, 0)):
+    # (the last two: residual sums around the upper layers, inside the pipeline and as add launches between the layers)
+    for layers, bidir, T, mode, first_res in ((1, True, 20, 0, None), (1, False, 18, 4, None), (3, False, 21, 0, None), (2, False, 7, 0, None),
+                                              (1, True, 7, 0, None), (1, False, 7, 0, None), (3, False, 21, 0, 1), (3, False, 7, 0, 1)):
         params, x, h0, c0 = workloads.lstm_inputs(7101 + layers + 2 * bidir + T, I, Hs, layers, bidir, T)
         plan = ops.LstmPlan([p.to(DEV) for p in params], True, layers, bidir, T)
         plan.set_mode(mode)
+        plan.set_residual(first_res)
         xd, hd, cd = x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV)
         x2 = (0.5 * xd + 0.25).contiguous()
         eager = {k: [t.clone() for t in plan.forward(v, hd, cd)] for k, v in (("a", xd), ("b", x2))}
@@ -170,6 +173,12 @@ def test_sequence_forward_replays_from_a_graph(ops):
                 for got, w in zip(again, eager["b"]):
                     assert torch.equal(got, w)
     # a pending re-initialisation (mode 3 lays the single chain's entries out differently) is not recorded
+    params, x, h0, c0 = workloads.lstm_inputs(7109, I, Hs, 1, False, 7)
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 1, False, 7)
+    xd, hd, cd = x.reshape(7, I).to(DEV), h0.to(DEV), c0.to(DEV)
+    eager = {"a": [t.clone() for t in plan.forward(xd, hd, cd)]}
+    x_static = xd.clone()
+    out = tuple(torch.zeros_like(t) for t in eager["a"])
     plan.set_mode(3)
     graph2 = torch.cuda.CUDAGraph()
     scratch_out = torch.empty_like(hd)
