@@ -41,6 +41,8 @@ constexpr int kMoeRows1 = kMoeMaxFf / kMoeBlocks / kMoeWaves;     // W1 rows per
 constexpr int kMoeRows2 = kMoeMaxModel / kMoeBlocks / kMoeWaves;  // W2 rows per wavefront: 2
 constexpr int kMoeEntryWords = 8;                     // 8-byte words per entry (64 bytes); the first four carry values
 constexpr unsigned long long kMoeEmpty = ~0ull;
+static_assert(kMoeBlocks <= kMoeThreads, "thread t of a block polls block t's entry");
+static_assert(kMoeRows1 * kMoeWaves <= 16, "a block's hidden values fit the four 8-byte words of its entry");
 
 struct MoeStepArgs {
     const half_t* x;                 // [d_model]
