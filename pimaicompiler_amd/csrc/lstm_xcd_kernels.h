@@ -142,8 +142,8 @@ __device__ __forceinline__ float row16_transpose_sum4(const float (&acc)[4], int
 // that hands the previous step's 32 h values to the layer above adds the layer's own input of that step, which it asked
 // for a step earlier, and stores y from there too (one step late; hn stays h).  Compiled in only for stacks that have such
 // layers.
-template <bool PIPE, bool RES = false>
-__global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p)
+template <bool PIPE, bool RES>
+__device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
 {
     __shared__ __align__(16) half_t hbuf[2][kXcdMaxH];  // h of the previous step, double buffered by step parity
     __shared__ __align__(16) float xring[kXcdWaves][32][4][4];  // per wavefront: [step & 31][gate][unit] projection terms
@@ -499,6 +499,18 @@ __global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p
     // every member has read the counter by now.
     if (rank == 0 && tid == 0)
         __hip_atomic_store(p.g_counter + k, g_base + (unsigned int)T, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <bool PIPE>
+__global__ __launch_bounds__(kXcdThreads) void lstm_xcd_f16_kernel(LstmXcdArgs p)
+{
+    lstm_xcd_body<PIPE, false>(p);
+}
+
+// The pipeline for stacks that have layers with a residual sum.
+__global__ __launch_bounds__(kXcdThreads) void lstm_xcd_res_f16_kernel(LstmXcdArgs p)
+{
+    lstm_xcd_body<true, true>(p);
 }
 
 }  // namespace pimhip

@@ -969,7 +969,7 @@ extern "C" int pimhip_lstm_plan_create(PimHipLstmPlan** plan_out, const void* co
         PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_pipe, lstm_xcd_f16_kernel<true>, kXcdThreads, 0));
         plan->xcd_ok = per_cu >= 1 && per_cu_pipe >= 1;
         int per_cu_res = 0;
-        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_res, lstm_xcd_f16_kernel<true, true>, kXcdThreads, 0));
+        PLAN_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu_res, lstm_xcd_res_f16_kernel, kXcdThreads, 0));
         plan->xcd_res_ok = plan->xcd_ok && per_cu_res >= 1;
     }
     if (plan->xcd_ok) {
@@ -1273,7 +1273,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             a.T = (int)T;
             a.spin_limit = plan->spin_limit;
             if (any_res)
-                lstm_xcd_f16_kernel<true, true><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
+                lstm_xcd_res_f16_kernel<<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
             else
                 lstm_xcd_f16_kernel<true><<<dim3((unsigned)(kXcdCount * members)), dim3(kXcdThreads), 0, s>>>(a);
             PIMHIP_HIP_CHECK(hipGetLastError());
