@@ -436,10 +436,12 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
         const unsigned short flag = (unsigned short)((g & 1u) << 14);
         bool gave_up = false;
         // one step of a bounded wait: true when the caller should stop waiting
+        unsigned long long t_first = 0ull;
         auto give_up_check = [&](unsigned int& spins) {
             ++spins;
             if ((spins & 255u) == 0u) {
                 if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
+                if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
             }
             if (spins >= p.spin_limit) {
                 __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -59,6 +59,21 @@ __device__ __forceinline__ float wave_sum(float v)
     return v;
 }
 
+// Every bounded wait of the kernels here also ends after kWaitTicks of the constant 100 MHz clock, whatever its poll
+// count: where a poll takes far longer than usual (counter collection serialising the memory system, a tool stepping the
+// device), the poll limit alone bounds nothing useful.  Called every 256 unsuccessful polls; `t_first` keeps the time of
+// the first such call.
+static constexpr unsigned long long kWaitTicks = 100000000ull;  // one second
+__device__ __forceinline__ bool wait_clock_expired(unsigned int spins, unsigned long long& t_first)
+{
+    const unsigned long long now = __builtin_amdgcn_s_memrealtime();
+    if (spins <= 256u) {
+        t_first = now;
+        return false;
+    }
+    return now - t_first > kWaitTicks;
+}
+
 __device__ __forceinline__ float sigmoid_f32(float v) { return 1.0f / (1.0f + __expf(-v)); }
 
 // Sigmoid on the hardware exp2 and reciprocal (about 1 ulp each): exact limits 0 and 1 at -+inf, absolute error

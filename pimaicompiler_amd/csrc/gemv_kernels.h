@@ -338,7 +338,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
             float* rec = partial + (long)sl * N + col0;
             float4_t lo, hi;
             unsigned int spins = 0;
+            unsigned long long t_first = 0ull;
             while (true) {
+                if (spins > 0u && (spins & 255u) == 0u && wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
                 if (spins++ >= spin_limit) {
                     __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                     lo = hi = float4_t{0.0f, 0.0f, 0.0f, 0.0f};

@@ -342,6 +342,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
                 const unsigned long long* src =
                     reinterpret_cast<const unsigned long long*>(p.hx + ((long)(gp & 1u) * nb + tid) * kSeqEntryWords);
                 unsigned int spins = 0;
+                unsigned long long t_first = 0ull;
                 while (true) {
                     bool ok = true;
 #pragma unroll
@@ -355,6 +356,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
                     ++spins;
                     if ((spins & 255u) == 0u) {
                         if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
+                        if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
                     }
                     if (spins >= p.spin_limit) {
                         __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -209,14 +209,18 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(MoeStepAr
         }
         bool ok = poll();
         unsigned int spins = 0;
+        unsigned long long t_first = 0ull;
         while (!ok) {
-            if ((spins & 255u) == 255u && __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
+            if (spins > 0u && (spins & 255u) == 0u) {
+                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
+                if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
+            }
             if (spins >= p.spin_limit) {  // (with a limit of 0 a lane whose first look failed gives up without another)
                 __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                 break;
             }
-            ++spins;
+            if (spins != 0xffffffffu) ++spins;
             ok = poll();
         }
         for (int i = 0; i < rows && tid < nb; ++i)
