@@ -539,15 +539,9 @@ def main():
             lib.pimhip_execute_gemv(d_logits.data_ptr(), d_res[1].data_ptr(), d_w.data_ptr(), None, 1024, 32000, 0,
                                     L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, torch.cuda.current_stream().cuda_stream)
         eager_us = timed_us(decoder_step, 100, settle_s=0.3)
-        graph = torch.cuda.CUDAGraph()
-        side = torch.cuda.Stream()
-        side.wait_stream(stream)
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(graph, stream=side):
-                decoder_step()
-        stream.wait_stream(side)
-        torch.cuda.synchronize()
-        graph_us = timed_us(graph.replay, 100)
+        # (replayed: sixteen steps per graph, as a decoding loop would record them; two graph launches are 15 us apart on
+        # the device whatever they hold, which a graph of one step would add to every step)
+        graph_us = graph_timed_us(lambda _s: decoder_step(), 16)
         other["decoder_step_8_launches"] = {"issued_one_by_one_us": round(eager_us, 2), "hip_graph_replay_us": round(graph_us, 2),
                                              "bytes": 4 * 4096 * 1024 * 2 + (4096 * 1024 + 3 * 4096 * 2048) * 2 + 32000 * 1024 * 2}
         # the same step as ONE launch (pimhip_decoder_step): same weights, state, attention weights and classifier; the
@@ -568,14 +562,7 @@ def main():
         if not fused_err <= 5e-3:
             raise RuntimeError(f"fused decoder step differs from the operator-by-operator step by {fused_err}")
         fused_eager_us = timed_us(fstep, 200, settle_s=0.3)
-        fgraph = torch.cuda.CUDAGraph()
-        side.wait_stream(stream)
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(fgraph, stream=side):
-                fstep(torch.cuda.current_stream())
-        stream.wait_stream(side)
-        torch.cuda.synchronize()
-        fused_graph_us = timed_us(fgraph.replay, 200)
+        fused_graph_us = graph_timed_us(lambda s_: fstep(s_), 16)
         fplan.status()
 
         def reproject():
