@@ -110,6 +110,9 @@ class AtenLSTM1Layer(NNLayer):          # ir/include/layers/aten_lstm1_layer.h
     custom_opt_number: int = 0
     custom_cat_mem_id: int = -1
     output_cat_mem_id: int = -1
+    # Not in the reference's record: set by a graph rewrite that has folded the aten::add layers of a residual stack
+    # (out = lstm(in) + in from this layer of the record on) into it; negative = no such sums.
+    first_residual_layer: int = -1
 
 
 @dataclass
@@ -505,7 +508,8 @@ def execute_aten_lstm1(layer, executor):
         raise NNRuntimeException("lstm needs three output ids")
     out = _gnmt_lstm_destinations(layer, executor, x, out_ids, hx[0].size(-1), num_layers, bool(bidirectional), bool(batch_first))
     y, hy, cy = ops.aten_lstm1(x, tuple(hx), layer.param_vector, bool(has_biases), num_layers, dropout, bool(train),
-                               bool(bidirectional), bool(batch_first), out=out)
+                               bool(bidirectional), bool(batch_first), out=out,
+                               first_residual_layer=layer.first_residual_layer if layer.first_residual_layer >= 0 else None)
     for i, v in zip(out_ids, (y, hy, cy)):
         executor.update_blob(i, DataType.TENSOR, v)
 

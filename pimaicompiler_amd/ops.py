@@ -849,10 +849,12 @@ def prepare_lstm(params, has_biases, num_layers, bidirectional, max_seq_len=64):
 
 
 def aten_lstm1(input, hx, params, has_biases, num_layers, dropout, train, bidirectional, batch_first, stream=None,
-               out=None):
+               out=None, first_residual_layer=None):
     """atenLstm1: padded-sequence aten::lstm, batch 1 (the reference's GPU LSTM hard-codes batch 1,
     miopen_ops_executor.cpp:117).  dropout is ignored as in the reference (aten_ops.cpp:333); train must be false.
-    Returns (output, hy, cy) shaped like at::lstm's results."""
+    Returns (output, hy, cy) shaped like at::lstm's results.  `first_residual_layer` (not part of aten::lstm): layers from
+    that one on return and hand up h + their own input (LstmPlan.set_residual), the wiring a fused stack of GNMT's
+    lstm + add layers has."""
     del dropout
     if train:
         raise NNRuntimeException("training mode is not part of this inference path")
@@ -864,6 +866,7 @@ def aten_lstm1(input, hx, params, has_biases, num_layers, dropout, train, bidire
     T = input.size(1) if batch_first else input.size(0)
     h0, c0 = hx[0], hx[1]
     plan = _plan_for(list(params), has_biases, num_layers, bidirectional, T)
+    plan.set_residual(first_residual_layer)  # (a cached plan serves calls with and without: set on every call)
     y, hn, cn = plan.forward(input.reshape(T, input.size(2)), h0, c0, stream, out=out)
     D, H = plan.num_dirs, plan.hidden
     seq = y.view(1, T, D * H) if batch_first else y.view(T, 1, D * H)

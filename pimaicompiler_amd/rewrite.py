@@ -550,16 +550,6 @@ def fuse_lstm_stack(g: Graph):
     return g
 
 
-def _stack_plan(op: Op, ops, params, n, T):
-    """The plan of a pimhip::lstm_stack op, kept on the op (its weights are constants of the graph)."""
-    plan = op.attrs.get("_plan")
-    if plan is None or plan.max_seq_len < T or any(p.data_ptr() != q.data_ptr() for p, q in zip(plan.params, params)):
-        plan = ops.LstmPlan(list(params), True, n, False, max(T, 16))
-        plan.set_residual(op.attrs["first_residual_layer"])
-        op.attrs["_plan"] = plan
-    return plan
-
-
 def _as_row_major_weight(t):
     """For a [..1.., in, out] tensor that is a transposed view of a dense row-major [out, in] matrix: that matrix."""
     if t.dim() < 2 or any(d != 1 for d in t.shape[:-2]) or t.dtype != torch.float16:
@@ -664,10 +654,9 @@ def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0", same_sent
             continue
         elif op.type == "pimhip::lstm_stack":
             n = op.attrs["num_layers"]
-            T = a[0].size(0)
-            plan = _stack_plan(op, ops, a[3:3 + 4 * n], n, T)
-            y, hn, cn = plan.forward(a[0].reshape(T, a[0].size(2)), a[1], a[2])
-            env[op.outputs[0]], env[op.outputs[1]], env[op.outputs[2]] = y.view(T, 1, -1), hn.view(n, 1, -1), cn.view(n, 1, -1)
+            y, hn, cn = ops.aten_lstm1(a[0], (a[1], a[2]), a[3:3 + 4 * n], True, n, 0.0, False, False, False,
+                                       first_residual_layer=op.attrs["first_residual_layer"])
+            env[op.outputs[0]], env[op.outputs[1]], env[op.outputs[2]] = y, hn, cn
             continue
         elif op.type == "aten::lstm":
             n = op.attrs.get("num_layers", 1)

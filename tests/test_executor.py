@@ -368,6 +368,32 @@ def test_lstm1_layer_with_flags_from_blobs(ops, bidirectional, num_layers):
 
 
 @pytest.mark.gpu
+def test_lstm1_layer_with_residual_sums_folded_in(ops):
+    """A record a graph rewrite has folded GNMT's aten::add layers into: three layers, sums around the upper two, against
+    one at::lstm and one at::add per layer on LibTorch CPU."""
+    T, H = 24, 256
+    params, x, h0, c0 = workloads.lstm_inputs(13, 2 * H, H, 3, False, T)
+    ex = E.StreamExecutor([], device=0)
+    _blobs(ex, b0=x.to(DEV), b1=[h0.to(DEV), c0.to(DEV)])
+    layer = E.AtenLSTM1Layer(LayerType.ATENLSTM1, 0, [0, 1], [20, 21, 22], has_biases=1, num_layers=3, dropout=0.0, train=0,
+                             bidirectional=0, batch_first=0, param_vector=[p.to(DEV) for p in params], first_residual_layer=1)
+    E.execute_aten_lstm1(layer, ex)
+    cur, hs = x, []
+    for l in range(3):
+        y, hn, _ = torch.lstm(cur, (h0[l:l + 1], c0[l:l + 1]), params[4 * l:4 * l + 4], True, 1, 0.0, False, False, False)
+        hs.append(hn)
+        cur = y + cur if l >= 1 else y
+    got = [ex.find_blob(i)[1] for i in (20, 21, 22)]
+    assert list(got[0].shape) == [T, 1, H]
+    assert maxabs(got[0], cur) <= TOL_LSTM and maxabs(got[1], torch.cat(hs, 0)) <= TOL_LSTM
+    # the same record without the attribute is a plain stack again (the cached plan is told so on every call)
+    layer.first_residual_layer = -1
+    E.execute_aten_lstm1(layer, ex)
+    ty, _, _ = torch.lstm(x, (h0, c0), params, True, 3, 0.0, False, False, False)
+    assert maxabs(ex.find_blob(20)[1], ty) <= TOL_LSTM
+
+
+@pytest.mark.gpu
 def test_lstm2_layer_on_the_rnnt_feature_shape(ops):
     params, x, h0, c0 = workloads.lstm_inputs(12, 240, 256, 2, False, 21)
     ex = E.StreamExecutor([], device=0)
