@@ -29,6 +29,23 @@ def test_library_loads_and_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_header_is_plain_c_and_links_against_the_library(tmp_path):
+    """include/pimhip.h is what a cgo / JNI / ctypes binding reads: it has to compile as C99 with nothing but the standard
+    headers, and a C program that names every declared function has to link against libpimhip.so."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "uses_every_entry_point.c"
+    names = declared_functions()
+    src.write_text('#include "pimhip.h"\n#include <stdio.h>\nint main(void)\n{\n    const void* table[] = {\n' +
+                   "".join(f"        (const void*)&{n},\n" for n in names) +
+                   '    };\n    printf("%d\\n", (int)(sizeof(table) / sizeof(table[0])));\n    return 0;\n}\n')
+    exe = tmp_path / "uses_every_entry_point"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                    L.LIB_PATH, "-Wl,-rpath," + os.path.dirname(L.LIB_PATH), "-Wl,--allow-shlib-undefined"], check=True, capture_output=True)
+
+
 def test_last_error_is_a_string():
     lib = L.load()
     assert isinstance(lib.pimhip_last_error(), bytes)
