@@ -486,6 +486,31 @@ def main():
             "max_abs_diff_to_the_three_gemvs": round(float((y_one.float() - yo.float()).abs().max()), 6),
             "expert": int(e_one.item())}
         moe_plan.status()
+        # RNNT joint network, one (t, u) step: relu(W1[512, 1344] . cat(f[1024], g[320]) + b1), then W2[29, 512] . + b2.  The
+        # reference's RemoveCatForAddmm makes two dependent products of the first layer (three launches per step); one launch
+        # that reads f and g where they lie leaves two.
+        jw1, jb1 = (0.03 * torch.randn(512, 1344, device=dev)).half(), (0.05 * torch.randn(512, device=dev)).half()
+        jw2, jb2 = (0.05 * torch.randn(29, 512, device=dev)).half(), (0.05 * torch.randn(29, device=dev)).half()
+        jw1a, jw1b = jw1[:, :1024].contiguous(), jw1[:, 1024:].contiguous()
+        jf, jg = torch.randn(1024, device=dev).half(), torch.randn(320, device=dev).half()
+        jmid, jhid, jout = (torch.empty(n_, dtype=torch.float16, device=dev) for n_ in (512, 512, 29))
+
+        def joint_three(s_h=sh):
+            lib.pimhip_execute_gemv(jmid.data_ptr(), jf.data_ptr(), jw1a.data_ptr(), jb1.data_ptr(), 1024, 512, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, s_h)
+            lib.pimhip_execute_gemv(jhid.data_ptr(), jg.data_ptr(), jw1b.data_ptr(), jmid.data_ptr(), 320, 512, 0, L.PIMHIP_ACT_RELU, L.PIMHIP_W_X_I, s_h)
+            lib.pimhip_execute_gemv(jout.data_ptr(), jhid.data_ptr(), jw2.data_ptr(), jb2.data_ptr(), 512, 29, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, s_h)
+
+        def joint_two(s_h=sh):
+            lib.pimhip_execute_gemv_cat2(jhid.data_ptr(), jf.data_ptr(), 1024, jg.data_ptr(), 320, jw1.data_ptr(), jb1.data_ptr(), 512, 0,
+                                         L.PIMHIP_ACT_RELU, s_h)
+            lib.pimhip_execute_gemv(jout.data_ptr(), jhid.data_ptr(), jw2.data_ptr(), jb2.data_ptr(), 512, 29, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, s_h)
+        joint_three()
+        ref_out = jout.clone()
+        joint_two()
+        torch.cuda.synchronize()
+        other["rnnt_joint_step"] = {"three_launches_us": round(graph_timed_us(joint_three, 32), 3),
+                                    "two_launches_us": round(graph_timed_us(joint_two, 32), 3),
+                                    "max_abs_diff": round(float((jout.float() - ref_out.float()).abs().max()), 6)}
         # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
         big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
         big_c = torch.empty_like(big_a)

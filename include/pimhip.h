@@ -105,6 +105,14 @@ int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* other_shape4
 int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
                         int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
 
+/* out[out_w] = act(weight[out_w, in1_w + in2_w] . cat(in1, in2) + bias) without the concatenation (order W_X_I): in1 and
+ * in2 lie apart, as the encoder frame and the prediction that the RNNT joint network's first layer reads do.  Replaces the
+ * pair of dependent products RemoveCatForAddmm makes of such a layer
+ * (compiler/source/frontend/optimizer/remove_cat_for_addmm.cpp:46-191) by one launch on the whole weight.  in1_w, in2_w and
+ * ld_weight (0 = dense) must be multiples of 8 and in1, in2, weight 16-byte aligned (PIMHIP_ERR_UNSUPPORTED otherwise). */
+int pimhip_execute_gemv_cat2(void* out, const void* in1, int64_t in1_w, const void* in2, int64_t in2_w, const void* weight,
+                             const void* bias, int64_t out_w, int64_t ld_weight, int act, void* stream);
+
 /* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  Same arguments, result and bits as pimhip_execute_gemv,
  * but the partial sums of a sliced I_X_W product go through a 256 KiB array that is part of the library's

@@ -16,6 +16,7 @@ from .ops import (  # noqa: F401
     custom_aten_addmm,
     custom_aten_matmul,
     aten_linear,
+    aten_linear_cat2,
     aten_bmm,
     aten_add,
     aten_lstm1,

@@ -26,10 +26,13 @@ namespace pimhip
 // ks*64 + lane, then strides by 64*KS), so one block covers (WAVES / KS) * R rows.  Each lane
 // keeps U chunks per row in flight: R*U independent 16-byte weight loads per lane per iteration.
 // ---------------------------------------------------------------------------------------------
-template <int R, int U, int WAVES, int KS>
+// SPLIT: x is the concatenation of two vectors that lie apart (x: the first split_chunks 16-byte pieces, x2: the rest);
+// compiled out of every other instance.
+template <int R, int U, int WAVES, int KS, bool SPLIT = false>
 __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, const half_t* __restrict__ x,
                                                  const half_t* __restrict__ bias, half_t* __restrict__ y, int N,
-                                                 int K, long ldw, int relu, int block)
+                                                 int K, long ldw, int relu, int block,
+                                                 const half_t* __restrict__ x2 = nullptr, int split_chunks = 0)
 {
     static_assert(WAVES % KS == 0, "KS must divide WAVES");
     constexpr int RG = WAVES / KS;  // row groups per block
@@ -51,6 +54,8 @@ __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, c
         wrow[r] = reinterpret_cast<const half8_t*>(W + row * ldw);
     }
     const half8_t* xv = reinterpret_cast<const half8_t*>(x);
+    const half8_t* xv2 = SPLIT ? reinterpret_cast<const half8_t*>(x2) - split_chunks : nullptr;  // (indexed from split_chunks on)
+    auto x_at = [&](int c) { return (SPLIT && c >= split_chunks) ? xv2[c] : xv[c]; };
     const int nchunks = K >> 3;
     constexpr int STEP = 64 * KS;
 
@@ -65,7 +70,7 @@ __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, c
             for (int r = 0; r < R; ++r) wr[r][u] = load_stream(wrow[r] + c + u * STEP);
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) xr[u] = xv[c + u * STEP];
+        for (int u = 0; u < U; ++u) xr[u] = x_at(c + u * STEP);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -77,7 +82,7 @@ __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, c
         half8_t wr[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) wr[r] = load_stream(wrow[r] + c);
-        const half8_t xr = xv[c];
+        const half8_t xr = x_at(c);
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[r] = dot8(wr[r], xr, acc[r]);
     }
@@ -124,6 +129,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_kernel(const half_t* _
                                                                  int relu)
 {
     gemv_mv_f16_body<R, U, WAVES, KS>(W, x, bias, y, N, K, ldw, relu, blockIdx.x);
+}
+
+// y = act(W . cat(x1, x2) + bias) without the concatenation: the second operand of the RNNT joint network's first layer
+// is cat(encoder frame, prediction), which the reference either materialises or splits the product over
+// (compiler/source/frontend/optimizer/remove_cat_for_addmm.cpp:46-191: two dependent launches).
+template <int R, int U, int WAVES, int KS>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mv_cat2_f16_kernel(const half_t* __restrict__ W,
+                                                                      const half_t* __restrict__ x1,
+                                                                      const half_t* __restrict__ x2, int split_chunks,
+                                                                      const half_t* __restrict__ bias,
+                                                                      half_t* __restrict__ y, int N, int K, long ldw,
+                                                                      int relu)
+{
+    gemv_mv_f16_body<R, U, WAVES, KS, true>(W, x1, bias, y, N, K, ldw, relu, blockIdx.x, x2, split_chunks);
 }
 
 // Several independent MV GEMVs in one launch (sibling projections that the reference issues on separate

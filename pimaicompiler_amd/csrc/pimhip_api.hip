@@ -394,6 +394,46 @@ extern "C" int pimhip_execute_gemv(void* out, const void* in, const void* weight
     return execute_gemv(out, in, weight, bias, in_w, out_w, ld_weight, act, order, stream, false);
 }
 
+extern "C" int pimhip_execute_gemv_cat2(void* out, const void* in1, int64_t in1_w, const void* in2, int64_t in2_w,
+                                        const void* weight, const void* bias, int64_t out_w, int64_t ld_weight, int act,
+                                        void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!out || !in1 || !in2 || !weight) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "out, in1, in2 and weight must be non-null");
+    if (in1_w < 1 || in2_w < 1 || out_w < 1) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "in1_w=%lld in2_w=%lld out_w=%lld must be positive",
+                                                         (long long)in1_w, (long long)in2_w, (long long)out_w);
+    if (act != PIMHIP_ACT_NONE && act != PIMHIP_ACT_RELU) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "act=%d", act);
+    const int64_t K = in1_w + in2_w;
+    const int64_t ldw = ld_weight > 0 ? ld_weight : K;
+    if (ldw < K) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "ld_weight=%lld is less than in1_w + in2_w=%lld", (long long)ldw, (long long)K);
+    if ((in1_w & 7) || (in2_w & 7) || (ldw & 7) || !aligned16(in1) || !aligned16(in2) || !aligned16(weight))
+        return fail(PIMHIP_ERR_UNSUPPORTED, "both widths and the row pitch must be multiples of 8 and in1, in2, weight 16-byte aligned: "
+                                            "concatenate and call pimhip_execute_gemv otherwise");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int relu = act == PIMHIP_ACT_RELU;
+    const int N = (int)out_w;
+    const int split = (int)(in1_w >> 3);
+    // (the launch shapes of gemv_mv)
+    if (out_w < 1024) {
+        if (K >= 2048)
+            gemv_mv_cat2_f16_kernel<1, 4, 4, 4><<<N, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
+                                                                    (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+        else
+            gemv_mv_cat2_f16_kernel<1, 2, 4, 4><<<N, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
+                                                                    (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+    } else if (K >= 4096) {
+        gemv_mv_cat2_f16_kernel<2, 4, 4, 4><<<(N + 1) / 2, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
+                                                                          (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+    } else {
+        gemv_mv_cat2_f16_kernel<2, 2, 4, 2><<<(N + 3) / 4, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
+                                                                          (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+    }
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
 extern "C" int pimhip_execute_gemv_static(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
                                           int64_t out_w, int64_t ld_weight, int act, int order, void* stream)
 {

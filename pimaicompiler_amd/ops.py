@@ -305,6 +305,31 @@ def aten_linear(input_tensor, weight, bias=None, act_type="none", stream=None):
     return y.view(list(input_tensor.shape[:-1]) + [out_w])
 
 
+def aten_linear_cat2(input1, input2, weight, bias=None, act_type="none", stream=None):
+    """y = act(W[out, in1 + in2] . cat(input1, input2) + b) for two batch-1 inputs that lie apart, without concatenating
+    them (pimhip_execute_gemv_cat2): the first layer of the RNNT joint network, which the reference turns into two
+    dependent addmm launches (RemoveCatForAddmm, compiler/source/frontend/optimizer/remove_cat_for_addmm.cpp:46-191).
+    Shapes the launch does not take (widths not multiples of 8, more than one row) are concatenated and go through
+    aten_linear."""
+    _require_half_cuda(input1, input2, weight, bias)
+    out_w, in_w = weight.shape
+    n1, n2 = input1.numel(), input2.numel()
+    w = weight if weight.stride(1) == 1 else weight.contiguous()
+    if n1 + n2 != in_w or (n1 & 7) or (n2 & 7) or (w.stride(0) & 7) or input1.shape[:-1] != input2.shape[:-1]:
+        return aten_linear(torch.cat([input1, input2], -1), weight, bias, act_type, stream)
+    _ensure_init(w)
+    x1, x2 = input1.contiguous(), input2.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()
+        if bias.numel() != out_w:
+            raise NNRuntimeException(f"bias has {bias.numel()} elements, the GEMV produces {out_w}")
+    out = torch.empty(out_w, dtype=torch.float16, device=w.device)
+    _check(L.load().pimhip_execute_gemv_cat2(out.data_ptr(), x1.data_ptr(), n1, x2.data_ptr(), n2, w.data_ptr(),
+                                             bias.data_ptr() if bias is not None else None, out_w,
+                                             w.stride(0) if out_w > 1 else in_w, _act_code(act_type), _stream_handle(stream)))
+    return out.view(list(input1.shape[:-1]) + [out_w])
+
+
 def execute_gemv_group(inputs, weights, biases=None, act_types=None, stream=None):
     """N sibling MV GEMVs (y_i = act_i(W_i . x_i + b_i)) in one launch.
 

@@ -20,6 +20,9 @@ one join and hang off one common start are collected into a single `multi_stream
 here where the reference gives each sibling its own stream.  `execute` runs a graph through the operator layer
 (pimaicompiler_amd.ops) on the GPU.
 
+`gemv_over_cat` is an alternative to remove_cat_for_addmm: the product over cat([f, g]) stays ONE op on the whole weight
+that reads f and g where they lie (one launch instead of the reference's two dependent ones).
+
 `fuse_decoder_step` has no counterpart in the reference: it collects the per-token chain of the GNMT decoder — the
 seq_len-1 `aten::lstm` cells that read cat(previous output, context), the residual `aten::add`s, the attention `aten::bmm`
 and the classifier — which the reference's interpreter runs operator by operator (executeAtenLSTM1 / executeAtenBmm /
@@ -182,6 +185,39 @@ def lower_to_hot_path(g: Graph):
         op.attrs = {"act_type": op.attrs.get("act_type", "none"), "has_bias": bias is not None}
         g.ops.remove(t_in)
         g.ops.remove(t_out)
+    return g
+
+
+def gemv_over_cat(g: Graph):
+    """linear(cat([f, g], last dim), Wconst, b) [-> relu]  becomes one `pimhip::gemv_cat2` op on the whole weight
+    (ops.aten_linear_cat2: one launch that reads f and g where they lie), where the reference's RemoveCatForAddmm makes two
+    dependent addmm launches on the two column blocks of the weight (remove_cat_for_addmm.cpp:46-191).  Run it before
+    apply_reference_passes; what it leaves alone (a cat with another reader, more than two parts, a weight that is not a
+    constant) goes the reference's way."""
+    for lst in [op for op in g.ops if op.type == "prim::ListConstruct" and len(op.inputs) == 2]:
+        users = g.consumers(lst.outputs[0])
+        if len(users) != 1 or users[0].type != "aten::cat" or users[0].attrs.get("dim", -1) not in (-1,) or lst.outputs[0] in g.outputs:
+            continue
+        cat = users[0]
+        users = g.consumers(cat.outputs[0])
+        if len(users) != 1 or users[0].type != "aten::linear" or users[0].inputs[0] != cat.outputs[0] or cat.outputs[0] in g.outputs:
+            continue
+        lin = users[0]
+        if not g.is_constant(lin.inputs[1]) or g.constants[lin.inputs[1]] is None or g.constants[lin.inputs[1]].dim() != 2:
+            continue
+        has_bias = len(lin.inputs) > 2 and not (g.is_constant(lin.inputs[2]) and g.constants[lin.inputs[2]] is None)
+        out, act = lin.outputs[0], "none"
+        nxt = g.consumers(out)
+        relu = nxt[0] if len(nxt) == 1 and nxt[0].type == "aten::relu" and out not in g.outputs else None
+        if relu is not None:
+            out, act = relu.outputs[0], "aten::relu"
+            g.ops.remove(relu)
+        lin.type = "pimhip::gemv_cat2"
+        lin.inputs = [lst.inputs[0], lst.inputs[1], lin.inputs[1]] + ([lin.inputs[2]] if has_bias else [])
+        lin.outputs = [out]
+        lin.attrs = {"act_type": act, "has_bias": has_bias}
+        g.ops.remove(lst)
+        g.ops.remove(cat)
     return g
 
 
@@ -622,6 +658,8 @@ def execute(g: Graph, feeds: Dict[int, torch.Tensor], device="cuda:0", same_sent
             r = ops.custom_aten_matmul(a[0], a[1])
         elif op.type == "pimhip::gemv":
             r = ops.aten_linear(a[0], a[1], a[2] if op.attrs["has_bias"] else None, act_type=op.attrs["act_type"])
+        elif op.type == "pimhip::gemv_cat2":
+            r = ops.aten_linear_cat2(a[0], a[1], a[2], a[3] if op.attrs["has_bias"] else None, act_type=op.attrs["act_type"])
         elif op.type == "multi_stream":
             subs = op.attrs["layers"]
             if all(m.type == "pimhip::gemv" for m in subs):

@@ -229,6 +229,41 @@ def test_sliced_vm_product_that_gives_up_is_reported_and_the_workspace_recovers(
     ops.synchronize_and_check()
 
 
+@pytest.mark.parametrize("n1,n2,out_w,bias,act", [(1024, 320, 512, True, "aten::relu"), (8, 8, 1, False, "none"), (4096, 64, 2000, True, "none"),
+                                                  (136, 4104, 77, True, "aten::relu"), (512, 512, 4096, False, "none")])
+def test_gemv_over_two_separate_inputs_matches_libtorch_on_their_concatenation(ops, n1, n2, out_w, bias, act):
+    g = torch.Generator().manual_seed(n1 + n2)
+    W = (torch.randn(out_w, n1 + n2, generator=g) / (n1 + n2) ** 0.5).half()
+    b = (0.1 * torch.randn(out_w, generator=g)).half() if bias else None
+    x1, x2 = torch.randn(1, n1, generator=g).half(), torch.randn(1, n2, generator=g).half()
+    want = torch.nn.functional.linear(torch.cat([x1, x2], -1), W, b)
+    want = torch.relu(want) if act == "aten::relu" else want
+    y = ops.aten_linear_cat2(x1.to(DEV), x2.to(DEV), W.to(DEV), b.to(DEV) if bias else None, act_type=act)
+    assert list(y.shape) == [1, out_w] and maxabs(y, want.numpy()) <= GEMV_TOL
+    # the same bits as the one-input launch on the concatenation (same kernel shape, same order of sums)
+    y1 = ops.aten_linear(torch.cat([x1, x2], -1).to(DEV), W.to(DEV), b.to(DEV) if bias else None, act_type=act)
+    assert torch.equal(y, y1)
+    # a weight that is a column block of a wider matrix (row pitch larger than the two widths together)
+    wide = torch.zeros(out_w, n1 + n2 + 24, dtype=torch.float16)
+    wide[:, :n1 + n2] = W
+    yv = ops.aten_linear_cat2(x1.to(DEV), x2.to(DEV), wide.to(DEV)[:, :n1 + n2], b.to(DEV) if bias else None, act_type=act)
+    assert torch.equal(yv, y)
+
+
+def test_gemv_over_two_inputs_with_widths_the_launch_does_not_take(ops):
+    g = torch.Generator().manual_seed(3)
+    W = (0.05 * torch.randn(40, 12 + 20, generator=g)).half()
+    x1, x2 = torch.randn(1, 12, generator=g).half(), torch.randn(1, 20, generator=g).half()
+    y = ops.aten_linear_cat2(x1.to(DEV), x2.to(DEV), W.to(DEV))          # 12 is no multiple of 8: concatenated, then one GEMV
+    assert maxabs(y, torch.nn.functional.linear(torch.cat([x1, x2], -1), W).numpy()) <= GEMV_TOL
+    from pimaicompiler_amd import _lib as L
+    lib = L.load()
+    out = torch.empty(40, dtype=torch.float16, device=DEV)
+    rc = lib.pimhip_execute_gemv_cat2(out.data_ptr(), x1.to(DEV).data_ptr(), 12, x2.to(DEV).data_ptr(), 20, W.to(DEV).data_ptr(), None, 40, 0,
+                                      L.PIMHIP_ACT_NONE, None)
+    assert rc == L.PIMHIP_ERR_UNSUPPORTED
+
+
 def test_moe_ffn_decode_step_matches_libtorch(ops, golden):
     import importlib.util, os
     spec = importlib.util.spec_from_file_location("make_golden", os.path.join(os.path.dirname(__file__), "golden", "make_golden.py"))

@@ -51,6 +51,21 @@ def test_remove_cat_splits_the_weight_by_columns():
     assert 10 not in g.constants and second.outputs == [4]
 
 
+def test_product_over_a_cat_becomes_one_op():
+    g, f, h = joint_graph()
+    R.gemv_over_cat(g)
+    assert g.types() == ["pimhip::gemv_cat2"]
+    op = g.ops[0]
+    assert op.inputs == [0, 1, 10, 11] and op.outputs == [5] and op.attrs == {"act_type": "aten::relu", "has_bias": True}
+    R.apply_reference_passes(g)                       # nothing left for the reference's passes to split
+    assert g.types() == ["pimhip::gemv_cat2"]
+    # a cat that something else reads as well is left to the reference's way
+    g, f, h = joint_graph()
+    g.outputs.append(3)
+    R.gemv_over_cat(g)
+    assert g.types() == ["prim::ListConstruct", "aten::cat", "aten::linear", "aten::relu"]
+
+
 def test_matmul_swap_and_fusion_guards():
     c = {10: torch.randn(8, 8).half(), 11: torch.randn(2, 8, 8).half()}
     g = R.Graph([R.Op("aten::matmul", [0, 10], [1]), R.Op("aten::matmul", [0, 11], [2]), R.Op("aten::matmul", [1, 2], [3])], [0], [3], c, 20)
@@ -105,6 +120,11 @@ def test_rewritten_graphs_compute_what_eager_libtorch_computes(ops):
         assert list(y.shape) == [1, 512], stage
         # two roundings (the split product is rounded to fp16 in between): 2 x 2e-3
         assert float((y.float().cpu() - want).abs().max()) <= 4e-3, stage
+    # the same layer as one launch that reads f and g where they lie: one rounding
+    g, _, _ = joint_graph()
+    R.gemv_over_cat(g)
+    (y,) = R.execute(g, {0: f, 1: gg}, DEV)
+    assert list(y.shape) == [1, 512] and float((y.float().cpu() - want).abs().max()) <= 2e-3
 
 
 def attention_projection_graph(seed=3, d=512, n=4, constant_weights=True):
