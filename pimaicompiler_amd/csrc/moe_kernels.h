@@ -182,8 +182,10 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(MoeStepAr
     half8_t w2r[kMoeRows2][kMoeFC];
     {
         const int first = tid * p.rpb1;               // block tid's first row
-        const int rows = min(p.rpb1, p.d_ff - first);  // <= 0: that block has no row, nothing to wait for
-        const int words = (tid < nb && rows > 0) ? (rows + 3) >> 2 : 0;
+        const int rows = min(p.rpb1, p.d_ff - first);  // <= 0: that block has no row
+        // A block without rows publishes zeros and is waited for all the same: block 0 advances the launch count at its end,
+        // and no block may still be on its way to reading it then.
+        const int words = tid < nb ? (rows > 0 ? (rows + 3) >> 2 : 1) : 0;
         const unsigned long long* slot = p.hx + ((long)set * nb + tid) * kMoeEntryWords;
         unsigned long long got[4] = {0ull, 0ull, 0ull, 0ull};
         auto poll = [&]() {
