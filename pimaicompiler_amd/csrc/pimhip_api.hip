@@ -1181,7 +1181,11 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     // take longer to load the weights and the pipeline has to fill, which shorter sequences do not win back.)
     const bool xcd_pays = (D == 2 && T >= 16) || (D == 1 && L == 1 && T >= (H > 512 ? 64 : 16)) ||
                           (D == 1 && L >= 2 && T >= (L >= 3 ? 16 : 32));
-    const bool use_xcd = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && (plan->mode == 4 || (plan->mode == 0 && xcd_pays));
+    // (a stack with residual sums needs the pipeline kernel that makes them; where that one is not resident the stack runs
+    // layer by layer on the other paths)
+    const bool res_pipeline_missing = D == 1 && L >= 2 && plan->first_residual_layer < L && !plan->xcd_res_ok;
+    const bool use_xcd = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && !res_pipeline_missing &&
+                         (plan->mode == 4 || (plan->mode == 0 && xcd_pays));
     const bool use_seq = !use_xcd && T >= 2 && T + kSeqMaxChains <= kSeqMaxT &&
                          (plan->mode == 2 || plan->mode == 3 || (plan->mode == 0 && plan->seq_kernel_ok));
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
