@@ -187,3 +187,54 @@ def test_moe_step_wait_that_gives_up_is_reported_once_and_recovered_from(ops):
     y, _, expert = plan.forward(x.to(DEV))    # the exchange buffer is refilled before this launch
     plan.status()
     assert int(expert.item()) == want[1] and maxabs(y, want[3]) <= TOL
+
+
+def test_resident_kernels_of_three_kinds_on_three_streams_take_turns(ops):
+    """The mixture-of-experts step, the decoder step and a pipelined LSTM sequence all need their blocks resident together.
+    Issued back to back on three streams without any synchronisation between them, the library orders them one after
+    another: every result equals the one computed alone, and no wait gives up."""
+    from pimaicompiler_amd import workloads
+    E, d_model, d_ff, H, T = 8, 768, 3072, 512, 24
+    g, Wr, br, W1, b1, W2, b2 = make(21, E, d_model, d_ff, False, scale=0.02)
+    moe = ops.MoePlan((Wr.to(DEV), None), dev(W1), dev(W2))
+    xm = torch.randn(d_model, generator=g).half().to(DEV)
+    ym = torch.empty(d_model, dtype=torch.float16, device=DEV)
+    moe_step = moe.bind(xm, ym)
+    dparams = []
+    for k in range(3):
+        dparams += [p.to(DEV) for p in workloads.lstm_inputs(300 + k, H if k == 0 else 2 * H, H, 1, False, 1)[0]]
+    dec = ops.DecoderPlan(dparams, True, 3)
+    xd = torch.randn(H, generator=g).half().to(DEV)
+    hs = [(0.3 * torch.randn(H, generator=g)).half().to(DEV) for _ in range(3)]
+    cs = [(0.3 * torch.randn(H, generator=g)).half().to(DEV) for _ in range(3)]
+    hn, cn = [torch.empty_like(t) for t in hs], [torch.empty_like(t) for t in cs]
+    ctx = torch.randn(H, generator=g).half().to(DEV)
+    dec_step = dec.bind(xd, hs, cs, ctx=ctx, hn=hn, cn=cn)
+    lp, lx, lh0, lc0 = workloads.lstm_inputs(310, H, H, 3, False, T)
+    lstm = ops.LstmPlan([p.to(DEV) for p in lp], True, 3, False, T)
+    lstm.set_mode(4)
+    lx, lh0, lc0 = lx.reshape(T, H).to(DEV), lh0.to(DEV), lc0.to(DEV)
+    # alone
+    moe_step()
+    dec_step()
+    want_l = [t.clone() for t in lstm.forward(lx, lh0, lc0)]
+    torch.cuda.synchronize()
+    want_m, want_h = ym.clone(), [t.clone() for t in hn]
+    s1, s2, s3 = torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.Stream()
+    for s in (s1, s2, s3):
+        s.wait_stream(torch.cuda.current_stream())
+    ym.zero_()
+    for t in hn:
+        t.zero_()
+    outs = tuple(torch.zeros_like(t) for t in want_l)
+    for _ in range(12):
+        moe_step(s1.cuda_stream)
+        dec_step(s2.cuda_stream)
+        lstm.forward(lx, lh0, lc0, s3.cuda_stream, out=outs)
+    torch.cuda.synchronize()
+    moe.status()
+    dec.status()
+    lstm.status()
+    assert torch.equal(ym, want_m)
+    assert all(torch.equal(a, b) for a, b in zip(hn, want_h))
+    assert all(torch.equal(a, b) for a, b in zip(outs, want_l))
