@@ -433,22 +433,50 @@ def main():
         # device's (64 launches replayed from a HIP graph), the second what a Python caller sees
         other["gemv_1024x1024_us"] = round(graph_timed_us(c1_launch, 64), 3)
         other["gemv_1024x1024_issued_from_python_us"] = round(timed_us(c1_launch, 200), 3)
-        # the same GEMV through the C++ operator with the reference's signature (customAtenAddmm: shape logic, output
-        # allocation, launch), 200 calls in a row from C++: the host's cost per call, and the rate the GPU sees
+        # The per-token calls of a decoding loop through the C++ operators with the reference's signatures: what one call
+        # costs the host thread (shape logic, output allocation, launch; 300 calls in a row from C++, nothing synchronises
+        # inside the loop) beside what its kernels take on the device (the same launches replayed from a HIP graph).
         try:
             from pimaicompiler_amd import _aten_ops_pimhip as cpp_ops
-            cpp_ops.initialize(0)
-            c1_w_t, c1_x2 = c1_pool[0].t(), c1_x.view(1, 1024)
-            cpp_ops.customAtenAddmmHostMicroseconds("none", c1_b, c1_x2, c1_w_t, 20)
-            torch.cuda.synchronize()
-            e0.record(stream)
-            host_us = cpp_ops.customAtenAddmmHostMicroseconds("none", c1_b, c1_x2, c1_w_t, 200)
-            e1.record(stream)
-            torch.cuda.synchronize()
-            other["cpp_custom_aten_addmm_1024x1024"] = {"host_us_per_call": round(host_us, 3),
-                                                        "us_per_call_on_the_stream": round(e0.elapsed_time(e1) * 1e3 / 200, 3)}
         except ImportError:
-            pass
+            cpp_ops = None
+        if cpp_ops is not None:
+            cpp_ops.initialize(0)
+            c1_w, c1_w_t, c1_x2 = c1_pool[0], c1_pool[0].t(), c1_x.view(1, 1024)
+            host = {}
+
+            def host_us(op, tensors, prm=()):
+                cpp_ops.opHostMicroseconds(op, list(tensors), list(prm), 30)
+                torch.cuda.synchronize()
+                e0.record(stream)
+                us_h = cpp_ops.opHostMicroseconds(op, list(tensors), list(prm), 300)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                return round(us_h, 3), round(e0.elapsed_time(e1) * 1e3 / 300, 3)
+            gemv_dev_us = other["gemv_1024x1024_us"]
+            for name_, op_, ts_ in (("customAtenAddmm_1024x1024", "addmm", (c1_b, c1_x2, c1_w_t)),
+                                    ("customAtenMatmul_1024x1024", "matmul", (c1_w, c1_x.view(1024, 1))),
+                                    ("atenLinear_1024x1024", "linear", (c1_x2, c1_w, c1_b))):
+                h_, s_ = host_us(op_, ts_)
+                host[name_] = {"host_us_per_call": h_, "us_per_call_on_the_stream": s_, "kernel_us": gemv_dev_us}
+            # atenLstm1 at seq_len 1: one layer of H = I = 1024 (a GNMT decoder cell), and the RNNT prediction network's two
+            # layers of H = I = 320; device time = the calls' launches on preallocated buffers, replayed from a graph
+            for name_, (I_, H_, L_) in (("atenLstm1_seq_len_1_H1024", (1024, 1024, 1)), ("atenLstm1_seq_len_1_H320_two_layers", (320, 320, 2))):
+                prm_, x_, h0_, c0_ = workloads.lstm_inputs(4201 + L_, I_, H_, L_, False, 1)
+                prm_ = [q.to(dev) for q in prm_]
+                x_, h0_, c0_ = x_.to(dev), h0_.to(dev).contiguous(), c0_.to(dev).contiguous()
+                y_, hn_, cn_ = cpp_ops.atenLstm1(x_, [h0_, c0_], prm_, True, L_, 0.0, False, False, False)
+                plan_ = P.LstmPlan(prm_, True, L_, False, 1)
+
+                def lstm_launch(s_h=sh, plan_=plan_, x_=x_, h0_=h0_, c0_=c0_, y_=y_, hn_=hn_, cn_=cn_):
+                    lib.pimhip_lstm_forward(plan_._handle, x_.data_ptr(), h0_.data_ptr(), c0_.data_ptr(), y_.data_ptr(),
+                                            hn_.data_ptr(), cn_.data_ptr(), 1, s_h)
+                dev_us = round(graph_timed_us(lstm_launch, 32), 3)
+                h_, s_ = host_us("lstm1", (x_, h0_, c0_), prm_)
+                hi_, si_ = host_us("lstm1_into", (x_, h0_, c0_, y_, hn_, cn_), prm_)
+                host[name_] = {"host_us_per_call": h_, "us_per_call_on_the_stream": s_, "kernel_us": dev_us,
+                               "into_caller_buffers_host_us_per_call": hi_, "into_caller_buffers_us_per_call_on_the_stream": si_}
+            other["cpp_operators_per_token_calls"] = host
         # MoE FFN decode step (router 768 -> 8, then one expert 768 -> 3072 ReLU -> 768): three dependent launches on
         # resident (warm) weights, the expert fixed so that no host round trip for the argmax is inside the figure
         wr, w1, w2 = (0.02 * torch.randn(8, 768, device=dev)).half(), (0.02 * torch.randn(3072, 768, device=dev)).half(), \
@@ -593,14 +621,14 @@ def main():
         def reproject():
             fplan.set_encoder(enc2d)
         # the floor beside it: one launch that only reads as many warm bytes as the step has weights
-        step_bytes = (2 * 4096 * 1024 + 3 * 2 * 4096 * 1024) * 2 + 3 * 4096 * 50 * 4 + 32000 * 1024 * 2
-        probe_buf = torch.randn(step_bytes // 4, device=dev)
-        probe_us = timed_us(lambda: lib.pimhip_probe_stream_read(probe_buf.data_ptr(), step_bytes // 16 * 16, sh), 100, settle_s=0.3)
+        dec_step_bytes = (2 * 4096 * 1024 + 3 * 2 * 4096 * 1024) * 2 + 3 * 4096 * 50 * 4 + 32000 * 1024 * 2
+        probe_buf = torch.randn(dec_step_bytes // 4, device=dev)
+        probe_us = timed_us(lambda: lib.pimhip_probe_stream_read(probe_buf.data_ptr(), dec_step_bytes // 16 * 16, sh), 100, settle_s=0.3)
         del probe_buf
         other["decoder_step_one_launch"] = {
             "issued_from_python_us": round(fused_eager_us, 2), "hip_graph_replay_us": round(fused_graph_us, 2),
             "read_only_kernel_us": round(probe_us, 2),
-            "bytes": (2 * 4096 * 1024 + 3 * 2 * 4096 * 1024) * 2 + 3 * 4096 * 50 * 4 + 32000 * 1024 * 2,
+            "bytes": dec_step_bytes,
             "max_abs_diff_of_logits_to_the_8_launch_step": round(fused_err, 6),
             "set_encoder_once_per_sentence_us": round(timed_us(reproject, 20), 2)}
         # the reference's own HIP GEMV (custom_ops.h addmv_kernel_Axy, compiled from its tree) on the same cold weights
@@ -696,6 +724,7 @@ def main():
                           "runs (<= 4 s) per sweep shape after 2 warm-ups, same weight every run (cache-warm), one pass of the "
                           "same 4-GEMV sweep; " + "; ".join(detail))
 
+    assert step_bytes == sum(gemv_bytes(n, k) for n, k in SWEEP) and abs(value * ms_per_step * 1e6 - step_bytes) <= 1e-3 * step_bytes
     out = {
         "metric": "fp16 GEMV HBM GB/s (% of peak) at 1 GPU; LSTM us/layer-step at H=1024",
         "value": round(value, 1),

@@ -240,18 +240,6 @@ int pimhip_input_projection_packed(void* out, const void* x, const void* packed,
 int pimhip_gemv_status(void* stream, int* gave_up);
 int pimhip_set_gemv_spin_limit(unsigned int spin_limit);
 
-/* ---- measurement ----------------------------------------------------------------------------- */
-
-/* No counterpart in the reference.  Reads `bytes` bytes (a multiple of 16, 16-byte aligned) once with the streaming loads
- * of the GEMV kernels and keeps nothing: what one launch of it takes is the floor for any kernel that has to read
- * those bytes, launch included.  The benchmark reports each GEMV beside it. */
-int pimhip_probe_stream_read(const void* data, int64_t bytes, void* stream);
-
-/* No counterpart in the reference.  Launches `blocks` workgroups of `threads` lanes; workgroup b stores the index of
- * the XCD it runs on (the hardware's XCC_ID) to out[b] (uint32).  What the per-XCD LSTM kernel (mode 4) relies on can be
- * looked at with it: consecutive workgroups go to consecutive XCDs. */
-int pimhip_probe_xcc_map(void* out, int blocks, int threads, void* stream);
-
 /* ---- decoder step ---------------------------------------------------------------------------- */
 
 typedef struct PimHipDecoderPlan PimHipDecoderPlan;

@@ -28,17 +28,38 @@ def hipcc():
     return exe
 
 
-def build_pimhip(verbose=True):
-    src = [os.path.join(CSRC, "pimhip_api.hip")]
-    cmd = [hipcc()] + HIP_FLAGS + src + ["-o", LIB_PATH]
+# One translation unit per kernel family (each kernel header is compiled once); api_common.h is what they share.
+SOURCES = ["api_core.hip", "api_gemv.hip", "api_xproj.hip", "api_lstm.hip", "api_decoder.hip", "api_moe.hip"]
+OBJ_DIR = os.path.join(PKG_DIR, "build")
+
+
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+    return res.returncode, out
+
+
+def build_pimhip(verbose=True, jobs=None):
+    """Compiles the translation units side by side (hipcc -c), then links libpimhip.so."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    compile_flags = [f for f in HIP_FLAGS if f != "-shared"]
+    objs = [os.path.join(OBJ_DIR, os.path.splitext(f)[0] + ".o") for f in SOURCES]
+    cmds = [[hipcc()] + compile_flags + ["-c", os.path.join(CSRC, f), "-o", o] for f, o in zip(SOURCES, objs)]
+    jobs = jobs or min(len(cmds), max(1, (os.cpu_count() or 2) - 1), 8)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        results = list(pool.map(lambda c: _run(c, verbose), cmds))
+    for (rc, out), cmd in zip(results, cmds):
+        if rc != 0:
+            raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + out)
+        if verbose and out.strip():
+            print(out)
+    rc, out = _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB_PATH], verbose)
+    if rc != 0:
+        raise RuntimeError("linking libpimhip.so failed:\n" + out)
     return LIB_PATH
 
 

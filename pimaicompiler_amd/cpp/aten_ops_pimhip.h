@@ -65,6 +65,15 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> atenLstm1(const at::Tensor& input
                                                          double dropout, bool train, bool bidirectional,
                                                          bool batch_first);
 
+// atenLstm1 with results written where the caller wants them: `output`, `hy`, `cy` that are defined (contiguous fp16 GPU
+// tensors with the results' element counts, e.g. rows of the decoder's state buffer or the head of an attention
+// concatenation buffer) are filled in place, undefined ones are allocated.  It takes the place of the at::cat / slice /
+// updateBlob sequence executeAtenLSTM1 runs after every GNMT decoder step to move hy / cy / output into those buffers
+// (aten_ops_executor.cpp:2238-2302), and of the three allocations per call.  The outputs must not overlap the inputs.
+void atenLstm1Into(const at::Tensor& input, at::TensorList hx, at::TensorList params, bool has_biases, int64_t num_layers,
+                   double dropout, bool train, bool bidirectional, bool batch_first, at::Tensor& output, at::Tensor& hy,
+                   at::Tensor& cy);
+
 std::tuple<at::Tensor, at::Tensor, at::Tensor> atenLstm2(const at::Tensor& data, const at::Tensor& batch_sizes,
                                                          at::TensorList hx, at::TensorList params, bool has_biases,
                                                          int64_t num_layers, double dropout, bool train,

@@ -19,13 +19,41 @@ PYBIND11_MODULE(_aten_ops_pimhip, m)
         ops::customAtenAddmm(act, self, mat1, mat2, beta, alpha, out, nullptr);
         return out.toTensor();
     });
-    // `iters` calls in a row from C++: what one call costs the host thread (wall time of the loop / iters, in us).
-    m.def("customAtenAddmmHostMicroseconds", [](const std::string& act, at::Tensor self, at::Tensor mat1, at::Tensor mat2, int iters) {
+    // `iters` calls in a row from C++: what one call costs the host thread (wall time of the loop / iters, in us).  Nothing
+    // synchronises inside the loop, so the figure is the host's, not the GPU's.
+    //   "addmm": t = {self, mat1, mat2}    "matmul": t = {self, other}    "linear": t = {input, weight[, bias]}
+    //   "lstm1": t = {input, h0, c0}, params in LibTorch order with biases, unidirectional, num_layers = params / 4
+    //   "lstm1_into": the same through atenLstm1Into with t = {input, h0, c0, output, hy, cy}
+    m.def("opHostMicroseconds", [](const std::string& op, std::vector<at::Tensor> t, std::vector<at::Tensor> params, int iters) {
         torch::jit::IValue out;
+        std::vector<at::Tensor> hx;
+        if (op == "lstm1" || op == "lstm1_into") hx = {t.at(1), t.at(2)};
+        const int64_t layers = (int64_t)params.size() / 4;
+        const c10::optional<at::Tensor> bias = (op == "linear" && t.size() > 2) ? c10::optional<at::Tensor>(t[2]) : c10::nullopt;
         const auto t0 = std::chrono::steady_clock::now();
-        for (int i = 0; i < iters; ++i) ops::customAtenAddmm(act, self, mat1, mat2, 1, 1, out, nullptr);
+        for (int i = 0; i < iters; ++i) {
+            if (op == "addmm")
+                ops::customAtenAddmm("none", t.at(0), t.at(1), t.at(2), 1, 1, out, nullptr);
+            else if (op == "matmul")
+                ops::customAtenMatmul(t.at(0), t.at(1), out, nullptr);
+            else if (op == "linear")
+                ops::atenLinear(t.at(0), t.at(1), bias);
+            else if (op == "lstm1")
+                ops::atenLstm1(t.at(0), hx, params, true, layers, 0.0, false, false, false);
+            else if (op == "lstm1_into")
+                ops::atenLstm1Into(t.at(0), hx, params, true, layers, 0.0, false, false, false, t.at(3), t.at(4), t.at(5));
+            else
+                throw utils::NNRuntimeException("unknown operator " + op);
+        }
         const auto t1 = std::chrono::steady_clock::now();
         return std::chrono::duration<double, std::micro>(t1 - t0).count() / (iters > 0 ? iters : 1);
+    });
+    m.def("atenLstm1Into", [](const at::Tensor& input, std::vector<at::Tensor> hx, std::vector<at::Tensor> params, bool has_biases,
+                              int64_t num_layers, double dropout, bool train, bool bidirectional, bool batch_first,
+                              c10::optional<at::Tensor> output, c10::optional<at::Tensor> hy, c10::optional<at::Tensor> cy) {
+        at::Tensor y = output.value_or(at::Tensor()), hn = hy.value_or(at::Tensor()), cn = cy.value_or(at::Tensor());
+        ops::atenLstm1Into(input, hx, params, has_biases, num_layers, dropout, train, bidirectional, batch_first, y, hn, cn);
+        return std::make_tuple(y, hn, cn);
     });
     m.def("customAtenMatmul", [](at::Tensor self, at::Tensor other) {
         torch::jit::IValue out;

@@ -98,21 +98,8 @@ struct DecoderStepArgs {
     unsigned int* abort_host;
     unsigned int spin_limit;
     int H;
-#ifdef PIMHIP_DECODER_TRACE
-    unsigned long long* trace;  // [blocks][16 wavefronts][32] timestamps (100 MHz), for tuning builds only
-#endif
 };
 
-#ifdef PIMHIP_DECODER_TRACE
-#define DEC_TRACE(slot)                                                                                            \
-    do {                                                                                                           \
-        if (p.trace && lane == 0) p.trace[((long)blockIdx.x * 16 + wave) * 32 + (slot)] = wall_clock64();           \
-    } while (0)
-#else
-#define DEC_TRACE(slot) \
-    do {                \
-    } while (0)
-#endif
 
 // Transpose-sum of four per-lane partial sums over the wavefront: lane l ends up with the total of slot
 // 2 * (l & 1) + ((l >> 1) & 1), i.e. with slots {0, 2, 1, 3} in lanes {0, 1, 2, 3} (and every lane with lane & 3 alike).
@@ -171,7 +158,6 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
     half8_t zero8;
 #pragma unroll
     for (int e = 0; e < 8; ++e) zero8[e] = (half_t)0.0f;
-    DEC_TRACE(0);
 
     if (wave < kDecStreamWaves) {
         // =========================================== the streaming wavefronts ===========================================
@@ -275,7 +261,6 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
         auto deliver = [&](int k) __attribute__((always_inline)) {
             const float a = transpose_sum4(acc[k], lane);  // gate (lane & 3), this wavefront's half of the columns
             if (lane < 4) part[wave][lane] = a;
-            DEC_TRACE(8 + 4 * k);
             __syncthreads();  // B1: the gate sums of layer k are in LDS
         };
 
@@ -294,9 +279,7 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                 cls_bias[it] = p.cls_b ? b : 0.0f;
             }
         }
-        DEC_TRACE(1);
         if (staged_ctx_first) __syncthreads();  // B0: a given context is in LDS (a first layer that takes it)
-        DEC_TRACE(2);
         half8_t cvec = (staged_ctx_first && active) ? *reinterpret_cast<const half8_t*>(&ctx_vec[chunk * 8]) : zero8;
         consume_a(0, cvec, hv0);
         if (x_one_piece) {
@@ -353,7 +336,6 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
         cls_prefetch(cls_groups_after<L>(0));
         if (L > 1 || has_cls) {
             __syncthreads();  // B3 of layer 0: its whole output (the next input) is in LDS
-            DEC_TRACE(10);
         }
 #pragma unroll
         for (int k = 1; k < L; ++k) {
@@ -366,7 +348,6 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
             cls_prefetch(cls_groups_after<L>(k));
             if (k + 1 < L || has_cls) {
                 __syncthreads();  // B3: the layer's whole output (the next input) is in LDS
-                DEC_TRACE(10 + 4 * k);
             }
         }
 
@@ -405,7 +386,6 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                 cls_finish(cbuf[1], it + 1, 0.0f, false);
             }
         }
-        DEC_TRACE(25);
     } else {
         // ========================= the wavefronts that activate, publish and poll (no weights) =========================
         const int pw = wave - kDecStreamWaves;         // 0: also activates and publishes
@@ -481,16 +461,13 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                 }
             }
         }
-        DEC_TRACE(1);
         if (staged_ctx_first) __syncthreads();  // B0
-        DEC_TRACE(2);
 
         half_t keep_h = (half_t)0.0f, keep_c = (half_t)0.0f;  // layer 0's new state, stored once every block has read h_prev
 #pragma unroll
         for (int k = 0; k < L; ++k) {
             const DecoderLayerArgs& ly = p.layer[k];
             __syncthreads();  // B1: the gate sums of layer k are in LDS
-            DEC_TRACE(8 + 4 * k);
             const bool exchange = k + 1 < L || has_cls;
             if (pw == 0) {
                 // (the streamers leave gate k in lane k, i.e. in part[.][k])
@@ -521,7 +498,6 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                         ly.out[pj] = o;
                     }
                 }
-                DEC_TRACE(9 + 4 * k);
                 if (exchange) {
                     unsigned long long* slot = reinterpret_cast<unsigned long long*>(p.hx + ((long)k * nb) * kDecEntryWords);
                     const unsigned long long word = (unsigned long long)readlane_u32(hbits, 0) | ((unsigned long long)readlane_u32(hbits, 4) << 16) |
@@ -569,7 +545,6 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                         *reinterpret_cast<half4_t*>(&in_vec[blk * 4]) = nv;
                     }
                 }
-                DEC_TRACE(10 + 4 * k);
                 __syncthreads();  // B3: the next input is in LDS
                 if (k == 0 && owner) {
                     // every block has published layer 0's output, so every block is past its reads of h_prev:

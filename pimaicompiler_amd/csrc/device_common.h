@@ -15,6 +15,10 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 
 static constexpr int kWave = 64;
 
+// The bit pattern of a partial-sum record of the sliced I_X_W GEMV that has not arrived yet (gemv_kernels.h); host code
+// fills the record buffers with it.
+static constexpr unsigned int kVmEmpty = 0xffffffffu;
+
 // acc += sum_{i<8} w[i] * x[i], products and sum in fp32.
 __device__ __forceinline__ float dot8(const half8_t w, const half8_t x, float acc)
 {
@@ -58,6 +62,11 @@ __device__ __forceinline__ float wave_sum(float v)
     v += __shfl_xor(v, 32, kWave);
     return v;
 }
+
+// The XCD a wavefront runs on: HW_REG_XCC_ID (hardware register 20), bits 3:0.  The probe that reports the placement of a
+// launch and the kernel that relies on it read it through this one function.
+static constexpr unsigned int kXccIdMask = 15u;
+__device__ __forceinline__ unsigned int hw_xcc_id() { return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & kXccIdMask; }
 
 // Every bounded wait of the kernels here also ends after kWaitTicks of the constant 100 MHz clock, whatever its poll
 // count: where a poll takes far longer than usual (counter collection serialising the memory system, a tool stepping the

@@ -252,7 +252,6 @@ __device__ __forceinline__ void load32_device_scope_one(const float* p, float4_t
                  : "memory");
 }
 
-static constexpr unsigned int kVmEmpty = 0xffffffffu;
 
 template <int WAVES, int U, int LPR>
 __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* __restrict__ x,

@@ -153,9 +153,19 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    // HW_REG_XCC_ID (hardware register 20), bits 3:0: the XCD this workgroup runs on.
-    const int xcd = (int)(__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 7u);
+    const int xcd = (int)hw_xcc_id();  // the XCD this workgroup runs on
     const int rank = blockIdx.x >> 3;
+    if (xcd >= kXcdCount) {
+        // An id outside 0..7: not the part this kernel is laid out for (the host checks the placement of a probe launch
+        // before it chooses this kernel).  Reported like a rank taken twice; every other workgroup's waits are bounded.
+        if (tid == 0) {
+            __hip_atomic_store(p.abort_host + 1, (unsigned int)blockIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            __hip_atomic_store(p.abort_host + 2, (unsigned int)xcd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(p.abort_host, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        return;
+    }
     const int role = p.role[xcd];
     const int H = p.H;
     const int T = p.T;

@@ -309,16 +309,18 @@ def aten_linear_cat2(input1, input2, weight, bias=None, act_type="none", stream=
     """y = act(W[out, in1 + in2] . cat(input1, input2) + b) for two batch-1 inputs that lie apart, without concatenating
     them (pimhip_execute_gemv_cat2): the first layer of the RNNT joint network, which the reference turns into two
     dependent addmm launches (RemoveCatForAddmm, compiler/source/frontend/optimizer/remove_cat_for_addmm.cpp:46-191).
-    Shapes the launch does not take (widths not multiples of 8, more than one row) are concatenated and go through
-    aten_linear."""
+    Operands the launch does not take (widths not multiples of 8, more than one row, an input or weight that is not 16-byte
+    aligned) are concatenated and go through aten_linear."""
     _require_half_cuda(input1, input2, weight, bias)
     out_w, in_w = weight.shape
     n1, n2 = input1.numel(), input2.numel()
     w = weight if weight.stride(1) == 1 else weight.contiguous()
-    if n1 + n2 != in_w or (n1 & 7) or (n2 & 7) or (w.stride(0) & 7) or input1.shape[:-1] != input2.shape[:-1]:
+    x1, x2 = input1.contiguous(), input2.contiguous()
+    # (a view at an offset that is not a multiple of eight halves is not 16-byte aligned: the launch refuses it)
+    if (n1 + n2 != in_w or (n1 & 7) or (n2 & 7) or (w.stride(0) & 7) or input1.shape[:-1] != input2.shape[:-1] or
+            (x1.data_ptr() & 15) or (x2.data_ptr() & 15) or (w.data_ptr() & 15)):
         return aten_linear(torch.cat([input1, input2], -1), weight, bias, act_type, stream)
     _ensure_init(w)
-    x1, x2 = input1.contiguous(), input2.contiguous()
     if bias is not None:
         bias = bias.contiguous()
         if bias.numel() != out_w:

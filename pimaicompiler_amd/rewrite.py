@@ -364,7 +364,8 @@ def fuse_decoder_step(g: Graph):
 
     Left alone: cells whose weights are not constants, a pre-residual y with another consumer (the fused step only
     stores out_k, hn_k, cn_k), a context that is computed from the chain itself (in GNMT the attention query is layer
-    0's output: the chain then starts at layer 1), chains of fewer than two cells."""
+    0's output: the chain then starts at layer 1), a cell whose initial state is computed from the cells below it (the chain
+    ends in front of it), chains of fewer than two cells."""
     taken = []
     for first in list(g.ops):
         if all(first is not o for o in g.ops) or any(first is o for o in taken) or not _single_step_cell(g, first):
@@ -405,6 +406,13 @@ def fuse_decoder_step(g: Graph):
                 n = k
                 break
         forms = forms[:n]
+        # ---- a cell's initial state must not be computed from the chain below it (the previous cell's hn handed on, say):
+        # the fused op reads every h0 / c0 before any cell runs, so the chain is cut in front of such a cell
+        for k in range(1, len(forms)):
+            below = [m for f in forms[:k] for m in [f["cell"]] + ([f["add"]] if f["add"] is not None else [])]
+            if any(_depends_on(g, t, below) for t in forms[k]["cell"].inputs[1:3]):
+                forms = forms[:k]
+                break
         # ---- the context must not be computed from the chain
         if ctx is not None and forms and _depends_on(g, ctx, [f["cell"] for f in forms]):
             continue                          # (the chain that starts one cell later is found when the loop reaches that cell)
@@ -425,7 +433,7 @@ def fuse_decoder_step(g: Graph):
         last_out = forms[-1]["out"]
         cls = next((u for u in g.consumers(last_out)
                     if u.type in ("aten::linear", "pimhip::gemv") and u.inputs[0] == last_out and g.is_constant(u.inputs[1]) and
-                    g.constants[u.inputs[1]].dim() == 2 and g.constants[u.inputs[1]].size(1) == forms[0]["H"] and
+                    g.constants[u.inputs[1]] is not None and g.constants[u.inputs[1]].dim() == 2 and g.constants[u.inputs[1]].size(1) == forms[0]["H"] and
                     u.attrs.get("act_type", "none") == "none"), None)
         if cls is not None:
             members.append(cls)

@@ -13,10 +13,21 @@ from pimaicompiler_amd import _lib as L
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "pimhip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(pimhip_[a-z0-9_]+)\s*\(", text)))
+HEADERS = ("pimhip.h", "pimhip_probe.h")   # the drop-in interface; the measurement aids
+
+
+def declared_functions(headers=HEADERS):
+    names = set()
+    for h in headers:
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(pimhip_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_the_drop_in_header_carries_no_measurement_aids():
+    assert not [n for n in declared_functions(("pimhip.h",)) if "probe" in n or "debug" in n or "trace" in n]
+    assert declared_functions(("pimhip_probe.h",)) == ["pimhip_probe_stream_read", "pimhip_probe_xcc_map"]
 
 
 def test_header_declares_what_the_binding_binds():
@@ -38,7 +49,7 @@ def test_header_is_plain_c_and_links_against_the_library(tmp_path):
         pytest.skip("no C compiler")
     src = tmp_path / "uses_every_entry_point.c"
     names = declared_functions()
-    src.write_text('#include "pimhip.h"\n#include <stdio.h>\nint main(void)\n{\n    const void* table[] = {\n' +
+    src.write_text('#include "pimhip.h"\n#include "pimhip_probe.h"\n#include <stdio.h>\nint main(void)\n{\n    const void* table[] = {\n' +
                    "".join(f"        (const void*)&{n},\n" for n in names) +
                    '    };\n    printf("%d\\n", (int)(sizeof(table) / sizeof(table[0])));\n    return 0;\n}\n')
     exe = tmp_path / "uses_every_entry_point"

@@ -187,3 +187,62 @@ def test_cpp_plan_cache_follows_weight_updates(cpp_gpu):
     y1 = cpp_gpu.atenLstm1(*args)[0]
     assert maxabs(y1, oracle.torch_lstm(x, h0, c0, params2, True, 1, False)[0]) <= 2e-3
     assert cpp_gpu.invalidateLstmPlans(pd) == 1 and cpp_gpu.invalidateLstmPlans(pd) == 0
+
+
+@pytest.mark.gpu
+def test_cpp_gemv_reads_strided_and_transposed_views_where_they_lie(cpp_gpu):
+    """The operators make no tensor besides the output: a column block of a wider weight (row pitch above the row length),
+    the transposed view SwapAddmmInputs leaves, operands with leading dims of one, and a bias that is a strided view all
+    reach the kernel through pointers and a pitch, and give the bits of the launch on contiguous copies."""
+    W, x, b = workloads.gemv_inputs(2102, 512, 1024)
+    wide = torch.zeros(512, 2048, dtype=torch.float16, device=DEV)
+    wide[:, 512:1536] = W.to(DEV)
+    Wd, xd, bd = W.to(DEV), x.to(DEV), b.to(DEV)
+    want = cpp_gpu.customAtenAddmm("none", bd, Wd, xd.t(), 1.0, 1.0)            # MV on contiguous operands: [512, 1]
+    assert maxabs(want, oracle.torch_addmm(b, x, W)) <= 2e-3
+    block = wide[:, 512:1536]                                                    # [512, 1024], pitch 2048
+    assert torch.equal(cpp_gpu.customAtenAddmm("none", bd, block, xd.t(), 1.0, 1.0), want)
+    assert torch.equal(cpp_gpu.customAtenAddmm("none", bd, xd, block.t(), 1.0, 1.0).reshape(-1), want.reshape(-1))   # VM on the .t() view
+    assert torch.equal(cpp_gpu.atenLinear(xd, block, bd).reshape(-1), want.reshape(-1))
+    assert torch.equal(cpp_gpu.customAtenAddmm("none", bd, block.view(1, 1, 512, 1024).squeeze(0), xd.t().unsqueeze(0), 1.0, 1.0).reshape(-1),
+                       want.reshape(-1))
+    b2 = torch.zeros(512, 2, dtype=torch.float16, device=DEV)
+    b2[:, 0] = bd
+    assert torch.equal(cpp_gpu.customAtenAddmm("none", b2[:, 0], Wd, xd.t(), 1.0, 1.0), want)                         # strided bias
+    x2 = torch.zeros(1024, 2, dtype=torch.float16, device=DEV)
+    x2[:, 1] = xd.reshape(-1)
+    assert torch.equal(cpp_gpu.customAtenMatmul(Wd, x2[:, 1:2]), cpp_gpu.customAtenMatmul(Wd, xd.t()))               # strided vector
+    with pytest.raises(Exception):
+        cpp_gpu.customAtenAddmm("none", bd[:100], Wd, xd.t(), 1.0, 1.0)                                                # bias of the wrong length
+
+
+@pytest.mark.gpu
+def test_cpp_lstm_into_fills_the_callers_buffers(cpp_gpu):
+    """atenLstm1Into: one decoder step (seq_len 1, two layers) written into rows of a state buffer and the head of a
+    concatenation buffer, as the GNMT decoder's executor wants them; undefined outputs are allocated; the bits are
+    atenLstm1's."""
+    params, x, h0, c0 = workloads.lstm_inputs(4301, 320, 320, 2, False, 1)
+    pd = [p.to(DEV) for p in params]
+    h0d, c0d = (0.3 * torch.randn(2, 1, 320)).half().to(DEV), (0.3 * torch.randn(2, 1, 320)).half().to(DEV)
+    xd = x.to(DEV)
+    y, hn, cn = cpp_gpu.atenLstm1(xd, [h0d, c0d], pd, True, 2, 0.0, False, False, False)
+    wy, whn, wcn = oracle.torch_lstm(x, h0d.cpu(), c0d.cpu(), params, True, 2, False)
+    assert maxabs(y, wy) <= 5e-3 and maxabs(hn, whn) <= 5e-3 and maxabs(cn, wcn) <= 5e-3
+    state = torch.zeros(4, 1, 320, dtype=torch.float16, device=DEV)
+    cat = torch.zeros(1, 1, 640, dtype=torch.float16, device=DEV)
+    y_dst = cat.view(-1)[:320].view(1, 1, 320)
+    y2, hn2, cn2 = cpp_gpu.atenLstm1Into(xd, [h0d, c0d], pd, True, 2, 0.0, False, False, False, y_dst, state[0:2], state[2:4])
+    assert y2.data_ptr() == cat.data_ptr() and hn2.data_ptr() == state.data_ptr()
+    assert torch.equal(cat.view(-1)[:320], y.view(-1)) and torch.equal(state[0:2], hn) and torch.equal(state[2:4], cn)
+    assert float(cat.view(-1)[320:].abs().max()) == 0
+    y3, hn3, cn3 = cpp_gpu.atenLstm1Into(xd, [h0d, c0d], pd, True, 2, 0.0, False, False, False, None, None, None)
+    assert torch.equal(y3, y) and torch.equal(hn3, hn) and torch.equal(cn3, cn) and list(y3.shape) == [1, 1, 320]
+    with pytest.raises(Exception):
+        cpp_gpu.atenLstm1Into(xd, [h0d, c0d], pd, True, 2, 0.0, False, False, False, cat.view(-1)[:300], None, None)   # wrong size
+    # a sequence after the single steps, same parameter objects: the cached plan grows, the hit path still recognises it
+    xs = torch.randn(40, 1, 320).half()
+    ys, hs, cs = cpp_gpu.atenLstm1(xs.to(DEV), [h0d, c0d], pd, True, 2, 0.0, False, False, False)
+    ws = oracle.torch_lstm(xs, h0d.cpu(), c0d.cpu(), params, True, 2, False)
+    assert maxabs(ys, ws[0]) <= 5e-3 and maxabs(hs, ws[1]) <= 5e-3
+    y4 = cpp_gpu.atenLstm1(xd, [h0d, c0d], pd, True, 2, 0.0, False, False, False)[0]
+    assert torch.equal(y4, y)

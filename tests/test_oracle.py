@@ -142,6 +142,29 @@ def test_dot_brute_force():
     assert oracle.dot(a[:0], b[:0])[0] == 0
 
 
+def test_add_is_the_fp16_sum_rounded_once_in_both_broadcast_forms():
+    """oracle.add against LibTorch CPU's fp16 add (the op executeAtenAdd's fallback calls) and against the exact sum in
+    float64 rounded once by numpy: element-wise, and one row added to every row.  Includes ties, a sum that overflows and
+    cancellation to zero; a row taken for a column, a second rounding or a dropped operand changes a bit somewhere."""
+    import torch
+    rng = np.random.default_rng(9)
+    a = _rand_half(rng, 7 * 40, scale=3.0).reshape(7, 40)
+    b = _rand_half(rng, 7 * 40, scale=3.0).reshape(7, 40)
+    a[0, :4] = np.array([1.0, 2048.0, 65504.0, 0.333251953125], dtype=np.float16)
+    b[0, :4] = np.array([2.0 ** -11, 1.0, 65504.0, -0.333251953125], dtype=np.float16)   # tie to even, tie, overflow, zero
+    row = _rand_half(rng, 40, scale=3.0)
+    for other in (b, row):
+        got = oracle.add(a, other)
+        with np.errstate(over="ignore"):
+            want_np = (a.astype(np.float64) + other.astype(np.float64)).astype(np.float16)
+        want_torch = (torch.from_numpy(a) + torch.from_numpy(other)).numpy()
+        assert got.shape == a.shape
+        assert np.array_equal(got.view(np.uint16), want_np.view(np.uint16))
+        assert np.array_equal(got.view(np.uint16), want_torch.view(np.uint16))
+    assert not np.array_equal(oracle.add(a, row).view(np.uint16), oracle.add(a, b).view(np.uint16))
+    assert np.isinf(oracle.add(a, b)[0, 2]) and oracle.add(a, b)[0, 3] == 0
+
+
 def test_gemv_f32_port_matches_numpy():
     rng = np.random.default_rng(8)
     W, x, b = rng.standard_normal((9, 40)).astype(np.float32), rng.standard_normal(40).astype(np.float32), rng.standard_normal(9).astype(np.float32)

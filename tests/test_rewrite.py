@@ -318,6 +318,27 @@ def test_decoder_chain_guards():
     g.outputs = [300]
     R.fuse_decoder_step(g)
     assert g.types() == ["aten::lstm"]
+    # a cell whose initial state is computed from the cells below it (layer 2 starts from layer 1's hn): the fused op reads
+    # every h0 / c0 before any cell runs, so the chain ends in front of that cell and nothing reads a tensor nobody makes
+    g, _ = decoder_graph()
+    cell2 = [o for o in g.ops if o.type == "aten::lstm"][2]
+    cell2.inputs[1] = 311
+    R.fuse_decoder_step(g)
+    fused = [o for o in g.ops if o.type == "pimhip::decoder_step"]
+    # (two steps of two cells: the second starts at that cell and reads the hn the first one produces)
+    assert [f.attrs["num_layers"] for f in fused] == [2, 2] and fused[0].attrs["classifier"] is None
+    assert 311 in fused[0].outputs and 311 in fused[1].inputs and fused[1].attrs["classifier"] == (200, 201)
+    assert "aten::lstm" not in g.types()
+    produced = set(g.inputs) | set(g.constants)
+    for o in g.ops:
+        assert all(t in produced for t in o.inputs), o
+        produced.update(o.outputs)
+    # a classifier-shaped linear whose weight is a constant without a value (not loaded yet) is not taken, and does not
+    # make the pass fail
+    g, _ = decoder_graph()
+    g.constants[200] = None
+    R.fuse_decoder_step(g)
+    assert g.types() == ["pimhip::decoder_step", "aten::linear"] and g.ops[0].attrs["classifier"] is None
 
 
 @pytest.mark.gpu
