@@ -315,20 +315,34 @@ typedef struct PimHipMoePlan PimHipMoePlan;
  *   w1, b1, w2, b2: host arrays of E device pointers (b1 / b2 may be null arrays: no bias); all weights row-major, dense,
  *   fp16, 16-byte aligned.  E <= 64; d_model <= 2048 and d_ff <= 4096, multiples of 8 (PIMHIP_ERR_UNSUPPORTED
  *   otherwise: three pimhip_execute_gemv calls serve any size); act as in pimhip_execute_gemv.
- * The plan keeps the pointers (the weights must outlive it) and owns a 32 KiB exchange buffer.  Needs a device whose
- * 256 blocks are resident together; the library orders it against its other such launches (pimhip_lstm_forward,
- * pimhip_decoder_step), and steps sharing a plan must be ordered on one stream. */
+ * The plan keeps the pointers (the weights must outlive it) and owns a 32 KiB exchange buffer.  The workgroups of a step
+ * (at most 256) exchange the hidden values among themselves and have to be resident together; the library orders the step
+ * against its other such launches (pimhip_lstm_forward, pimhip_decoder_step), and steps sharing a plan must be ordered
+ * on one stream. */
 int pimhip_moe_plan_create(PimHipMoePlan** plan, const void* router_w, const void* router_b, const void* const* w1,
                            const void* const* b1, const void* const* w2, const void* const* b2, int num_experts,
                            int64_t d_model, int64_t d_ff, int act, int scale_by_router_prob, void* stream);
 int pimhip_moe_plan_destroy(PimHipMoePlan* plan);
 
 /* x [d_model] (16-byte aligned), y [d_model]; router_logits [E] fp16 and expert [1] int32 are device pointers or null.
- * Records one kernel.  Every wait inside is bounded: see pimhip_moe_plan_status. */
+ * Records one kernel.  Every wait inside is bounded, and a wait that gives up (other work kept part of the GPU from running
+ * the step's workgroups together) costs time, not the result: the workgroups that waited in vain compute the missing
+ * hidden values themselves, inside the same launch, and y is what it would have been.  Later steps do the same from the
+ * start until a step issued outside a graph capture has put the exchange back in order (it synchronises the stream then);
+ * after the third such event the plan stops exchanging for good (about 25 times slower per step, still one launch). */
 int pimhip_moe_ffn_step(PimHipMoePlan* plan, const void* x, void* y, void* router_logits, int* expert, void* stream);
 
-/* As pimhip_decoder_plan_status / pimhip_decoder_plan_set_spin_limit. */
+/* Always PIMHIP_OK for a valid plan: no step of this plan leaves an undefined result (kept for callers of the earlier
+ * interface, where a wait that gave up was an error). */
 int pimhip_moe_plan_status(PimHipMoePlan* plan);
+
+/* No counterpart in the reference.  *events: how many times a wait inside a step of this plan has given up so far (as far
+ * as the host has seen: ask after synchronising the stream); *exchanging (may be null): 1 while steps still exchange
+ * hidden values between workgroups, 0 once the plan has gone over to the self-sufficient mode for good. */
+int pimhip_moe_plan_fallbacks(PimHipMoePlan* plan, uint64_t* events, int* exchanging);
+
+/* Polls of one wait before it gives up (default 2^22, roughly seconds).  Tests pass 0 so that every wait whose first look
+ * fails gives up at once: every kernel still ends by itself. */
 int pimhip_moe_plan_set_spin_limit(PimHipMoePlan* plan, unsigned int spin_limit);
 
 #ifdef __cplusplus

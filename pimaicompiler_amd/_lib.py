@@ -69,6 +69,7 @@ SIGNATURES = {
     "pimhip_moe_ffn_step": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                            ctypes.c_void_p, ctypes.c_void_p]),
     "pimhip_moe_plan_status": (ctypes.c_int, [ctypes.c_void_p]),
+    "pimhip_moe_plan_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), c_int_p]),
     "pimhip_moe_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "pimhip_input_projection": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),

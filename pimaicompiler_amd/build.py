@@ -17,6 +17,9 @@ LIB_PATH = os.path.join(PKG_DIR, "libpimhip.so")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first 16 dwords of a kernel's plain arguments arrive in scalar registers instead of through a load at its start
+    # (about 0.1 us off every launch whose first instructions need them; kernels that take a struct are unaffected)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wno-unused-result", "-Wno-unused-value",
 ]
 

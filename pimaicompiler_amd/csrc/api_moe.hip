@@ -14,20 +14,26 @@ struct PimHipMoePlan {
     const half_t* router_w = nullptr;
     const half_t* router_b = nullptr;
     const half_t** tables = nullptr;       // device: [4][E] pointers (W1, b1, W2, b2 of every expert)
-    unsigned long long* hx = nullptr;      // [2][kMoeBlocks][kMoeEntryWords], all ones = empty
+    unsigned long long* hx = nullptr;      // [2][kMoeMaxBlocks][kMoeEntryWords], all ones = empty
     unsigned int* g_counter = nullptr;
     unsigned int* abort_flag = nullptr;
     unsigned int* abort_host = nullptr;
     unsigned int* abort_host_dev = nullptr;
     unsigned int spin_limit = 1u << 22;
     bool reset_exchange = false;
+    int blocks = 0;                        // workgroups of a step, all resident together
+    int wpb = 1;                           // 16-byte words of hidden values per producing block
+    int rpb2 = 1;                          // rows of W2 per block
+    unsigned long long gave_up_events = 0; // waits that gave up, as far as the host has seen them (pimhip_moe_plan_fallbacks)
+    bool alone = false;                    // every block computes all hidden values itself: after kMoeEventsBeforeAlone events
 };
 
 namespace
 {
 std::vector<PimHipMoePlan*> g_moe_plans;
 
-constexpr size_t kMoeExchangeWords32 = (size_t)2 * kMoeBlocks * kMoeEntryWords * 2;  // the exchange buffer as 32-bit words
+constexpr size_t kMoeExchangeWords32 = (size_t)2 * kMoeMaxBlocks * kMoeEntryWords * 2;  // the exchange buffer as 32-bit words
+constexpr unsigned long long kMoeEventsBeforeAlone = 3;  // waits given up before a plan stops exchanging for good
 
 int destroy_moe_plan_locked(PimHipMoePlan* plan)
 {
@@ -76,8 +82,18 @@ extern "C" int pimhip_moe_plan_create(PimHipMoePlan** plan_out, const void* rout
         return fail(PIMHIP_ERR_UNSUPPORTED, "the one-launch step takes d_model in [8, %d] and d_ff in [8, %d], multiples of 8 (got %lld, %lld): "
                                             "use three pimhip_execute_gemv calls", kMoeMaxModel, kMoeMaxFf, (long long)d_model, (long long)d_ff);
     if (act != PIMHIP_ACT_NONE && act != PIMHIP_ACT_RELU) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "act=%d", act);
-    if (st->num_cus < kMoeBlocks)
-        return fail(PIMHIP_ERR_UNSUPPORTED, "the one-launch step needs %d compute units resident at once (device has %d)", kMoeBlocks, st->num_cus);
+    // Hidden values travel as 16-byte words of eight, at most two per producing block; every block owns at most eight rows
+    // of the second matrix.  The fewest blocks that allows: few, large participants shorten the all-to-all, which is what
+    // bounds a step (768 / 3072: 192 blocks, two words and four rows each).
+    const int nwords = (int)(d_ff / 8);
+    int blocks = (nwords + kMoeMaxWordsPerBlock - 1) / kMoeMaxWordsPerBlock;
+    const int blocks_for_w2 = (int)((d_model + kMoeMaxRows2 - 1) / kMoeMaxRows2);
+    if (blocks < blocks_for_w2) blocks = blocks_for_w2;
+    const int wpb_final = (nwords + blocks - 1) / blocks;
+    int per_cu = 0;
+    PIMHIP_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, moe_ffn_step_f16_kernel, kMoeThreads, 0));
+    if ((int64_t)per_cu * st->num_cus < blocks)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "the %d workgroups of the one-launch step cannot all be resident on this device", blocks);
     if (!aligned16(router_w)) return fail(PIMHIP_ERR_UNSUPPORTED, "router_w must be 16-byte aligned");
     std::vector<const half_t*> host_tables((size_t)4 * num_experts, nullptr);
     for (int e = 0; e < num_experts; ++e) {
@@ -98,6 +114,9 @@ extern "C" int pimhip_moe_plan_create(PimHipMoePlan** plan_out, const void* rout
     plan->scale_by_prob = scale_by_router_prob ? 1 : 0;
     plan->router_w = (const half_t*)router_w;
     plan->router_b = (const half_t*)router_b;
+    plan->blocks = blocks;
+    plan->wpb = wpb_final;
+    plan->rpb2 = (int)((d_model + blocks - 1) / blocks);
     auto cleanup_fail = [&](int status) {
         std::lock_guard<std::mutex> lock(g_mutex);
         destroy_moe_plan_locked(plan);
@@ -150,11 +169,16 @@ extern "C" int pimhip_moe_plan_set_spin_limit(PimHipMoePlan* plan, unsigned int 
 extern "C" int pimhip_moe_plan_status(PimHipMoePlan* plan)
 {
     if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
-    if (*plan->abort_host != 0u) {
-        *plan->abort_host = 0u;
-        plan->reset_exchange = true;
-        return fail(PIMHIP_ERR_TIMEOUT, "a bounded wait of the mixture-of-experts step kernel gave up: the results of that step are undefined");
-    }
+    // A wait that gave up no longer leaves anything undefined (the blocks complete the step by themselves): there is
+    // nothing to report as an error.  pimhip_moe_plan_fallbacks counts the events.
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_moe_plan_fallbacks(PimHipMoePlan* plan, uint64_t* events, int* exchanging)
+{
+    if (!plan || !events) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan and events must be non-null");
+    *events = plan->gave_up_events + (*plan->abort_host != 0u ? 1u : 0u);
+    if (exchanging) *exchanging = (plan->alone || *events >= kMoeEventsBeforeAlone) ? 0 : 1;
     return PIMHIP_OK;
 }
 
@@ -175,24 +199,19 @@ extern "C" int pimhip_moe_ffn_step(PimHipMoePlan* plan, const void* x, void* y, 
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
     const bool capturing = capture != hipStreamCaptureStatusNone;
-    if (*plan->abort_host != 0u) {
-        if (capturing)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "an earlier step of this plan gave up a wait; recovering from that is not for a graph");
+    if (*plan->abort_host != 0u && !capturing) {
+        // A wait of an earlier step gave up.  That step's result was completed by the blocks themselves, and every step
+        // since has run self-sufficient (the abort word stays up on the device); here, outside any capture, the exchange is
+        // put back in order: drain the stream (steps sharing a plan are ordered on one stream), refill the slots, clear the
+        // words.  A plan that has needed this kMoeEventsBeforeAlone times stops exchanging for good.
         PIMHIP_HIP_CHECK(hipStreamSynchronize(s));
         *plan->abort_host = 0u;
-        plan->reset_exchange = true;
-        return fail(PIMHIP_ERR_TIMEOUT, "an earlier step of this plan gave up a wait of the mixture-of-experts step kernel: its results are "
-                                        "undefined (this call was not launched; the next one starts from a re-initialised exchange buffer)");
-    }
-    if (plan->reset_exchange) {
-        if (capturing)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's exchange buffer has to be re-initialised after a time-out, which a graph must not "
-                                                "record: run one step outside the capture first");
+        ++plan->gave_up_events;
+        if (plan->gave_up_events >= kMoeEventsBeforeAlone) plan->alone = true;
         launch_fill_u32(reinterpret_cast<unsigned int*>(plan->hx), kMoeExchangeWords32, ~0u, s);
         launch_fill_u32(plan->g_counter, 1, 0u, s);
         launch_fill_u32(plan->abort_flag, 1, 0u, s);
         PIMHIP_HIP_CHECK(hipGetLastError());
-        plan->reset_exchange = false;
     }
     MoeStepArgs a;
     memset(&a, 0, sizeof(a));
@@ -212,15 +231,16 @@ extern "C" int pimhip_moe_ffn_step(PimHipMoePlan* plan, const void* x, void* y, 
     a.E = plan->num_experts;
     a.act = plan->act;
     a.scale_by_prob = plan->scale_by_prob;
-    a.rpb1 = (int)((plan->d_ff + kMoeBlocks - 1) / kMoeBlocks);
-    a.rpb2 = (int)((plan->d_model + kMoeBlocks - 1) / kMoeBlocks);
+    a.wpb = plan->wpb;
+    a.rpb2 = plan->rpb2;
+    a.alone = plan->alone ? 1 : 0;
     a.spin_limit = plan->spin_limit;
     // All blocks have to be resident at once, like the sequence kernel's: ordered after it on other streams.
     if (!capturing) {
         rc = order_after_previous_sequence_launch(st, s);
         if (rc != PIMHIP_OK) return rc;
     }
-    moe_ffn_step_f16_kernel<<<dim3(kMoeBlocks), dim3(kMoeThreads), 0, s>>>(a);
+    moe_ffn_step_f16_kernel<<<dim3((unsigned)plan->blocks), dim3(kMoeThreads), 0, s>>>(a.x, a.router_w, a.router_b, a.tables, a.d_model, a.d_ff, a.E, a.act, a);
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
 }

@@ -221,25 +221,6 @@ struct LstmSeqArgs {
     unsigned int spin_limit;
 };
 
-// One 16-byte device-scope load.  Each 8-byte half is validated on its own by the caller, so nothing depends on the
-// 16 bytes being read as a unit.
-__device__ __forceinline__ void load16_device_scope(const void* p, unsigned long long& lo, unsigned long long& hi)
-{
-    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-    u32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
-    lo = (unsigned long long)v[0] | ((unsigned long long)v[1] << 32);
-    hi = (unsigned long long)v[2] | ((unsigned long long)v[3] << 32);
-}
-
-// One 16-byte device-scope store of two 8-byte words (each validated on its own by the readers).
-__device__ __forceinline__ void store16_device_scope(void* p, unsigned long long lo, unsigned long long hi)
-{
-    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-    const u32x4 v = {(unsigned int)lo, (unsigned int)(lo >> 32), (unsigned int)hi, (unsigned int)(hi >> 32)};
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
-}
-
 template <int NC, bool WAVEFRONT, int UNITS = kSeqUnits, int COLS = 16>
 __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
 {

@@ -12,16 +12,29 @@
 // slice of `hidden` and, once it has everybody's, multiplies its rows of the second matrix, which are already in
 // registers by then.
 //
-// Grid: kMoeBlocks blocks of four wavefronts, all resident at once.  Block b owns rows [b * rpb1, (b + 1) * rpb1) of W1
-// and rows [b * rpb2, (b + 1) * rpb2) of W2; local row i belongs to wavefront i % 4, whose lanes stride over the row's
-// 16-byte pieces.
+// Grid: `blocks` blocks of eight wavefronts, all resident at once.  `hidden` travels as 16-byte words of eight values;
+// block b makes words [b * wpb, (b + 1) * wpb) (wpb = 1 or 2: at most 256 blocks make the at most 512 words), i.e.
+// rows 8 * wpb * b .. of W1, wavefront w the rows w * wpb .. of those.  Of W2 block b owns rows [b * rpb2, (b + 1) * rpb2),
+// rpb2 <= 8, one row per wavefront.
 //
-// Exchange: hx[2][blocks] entries of 64 bytes; a block's hidden values (at most 16) in the first 32 bytes as four 8-byte
-// words.  An empty word is all ones, which no four fp16 values written here can be (a NaN is written as 0x7e00).  The
-// two sets alternate by the launch count g (a device word read at the start and advanced by block 0 at the end): a
-// launch uses set g & 1 and marks its own entry of the other set empty for the launch after it.  Every wait is bounded:
-// after `spin_limit` polls a lane raises the abort flags, all lanes stop waiting, the kernel runs to its end with
-// undefined results and the host reports a time-out and refills both sets before the next launch.
+// What bounds the step is not bandwidth (9.4 MB) but a chain of dependent round trips: token and router rows, the expert's
+// W1 rows, the all-to-all of `hidden`, the store of y.  So nothing else may stand in that chain: the launch count (which
+// says which set of exchange slots this launch uses) is a device-scope load and is asked for behind the router's cached
+// loads, not in front of them; the
+// slots of the other set are emptied at the very end; a lane that waits looks at ONE 16-byte word of ONE producer per poll
+// (a poll round over all blocks gets slower with every further load per lane); the row of W2 is asked for right behind
+// the rows of W1 and has arrived when the hidden values have.
+//
+// Exchange: hx[2][blocks] entries of 64 bytes, a block's words in the first 16 * wpb bytes.  An empty 8-byte half is all
+// ones, which no four fp16 values written here can be (a NaN is written as 0x7e00).  The two sets alternate by the launch
+// count g (a device word read at the start and advanced by block 0 at the end): a launch uses set g & 1 and marks its own
+// entry of the other set empty for the launch after it.
+//
+// A wait that gives up does not leave the result undefined.  Every wait is bounded (`spin_limit` polls, one second); a block
+// in which a lane gave up computes every hidden value itself from W1[e] (no other block is needed for that: it is only
+// slower, a few tens of microseconds) and goes on.  It raises the plan's abort word, which stays up: every later launch
+// starts in that self-sufficient mode (the exchange slots may hold values of the launch that was cut short) until the
+// host has refilled the slots and cleared the word.
 #pragma once
 
 #include "device_common.h"
@@ -29,20 +42,21 @@
 namespace pimhip
 {
 
-constexpr int kMoeThreads = 256;
+constexpr int kMoeThreads = 512;
 constexpr int kMoeWaves = kMoeThreads / 64;
-constexpr int kMoeBlocks = 256;
+constexpr int kMoeMaxBlocks = 256;
 constexpr int kMoeMaxExperts = 64;
 constexpr int kMoeMaxModel = 2048;                    // d_model: at most four 16-byte pieces of a row per lane
-constexpr int kMoeMaxFf = 4096;                       // d_ff: at most eight 16-byte pieces of a W2 row per lane
-constexpr int kMoeXC = kMoeMaxModel / 8 / 64;
-constexpr int kMoeFC = kMoeMaxFf / 8 / 64;
-constexpr int kMoeRows1 = kMoeMaxFf / kMoeBlocks / kMoeWaves;     // W1 rows per wavefront: 4
-constexpr int kMoeRows2 = kMoeMaxModel / kMoeBlocks / kMoeWaves;  // W2 rows per wavefront: 2
-constexpr int kMoeEntryWords = 8;                     // 8-byte words per entry (64 bytes); the first four carry values
+constexpr int kMoeMaxFf = 4096;                       // d_ff: at most 512 words of eight hidden values, one per thread
+constexpr int kMoeXC = kMoeMaxModel / 8 / 64;         // 16-byte pieces of a W1 row per lane
+constexpr int kMoeFC = kMoeMaxFf / 8 / 64;            // 16-byte pieces of a W2 row per lane
+constexpr int kMoeMaxWordsPerBlock = 2;               // wpb
+constexpr int kMoeMaxRows2 = kMoeWaves;               // W2 rows per block: one per wavefront
+constexpr int kMoeEntryWords = 8;                     // 8-byte words per entry (64 bytes); the first 2 * wpb carry values
 constexpr unsigned long long kMoeEmpty = ~0ull;
-static_assert(kMoeBlocks <= kMoeThreads, "thread t of a block polls block t's entry");
-static_assert(kMoeRows1 * kMoeWaves <= 16, "a block's hidden values fit the four 8-byte words of its entry");
+static_assert(kMoeMaxFf / 8 <= kMoeThreads, "thread t of a block polls word t");
+static_assert(kMoeMaxWordsPerBlock * kMoeMaxBlocks * 8 >= kMoeMaxFf, "every hidden value has a producer");
+static_assert(2 * kMoeMaxWordsPerBlock <= kMoeEntryWords, "a block's words fit its entry");
 
 struct MoeStepArgs {
     const half_t* x;                 // [d_model]
@@ -52,35 +66,45 @@ struct MoeStepArgs {
     half_t* y;                       // [d_model]
     half_t* router_logits;           // [E] or null
     int* expert;                     // [1] or null
-    unsigned long long* hx;          // [2][kMoeBlocks][kMoeEntryWords]
+    unsigned long long* hx;          // [2][blocks][kMoeEntryWords]
     unsigned int* g_counter;
-    unsigned int* abort_flag;
-    unsigned int* abort_host;
+    unsigned int* abort_flag;        // device word: non-zero from the first wait that gave up until the host clears it
+    unsigned int* abort_host;        // the same event for the host to see
     int d_model, d_ff, E, act, scale_by_prob;
-    int rpb1, rpb2;                  // rows of W1 / W2 per block
+    int wpb;                         // 16-byte words of hidden values per producing block
+    int rpb2;                        // rows of W2 per block
     unsigned int spin_limit;
+    int alone;                       // non-zero: every block computes all hidden values itself, nothing is exchanged
 };
 
-__global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(MoeStepArgs p)
+// What the kernel's first instructions need comes as plain arguments in front of the struct: those arrive in scalar
+// registers with the wavefront (kernel-argument preload) instead of through a load at its start.
+__global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const half_t* x_, const half_t* router_w_, const half_t* router_b_,
+                                                                       const half_t* const* tables_, int d_model_, int d_ff_, int E_, int act_,
+                                                                       MoeStepArgs p)
 {
+    p.x = x_;
+    p.router_w = router_w_;
+    p.router_b = router_b_;
+    p.tables = tables_;
+    p.d_model = d_model_;
+    p.d_ff = d_ff_;
+    p.E = E_;
+    p.act = act_;
     __shared__ __align__(16) half_t hidden[kMoeMaxFf];
     __shared__ float logit_s[kMoeMaxExperts];
     __shared__ const half_t* table_s[4][kMoeMaxExperts];
-    __shared__ __align__(8) unsigned short mine[16];  // this block's hidden values (bits), zeros where it has no row
+    __shared__ __align__(16) unsigned short mine[8 * kMoeMaxWordsPerBlock];  // this block's hidden values (bits)
+    __shared__ int someone_gave_up;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int b = blockIdx.x, nb = gridDim.x;
-    const int nx = p.d_model >> 3, nf = p.d_ff >> 3;
+    const int nx = p.d_model >> 3, nf = p.d_ff >> 3;  // 16-byte pieces of a W1 / W2 row; nf is also the number of hidden words
     half8_t zero8;
 #pragma unroll
     for (int e = 0; e < 8; ++e) zero8[e] = (half_t)0.0f;
 
-    const unsigned int g = __hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const unsigned int set = g & 1u;
-    // this block's entry of the other set is empty for the next launch (nobody reads that set during this one)
-    if (tid < kMoeEntryWords)
-        __hip_atomic_store(p.hx + ((long)(set ^ 1u) * nb + b) * kMoeEntryWords + tid, kMoeEmpty, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (tid < 16) mine[tid] = 0;
+    if (tid == 0) someone_gave_up = 0;
     // the experts' pointers, while the router's rows travel
     for (int i = tid; i < 4 * p.E; i += kMoeThreads) table_s[i / p.E][i % p.E] = p.tables[i];
 
@@ -89,7 +113,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(MoeStepAr
     const half8_t* x8 = reinterpret_cast<const half8_t*>(p.x);
 #pragma unroll
     for (int k = 0; k < kMoeXC; ++k) xr[k] = (lane + 64 * k < nx) ? x8[lane + 64 * k] : zero8;
-    // (two experts per wavefront and pass: all their loads are in flight together, one round trip for E <= 8)
+    // (two experts per wavefront and pass: all their loads are in flight together, one round trip for E <= 16)
     for (int e0 = wave; e0 < p.E; e0 += 2 * kMoeWaves) {
         const int e1 = e0 + kMoeWaves;
         const half8_t* w8a = reinterpret_cast<const half8_t*>(p.router_w) + (long)e0 * nx;
@@ -97,6 +121,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(MoeStepAr
         half8_t ra[kMoeXC], rb[kMoeXC];
 #pragma unroll
         for (int k = 0; k < kMoeXC; ++k) {
+            if (64 * k >= nx) break;  // (uniform) pieces past the row for every lane
             const int c = min(lane + 64 * k, nx - 1);
             ra[k] = w8a[c];
             rb[k] = w8b[c];
@@ -148,106 +173,125 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(MoeStepAr
     const half8_t* w2 = reinterpret_cast<const half8_t*>(table_s[2][best]);
     const half_t* b2 = table_s[3][best];
 
-    // ---- hidden = act(W1[e] . x + b1[e]): this block's rows ----
-    half8_t w1r[kMoeRows1][kMoeXC];
+    // One row of W1[e] times the token, bias and activation, as the bits `hidden` holds; a NaN in its canonical form.
+    auto hidden_bits = [&](float a, int r) {
+        if (b1) a += (float)b1[r];
+        if (p.act == 1) a = fmaxf(a, 0.0f);
+        unsigned short bits = __builtin_bit_cast(unsigned short, (half_t)a);
+        if (a != a) bits = 0x7e00u;
+        return bits;
+    };
+    // This wavefront's row of W2[e]: asked for here, consumed at the end.
+    half8_t w2r[kMoeFC];
+    const int r2 = b * p.rpb2 + wave;
+    const bool has_row2 = wave < p.rpb2 && r2 < p.d_model;
+    auto ask_for_w2 = [&]() {
+        const half8_t* src = w2 + (long)min(r2, p.d_model - 1) * nf;  // (a row this wavefront does not own is loaded and dropped)
 #pragma unroll
-    for (int s = 0; s < kMoeRows1; ++s) {
-        const int r = min(b * p.rpb1 + wave + kMoeWaves * s, p.d_ff - 1);  // (rows this block does not own are loaded and dropped)
+        for (int k = 0; k < kMoeFC; ++k) {
+            if (64 * k >= nf) break;  // (uniform) pieces past the row for every lane
+            w2r[k] = load_stream(src + min(lane + 64 * k, nf - 1));
+        }
+    };
+
+    // The launch count (which set of slots this launch uses) and the abort word are device-scope loads, which take longer
+    // than the cached ones above and would hold those up if they stood in front of them (a wavefront's loads return in
+    // order).  Asked for here, they travel with the rows of W1 and are needed when the block publishes.
+    const unsigned int g = __hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned int poisoned = __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // ---- hidden = act(W1[e] . x + b1[e]): this block's words (asked for whether or not they will be published) ----
+    const int row0 = 8 * p.wpb * b + wave * p.wpb;  // this wavefront's first row
+    half8_t w1r[kMoeMaxWordsPerBlock][kMoeXC];
 #pragma unroll
-        for (int k = 0; k < kMoeXC; ++k) w1r[s][k] = load_stream(w1 + (long)r * nx + min(lane + 64 * k, nx - 1));
+    for (int s = 0; s < kMoeMaxWordsPerBlock; ++s) {
+        const int r = min(row0 + min(s, p.wpb - 1), p.d_ff - 1);
+#pragma unroll
+        for (int k = 0; k < kMoeXC; ++k) {
+            if (64 * k >= nx) break;
+            w1r[s][k] = load_stream(w1 + (long)r * nx + min(lane + 64 * k, nx - 1));
+        }
     }
 #pragma unroll
-    for (int s = 0; s < kMoeRows1; ++s) {
-        const int i = wave + kMoeWaves * s;
-        const int r = b * p.rpb1 + i;
+    for (int s = 0; s < kMoeMaxWordsPerBlock; ++s) {
+        const int r = row0 + s;
         float a = 0.0f;
 #pragma unroll
         for (int k = 0; k < kMoeXC; ++k)
             if (lane + 64 * k < nx) a = dot8(w1r[s][k], xr[k], a);
         a = wave_sum(a);
-        if (lane == 0 && i < p.rpb1 && r < p.d_ff) {
-            if (b1) a += (float)b1[r];
-            if (p.act == 1) a = fmaxf(a, 0.0f);
-            unsigned short bits = __builtin_bit_cast(unsigned short, (half_t)a);
-            if (a != a) bits = 0x7e00u;
-            mine[i] = bits;
+        if (lane == 0 && s < p.wpb) mine[wave * p.wpb + s] = r < p.d_ff ? hidden_bits(a, r) : (unsigned short)0;
+    }
+    const bool alone = p.alone != 0 || poisoned != 0u;
+    const unsigned int set = g & 1u;
+    if (!alone) {
+        __syncthreads();
+        if (tid < p.wpb && b * p.wpb + tid < nf) {
+            const unsigned long long* src = reinterpret_cast<const unsigned long long*>(&mine[8 * tid]);
+            store16_device_scope(p.hx + ((long)set * nb + b) * kMoeEntryWords + 2 * tid, src[0], src[1]);
         }
-    }
-    __syncthreads();
-    if (tid < 4) {
-        const unsigned long long word = *reinterpret_cast<const unsigned long long*>(&mine[4 * tid]);
-        __hip_atomic_store(p.hx + ((long)set * nb + b) * kMoeEntryWords + tid, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    // ---- everybody's hidden values: thread t takes block t's entry ----
-    half8_t w2r[kMoeRows2][kMoeFC];
-    {
-        const int first = tid * p.rpb1;               // block tid's first row
-        const int rows = min(p.rpb1, p.d_ff - first);  // <= 0: that block has no row
-        // A block without rows publishes zeros and is waited for all the same: block 0 advances the launch count at its end,
-        // and no block may still be on its way to reading it then.
-        const int words = tid < nb ? (rows > 0 ? (rows + 3) >> 2 : 1) : 0;
-        const unsigned long long* slot = p.hx + ((long)set * nb + tid) * kMoeEntryWords;
-        unsigned long long got[4] = {0ull, 0ull, 0ull, 0ull};
-        auto poll = [&]() {
-            bool ok = true;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                if (w < words) {
-                    got[w] = __hip_atomic_load(const_cast<unsigned long long*>(slot) + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    ok = ok && got[w] != kMoeEmpty;
+        ask_for_w2();
+        // ---- everybody's hidden values: thread t takes word t ----
+        if (tid < nf) {
+            const unsigned long long* slot = p.hx + ((long)set * nb + tid / p.wpb) * kMoeEntryWords + 2 * (tid % p.wpb);
+            unsigned long long lo = kMoeEmpty, hi = kMoeEmpty;
+            unsigned int spins = 0;
+            unsigned long long t_first = 0ull;
+            bool gave_up = false;
+            while (true) {
+                load16_device_scope(slot, lo, hi);
+                if (lo != kMoeEmpty && hi != kMoeEmpty) break;
+                if (spins > 0u && (spins & 255u) == 0u) {
+                    if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
+                    if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
                 }
+                if (spins >= p.spin_limit) {  // (with a limit of 0 a lane whose first look failed gives up without another)
+                    __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    gave_up = true;
+                }
+                if (gave_up) break;
+                if (spins != 0xffffffffu) ++spins;
             }
-            return ok;
-        };
-        // This block's rows of W2[e] are asked for behind the store and in front of the first look: they travel while the
-        // hidden values do.  (Measured on MI355X, 768 / 3072 / 8 experts: 8.3 us per step this way; asked for together
-        // with W1's rows they delay every block's hidden values, 8.7 us; asked for behind the first look they put a whole
-        // round trip in front of the second, 9.1 us.)
-#pragma unroll
-        for (int s = 0; s < kMoeRows2; ++s) {
-            const int r = min(b * p.rpb2 + wave + kMoeWaves * s, p.d_model - 1);
-#pragma unroll
-            for (int k = 0; k < kMoeFC; ++k) w2r[s][k] = load_stream(w2 + (long)r * nf + min(lane + 64 * k, nf - 1));
+            if (gave_up) someone_gave_up = 1;
+            typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+            const u64x2 v = {lo, hi};
+            *reinterpret_cast<u64x2*>(&hidden[8 * tid]) = v;
         }
-        bool ok = poll();
-        unsigned int spins = 0;
-        unsigned long long t_first = 0ull;
-        while (!ok) {
-            if (spins > 0u && (spins & 255u) == 0u) {
-                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) break;
-                if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
-            }
-            if (spins >= p.spin_limit) {  // (with a limit of 0 a lane whose first look failed gives up without another)
-                __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                break;
-            }
-            if (spins != 0xffffffffu) ++spins;
-            ok = poll();
-        }
-        for (int i = 0; i < rows && tid < nb; ++i)
-            hidden[first + i] = __builtin_bit_cast(half_t, (unsigned short)(got[i >> 2] >> (16 * (i & 3))));
+        __syncthreads();
+    } else {
+        ask_for_w2();
+        __syncthreads();
     }
-    __syncthreads();
+    if (alone || someone_gave_up) {
+        // ---- self-sufficient: every hidden value from W1[e], by this block alone ----
+        for (int r = wave; r < p.d_ff; r += kMoeWaves) {
+            float a = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kMoeXC; ++k)
+                if (lane + 64 * k < nx) a = dot8(w1[(long)r * nx + lane + 64 * k], xr[k], a);
+            a = wave_sum(a);
+            if (lane == 0) hidden[r] = __builtin_bit_cast(half_t, hidden_bits(a, r));
+        }
+        __syncthreads();
+    }
 
     // ---- y = W2[e] . hidden + b2[e] ----
-    half8_t hr[kMoeFC];
-#pragma unroll
-    for (int k = 0; k < kMoeFC; ++k) hr[k] = (lane + 64 * k < nf) ? *reinterpret_cast<const half8_t*>(&hidden[(lane + 64 * k) * 8]) : zero8;
-#pragma unroll
-    for (int s = 0; s < kMoeRows2; ++s) {
-        const int i = wave + kMoeWaves * s;
-        const int r = b * p.rpb2 + i;
+    {
         float a = 0.0f;
 #pragma unroll
-        for (int k = 0; k < kMoeFC; ++k)
-            if (lane + 64 * k < nf) a = dot8(w2r[s][k], hr[k], a);
+        for (int k = 0; k < kMoeFC; ++k) {
+            const int c = lane + 64 * k;
+            if (c < nf) a = dot8(w2r[k], *reinterpret_cast<const half8_t*>(&hidden[c * 8]), a);
+        }
         a = wave_sum(a);
-        if (lane == 0 && i < p.rpb2 && r < p.d_model) {
-            if (b2) a += (float)b2[r];
-            p.y[r] = (half_t)(a * scale);
+        if (lane == 0 && has_row2) {
+            if (b2) a += (float)b2[r2];
+            p.y[r2] = (half_t)(a * scale);
         }
     }
+    // this block's entry of the other set is empty for the next launch (nobody reads that set during this one)
+    if (tid < 2 * kMoeMaxWordsPerBlock)
+        __hip_atomic_store(p.hx + ((long)(set ^ 1u) * nb + b) * kMoeEntryWords + tid, kMoeEmpty, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (b == 0 && tid == 0) __hip_atomic_store(p.g_counter, g + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 

@@ -786,9 +786,19 @@ class MoePlan:
         _check(L.load().pimhip_moe_plan_set_spin_limit(self._handle, limit))
 
     def status(self):
-        """Raises NNRuntimeException if a step's kernel gave up a wait since the last report.  Synchronises."""
+        """Synchronises.  No step of this plan leaves an undefined result (a wait that gives up is made good inside the same
+        launch), so there is nothing to raise; fallbacks() counts such events."""
         torch.cuda.synchronize(self.device)
         _check(L.load().pimhip_moe_plan_status(self._handle))
+
+    def fallbacks(self):
+        """(events, exchanging): waits that have given up inside steps of this plan so far, and whether steps still exchange
+        hidden values between workgroups (False once the plan has gone over to the self-sufficient mode for good).
+        Synchronises (pimhip_moe_plan_fallbacks)."""
+        torch.cuda.synchronize(self.device)
+        events, exchanging = ctypes.c_uint64(0), ctypes.c_int(0)
+        _check(L.load().pimhip_moe_plan_fallbacks(self._handle, ctypes.byref(events), ctypes.byref(exchanging)))
+        return int(events.value), bool(exchanging.value)
 
     def bind(self, x, y, router_logits=None, expert=None):
         """Fixes the buffers of a step (x, y [d_model] fp16; router_logits [E] fp16 and expert [1] int32 optional) and returns

@@ -162,31 +162,37 @@ def test_moe_step_nan_and_limits(ops):
         plan.bind(torch.zeros(8, dtype=torch.float16, device=DEV), torch.zeros(d_model, dtype=torch.float16, device=DEV))
 
 
-def test_moe_step_wait_that_gives_up_is_reported_once_and_recovered_from(ops):
+def test_moe_step_whose_waits_give_up_still_gives_the_right_result(ops):
+    """A wait that gives up costs time, not the result: the workgroups that waited in vain compute the missing hidden values
+    themselves, inside the same launch.  Forced from the host with a spin limit of 0 (a wait whose first look fails gives up
+    at once; every kernel still ends by itself): the step that timed out is right, the steps after it are right (they run
+    self-sufficient until a step outside a capture has put the exchange back in order), the events are counted, and after
+    the third the plan stops exchanging for good."""
     E, d_model, d_ff = 8, 768, 3072
-    g, Wr, br, W1, b1, W2, b2 = make(11, E, d_model, d_ff, False, scale=0.02)
-    plan = ops.MoePlan((Wr.to(DEV), None), dev(W1), dev(W2))
-    x = torch.randn(1, d_model, generator=g).half()
-    want = libtorch_cpu(x, Wr, None, W1, None, W2, None, "aten::relu", False)
-    y, _, _ = plan.forward(x.to(DEV))
-    plan.status()
-    assert maxabs(y, want[3]) <= TOL
-    plan.set_spin_limit(0)                    # every wait gives up at its first unsuccessful poll; the kernel still ends
-    gave_up = False
-    for _ in range(5):
-        plan.forward(x.to(DEV))
-        try:
-            plan.status()
-        except ops.NNRuntimeException as err:
-            assert "gave up" in str(err)
-            gave_up = True
-            break
-    assert gave_up
+    g, Wr, br, W1, b1, W2, b2 = make(11, E, d_model, d_ff, True, scale=0.02)
+    plan = ops.MoePlan((Wr.to(DEV), br.to(DEV)), dev(W1), dev(W2), dev(b1), dev(b2))
+    xs = [torch.randn(1, d_model, generator=g).half() for _ in range(10)]
+    wants = [libtorch_cpu(x, Wr, br, W1, b1, W2, b2, "aten::relu", False) for x in xs]
+
+    def check(i):
+        y, _, expert = plan.forward(xs[i].to(DEV))
+        plan.status()
+        assert wants[i][4] <= 2 * TOL or (int(expert.item()) == wants[i][1] and maxabs(y, wants[i][3]) <= TOL), i
+
+    check(0)
+    assert plan.fallbacks() == (0, True)
+    plan.set_spin_limit(0)
+    events = 0
+    for i in range(1, 8):
+        check(i)                              # right whether or not a wait gave up in it
+        now, exchanging = plan.fallbacks()
+        assert now >= events and exchanging == (now < 3)
+        events = now
+    assert events >= 3                        # with 192 workgroups some first look fails in nearly every step
     plan.set_spin_limit(1 << 22)
-    plan.status()                             # reported once
-    y, _, expert = plan.forward(x.to(DEV))    # the exchange buffer is refilled before this launch
-    plan.status()
-    assert int(expert.item()) == want[1] and maxabs(y, want[3]) <= TOL
+    check(8)
+    check(9)
+    assert plan.fallbacks() == (events, False)   # nothing waits any more: no further events
 
 
 def test_resident_kernels_of_three_kinds_on_three_streams_take_turns(ops):
