@@ -100,8 +100,10 @@ int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* other_shape4
  * The I_X_W order splits the reduction over blocks for all but small weights; the blocks exchange partial sums through
  * a per-stream workspace the library allocates on the first such call on a stream (the call synchronises that stream
  * then, and again whenever a later call needs a larger workspace).  Calls that share a stream must not overlap.  Every
- * wait inside the kernel is bounded; should one ever give up, the next I_X_W call on that stream returns
- * PIMHIP_ERR_TIMEOUT (the earlier result is undefined), re-initialises the workspace and launches nothing. */
+ * wait inside the kernel is bounded, and one that gives up costs time, not the result: the block computes the missing
+ * partial sums itself, in the order their own block would have, so the result has the bits it would have had
+ * (pimhip_gemv_fallbacks counts such events; the next I_X_W call on that stream outside a graph capture puts the workspace
+ * back in order, synchronising the stream once). */
 int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
                         int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
 
@@ -120,8 +122,9 @@ int pimhip_execute_gemv_cat2(void* out, const void* in1, int64_t in1_w, const vo
  * nothing and records kernels only.  A product that needs more than 65536 partial sums
  * ((slices - 1) * out_w; none that pimhip_execute_gemv slices on a 256-CU part does) is refused with
  * PIMHIP_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that may overlap there (different streams,
- * or replays of graphs holding such calls) race and must be ordered by the caller.  After a wait that gave up, the next
- * call returns PIMHIP_ERR_TIMEOUT, refills the array (it synchronises the stream then) and launches nothing. */
+ * or replays of graphs holding such calls) race and must be ordered by the caller.  A wait that gives up is made good
+ * inside the launch as in pimhip_execute_gemv; the next call outside a graph capture refills the array (the one case in
+ * which this entry point synchronises the stream). */
 int pimhip_execute_gemv_static(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
                                int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
 
@@ -179,20 +182,30 @@ int pimhip_lstm_plan_destroy(PimHipLstmPlan* plan);
  * previous such call is ordered after it (an event wait), so that two of them never share the GPU.  On a capturing
  * stream that wait is left out (a graph cannot wait for another stream's event): order replays of such a graph against
  * the device's other sequence calls yourself.  The call records kernels only; the one case a graph must not hold, the
- * re-initialisation of the plan's buffers after a time-out or a change of mode, returns PIMHIP_ERR_UNSUPPORTED there. */
+ * re-initialisation of the plan's buffers after a change of mode, returns PIMHIP_ERR_UNSUPPORTED there. */
 int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn,
                         void* cn, int64_t seq_len, void* stream);
 
-/* After the stream has been synchronised: 0 if every persistent-kernel wait in the forwards of this plan so far
- * completed, PIMHIP_ERR_TIMEOUT if a bounded wait gave up (the outputs of that forward are undefined).  A time-out is
- * reported exactly once: by this call, or else by the next pimhip_lstm_forward of the plan, which then returns
- * PIMHIP_ERR_TIMEOUT after synchronising its stream and launches nothing.  The forward after the report re-initialises
- * the plan's exchange buffer and runs normally. */
+/* After the stream has been synchronised.  PIMHIP_OK unless the workgroups of the per-XCD kernel (mode 4) were not dealt to
+ * the XCDs in rotation in some forward of this plan (PIMHIP_ERR_TIMEOUT, reported once, here or by the next
+ * pimhip_lstm_forward; that forward's outputs are undefined and the plan stops choosing that kernel; a probe launch at
+ * plan creation keeps the kernel from being offered where the placement is not a rotation to begin with).  A wait that
+ * gave up is not an error: see pimhip_lstm_plan_fallbacks. */
 int pimhip_lstm_plan_status(PimHipLstmPlan* plan);
 
-/* Upper bound on the polls of one wait inside the persistent kernel (default 2^22, roughly seconds).  A wait
- * that reaches it gives up, the kernel still runs to its end, and pimhip_lstm_plan_status reports the time-out.
- * Tests of that error path pass 0 here so that every wait gives up at once. */
+/* No counterpart in the reference.  The workgroups of the persistent sequence kernels wait for one another, every wait
+ * bounded (pimhip_lstm_plan_set_spin_limit, and one second).  A wait that gives up (other work kept part of the GPU from
+ * running the workgroups together) costs time, not the result: the workgroup stops publishing, and at the end of the launch
+ * computes its units of the recurrence by itself from the call's inputs, so y, hn and cn are what they would have been.
+ * Sequence launches after that run the same way from their start until a pimhip_lstm_forward issued outside a graph capture
+ * has re-initialised the exchange (it synchronises the stream then); after the third such event the plan runs one launch
+ * per step, whose workgroups wait for nobody.
+ *   *events: waits that have given up so far, as far as the host has seen (ask after synchronising the stream);
+ *   *exchanging (may be null): 1 while sequence calls still use the persistent kernels, 0 once they do not. */
+int pimhip_lstm_plan_fallbacks(PimHipLstmPlan* plan, uint64_t* events, int* exchanging);
+
+/* Upper bound on the polls of one wait inside the persistent kernels (default 2^22, roughly seconds).  Tests of the path
+ * above pass 0 here so that every wait whose first look fails gives up at once; every kernel still ends by itself. */
 int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limit);
 
 /* Selects how pimhip_lstm_forward runs the recurrence: 0 = automatic, 1 = one fused launch per step,
@@ -230,14 +243,15 @@ int pimhip_input_projection_packed(void* out, const void* x, const void* packed,
                                    int64_t in_w, int64_t n_out, void* stream);
 
 /* No counterpart in the reference (the PIM SDK's PimExecuteGemm reports nothing either, aten_ops.cpp:659).
- * A sliced I_X_W product whose reducing blocks gave up waiting for partial sums (a bounded wait: other work kept
- * part of the GPU from running the blocks that produce them) is reported by the NEXT sliced product on that stream,
- * which returns PIMHIP_ERR_TIMEOUT.  A caller that wants to know before it uses the result synchronises the stream and
- * asks here: *gave_up gets bit 0 if a product of pimhip_execute_gemv / _bmm on `stream` gave up since the last
- * re-initialisation, bit 1 if one of pimhip_execute_gemv_static on this GPU did.  Nothing is cleared.
+ * A reducing block of a sliced I_X_W product that gave up waiting for partial sums (a bounded wait: other work kept part
+ * of the GPU from running the blocks that produce them) computes them itself; nothing is left undefined.  For a caller that
+ * wants to know, after synchronising the stream: *gave_up gets bit 0 if a product of pimhip_execute_gemv / _bmm on `stream`
+ * did so since the workspace was last put in order, bit 1 if one of pimhip_execute_gemv_static on this GPU did;
+ * pimhip_gemv_fallbacks gives the number of such events so far on `stream` plus those of the static entry point.
  * pimhip_set_gemv_spin_limit sets the number of polls per record for the current GPU (default 2^22, seconds); with 0 a
  * reducing block gives up without polling, which is how tests force the condition while every kernel still ends. */
 int pimhip_gemv_status(void* stream, int* gave_up);
+int pimhip_gemv_fallbacks(void* stream, uint64_t* events);
 int pimhip_set_gemv_spin_limit(unsigned int spin_limit);
 
 /* ---- decoder step ---------------------------------------------------------------------------- */

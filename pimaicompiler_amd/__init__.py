@@ -31,6 +31,7 @@ from .ops import (  # noqa: F401
     prepare_lstm,
     invalidate_lstm_plans,
     gemv_status,
+    gemv_fallbacks,
     synchronize_and_check,
     set_gemv_spin_limit,
 )

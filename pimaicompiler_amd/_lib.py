@@ -32,6 +32,7 @@ SIGNATURES = {
     "pimhip_probe_stream_read": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
     "pimhip_probe_xcc_map": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "pimhip_gemv_status": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
+    "pimhip_gemv_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]),
     "pimhip_set_gemv_spin_limit": (ctypes.c_int, [ctypes.c_uint]),
     "pimhip_execute_dot": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                           ctypes.c_void_p]),
@@ -49,6 +50,7 @@ SIGNATURES = {
                                            ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                            ctypes.c_void_p]),
     "pimhip_lstm_plan_status": (ctypes.c_int, [ctypes.c_void_p]),
+    "pimhip_lstm_plan_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), c_int_p]),
     "pimhip_lstm_plan_set_mode": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "pimhip_lstm_plan_set_residual": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "pimhip_lstm_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),

@@ -37,6 +37,8 @@ struct SplitWorkspace {
     size_t partial_elems = 0;
     unsigned int* status = nullptr;      // pinned host word the kernel sets when a wait for a record gives up
     unsigned int* status_dev = nullptr;  // the same word as the device addresses it
+    unsigned int* poison = nullptr;      // device word set at the same time: until it is cleared, reducing blocks ignore the records
+    unsigned long long gave_up_events = 0;  // such events, as far as the host has seen them
 };
 
 struct DeviceState {
@@ -54,6 +56,8 @@ struct DeviceState {
     float* static_partial = nullptr;
     unsigned int* static_status = nullptr;
     unsigned int* static_status_dev = nullptr;
+    unsigned int* static_poison = nullptr;   // this device's copy of the poison word that goes with `scratch`
+    unsigned long long static_gave_up_events = 0;
     // Polls of one record before a reducing lane of the sliced I_X_W kernel gives up (pimhip_set_gemv_spin_limit).
     unsigned int vm_spin_limit = 1u << 22;
 };

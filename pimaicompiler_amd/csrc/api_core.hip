@@ -27,6 +27,10 @@ __global__ void fill_u32_kernel(unsigned int* p, size_t n, unsigned int v)
 // address a kernel can use is looked up once per device (pimhip_initialize) and kept in DeviceState::static_partial.
 constexpr size_t kStaticScratchFloats = 64 * 1024;
 static __device__ __align__(256) float scratch[kStaticScratchFloats];
+// Non-zero from the moment a reducing block of pimhip_execute_gemv_static has given up on a record until the host has
+// refilled `scratch`: while it is up, reducing blocks ignore the records (one that arrived late would pass for the next
+// launch's) and compute every slice themselves.
+static __device__ unsigned int scratch_poison;
 
 std::map<int, DeviceState> g_devices;
 }  // namespace
@@ -108,6 +112,10 @@ extern "C" int pimhip_initialize(int device)
     PIMHIP_HIP_CHECK(hipGetSymbolAddress(&scratch_ptr, HIP_SYMBOL(scratch)));
     st.static_partial = static_cast<float*>(scratch_ptr);
     launch_fill_u32(reinterpret_cast<unsigned int*>(st.static_partial), kStaticScratchFloats, kVmEmpty, nullptr);
+    void* poison_ptr = nullptr;
+    PIMHIP_HIP_CHECK(hipGetSymbolAddress(&poison_ptr, HIP_SYMBOL(scratch_poison)));
+    st.static_poison = static_cast<unsigned int*>(poison_ptr);
+    launch_fill_u32(st.static_poison, 1, 0u, nullptr);
     PIMHIP_HIP_CHECK(hipGetLastError());
     if (!st.static_status) {
         PIMHIP_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&st.static_status), sizeof(unsigned int), hipHostMallocMapped));
@@ -135,6 +143,7 @@ extern "C" int pimhip_deinitialize(void)
         hipDeviceSynchronize();
         for (auto& w : kv.second.workspaces) {
             if (w.second.partial) hipFree(w.second.partial);
+            if (w.second.poison) hipFree(w.second.poison);
             if (w.second.status) hipHostFree(w.second.status);
         }
         kv.second.workspaces.clear();

@@ -15,11 +15,13 @@ int get_split_workspace(DeviceState* st, hipStream_t stream, size_t partial_elem
     std::lock_guard<std::mutex> lock(g_mutex);
     SplitWorkspace& ws = st->workspaces[stream];
     const bool gave_up = ws.status && *ws.status != 0u;
+    bool capturing = false;
     if (!ws.status || ws.partial_elems < partial_elems || gave_up) {
-        // Allocation, synchronisation and the memset below are not for a graph: ask before touching anything.
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         PIMHIP_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
-        if (capture != hipStreamCaptureStatusNone)
+        capturing = capture != hipStreamCaptureStatusNone;
+        // Allocation, synchronisation and the memset below are not for a graph.
+        if (capturing && (!ws.status || ws.partial_elems < partial_elems))
             return fail(PIMHIP_ERR_UNSUPPORTED, "this I_X_W product needs its stream's workspace (re)allocated, which a graph must not "
                                                 "record: run it once on this stream before the capture");
     }
@@ -27,8 +29,14 @@ int get_split_workspace(DeviceState* st, hipStream_t stream, size_t partial_elem
         PIMHIP_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&ws.status), sizeof(unsigned int), hipHostMallocMapped));
         *ws.status = 0u;
         PIMHIP_HIP_CHECK(hipHostGetDevicePointer(reinterpret_cast<void**>(&ws.status_dev), ws.status, 0));
+        PIMHIP_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&ws.poison), sizeof(unsigned int)));
+        PIMHIP_HIP_CHECK(hipMemsetAsync(ws.poison, 0, sizeof(unsigned int), stream));
     }
-    if (ws.partial_elems < partial_elems || gave_up) {
+    // A reducing block of an earlier product on this stream gave up on a record.  That product's result was completed by
+    // the block itself, and the products since have ignored the records (the poison word is up); outside a capture the
+    // records are refilled here and both words cleared.  (Inside one the launch goes ahead as it is: right, only slower.)
+    const bool recover = gave_up && !capturing;
+    if (ws.partial_elems < partial_elems || recover) {
         // Work already queued on this stream may still use the old buffer.
         PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
         if (ws.partial_elems < partial_elems) {
@@ -39,10 +47,9 @@ int get_split_workspace(DeviceState* st, hipStream_t stream, size_t partial_elem
             ws.partial_elems = partial_elems;
         }
         PIMHIP_HIP_CHECK(hipMemsetAsync(ws.partial, 0xff, ws.partial_elems * sizeof(float), stream));  // every word kVmEmpty
+        PIMHIP_HIP_CHECK(hipMemsetAsync(ws.poison, 0, sizeof(unsigned int), stream));
+        if (recover) ++ws.gave_up_events;
         *ws.status = 0u;
-        if (gave_up)
-            return fail(PIMHIP_ERR_TIMEOUT, "an earlier GEMV on this stream gave up waiting for partial sums; its result is undefined "
-                                            "(the workspace has been re-initialised, this call was not launched)");
     }
     *out = &ws;
     return PIMHIP_OK;
@@ -86,30 +93,33 @@ int gemv_mv(const half_t* W, const half_t* x, const half_t* bias, half_t* y, int
 
 // The records of the static scratch array instead of the stream's workspace: nothing is allocated, freed or
 // synchronised (pimhip_execute_gemv_static).
-int get_static_workspace(DeviceState* st, hipStream_t stream, size_t partial_elems, float** partial, unsigned int** status)
+int get_static_workspace(DeviceState* st, hipStream_t stream, size_t partial_elems, float** partial, unsigned int** status,
+                         unsigned int** poison)
 {
-    if (!st->static_partial || !st->static_status)
+    if (!st->static_partial || !st->static_status || !st->static_poison)
         return fail(PIMHIP_ERR_NOT_INITIALIZED, "the static scratch buffer of this device has not been set up");
     if (partial_elems > kStaticScratchFloats)
         return fail(PIMHIP_ERR_UNSUPPORTED, "this I_X_W product needs %zu partial sums, the static scratch buffer holds %zu: "
                                             "use pimhip_execute_gemv", partial_elems, kStaticScratchFloats);
     if (*st->static_status != 0u) {
-        // An earlier launch gave up a wait and may have left records behind: bring every word back to kVmEmpty with
-        // a fill kernel on this stream (a caller may be recording a graph, which must hold no memset), launch nothing
-        // else.  The word is cleared first: the launch that set it has ended, or the caller's calls overlap.
+        // A reducing block of an earlier launch gave up on a record: that product was completed by the block itself, and
+        // the launches since have ignored the records.  Outside a capture every word is brought back to kVmEmpty here with
+        // fill kernels on this stream and both words are cleared (the status word first: the launch that set it has ended
+        // once the stream has drained).  Inside a capture the launch goes ahead as it is: right, only slower.
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         PIMHIP_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
-        if (capture != hipStreamCaptureStatusNone)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "an earlier static GEMV gave up a wait; its recovery is not for a graph");
-        PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
-        *st->static_status = 0u;
-        launch_fill_u32(reinterpret_cast<unsigned int*>(st->static_partial), kStaticScratchFloats, kVmEmpty, stream);
-        PIMHIP_HIP_CHECK(hipGetLastError());
-        return fail(PIMHIP_ERR_TIMEOUT, "an earlier static GEMV gave up waiting for partial sums; its result is undefined "
-                                        "(the scratch buffer has been re-initialised, this call was not launched)");
+        if (capture == hipStreamCaptureStatusNone) {
+            PIMHIP_HIP_CHECK(hipStreamSynchronize(stream));
+            *st->static_status = 0u;
+            ++st->static_gave_up_events;
+            launch_fill_u32(reinterpret_cast<unsigned int*>(st->static_partial), kStaticScratchFloats, kVmEmpty, stream);
+            launch_fill_u32(st->static_poison, 1, 0u, stream);
+            PIMHIP_HIP_CHECK(hipGetLastError());
+        }
     }
     *partial = st->static_partial;
     *status = st->static_status_dev;
+    *poison = st->static_poison;
     return PIMHIP_OK;
 }
 
@@ -146,25 +156,27 @@ int gemv_vm(DeviceState* st, const half_t* x, const half_t* A, const half_t* bia
     if (slices < 1) slices = 1;
     float* partial = nullptr;
     unsigned int* status = nullptr;
+    unsigned int* poison = nullptr;
     if (slices > 1) {
         // Records of all slices but the last: partial[slice][N].
         const size_t partial_elems = (size_t)(slices - 1) * (size_t)N;
         int rc;
         if (static_ws) {
-            rc = get_static_workspace(st, s, partial_elems, &partial, &status);
+            rc = get_static_workspace(st, s, partial_elems, &partial, &status, &poison);
         } else {
             SplitWorkspace* ws = nullptr;
             rc = get_split_workspace(st, s, partial_elems, &ws);
             if (rc == PIMHIP_OK) {
                 partial = ws->partial;
                 status = ws->status_dev;
+                poison = ws->poison;
             }
         }
         if (rc != PIMHIP_OK) return rc;
     }
     dim3 grid(col_blocks, slices);
     gemv_vm_f16_kernel<WAVES, U, LPR><<<grid, WAVES * 64, 0, s>>>(x, A, bias, outs, (int)K, (int)N, (long)lda, relu,
-                                                                    k_per_slice, partial, status, st->vm_spin_limit);
+                                                                    k_per_slice, partial, status, poison, st->vm_spin_limit);
     return PIMHIP_OK;
 }
 
@@ -283,6 +295,20 @@ extern "C" int pimhip_gemv_status(void* stream, int* gave_up)
     if (it != st->workspaces.end() && it->second.status && *it->second.status != 0u) flags |= 1;
     if (st->static_status && *st->static_status != 0u) flags |= 2;
     *gave_up = flags;
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_gemv_fallbacks(void* stream, uint64_t* events)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!events) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "events must be non-null");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    uint64_t n = st->static_gave_up_events + ((st->static_status && *st->static_status != 0u) ? 1u : 0u);
+    auto it = st->workspaces.find(static_cast<hipStream_t>(stream));
+    if (it != st->workspaces.end()) n += it->second.gave_up_events + ((it->second.status && *it->second.status != 0u) ? 1u : 0u);
+    *events = n;
     return PIMHIP_OK;
 }
 

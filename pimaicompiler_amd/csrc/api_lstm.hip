@@ -59,7 +59,17 @@ struct PimHipLstmPlan {
     // lower layer's h per step ([max_seq_len][H] fp16) and the upper layer's projection rows ([max_seq_len][4H] fp32).
     unsigned char* xcd_pipe = nullptr;
     size_t xcd_pipe_boundary_bytes = 0;
+    // Waits of the persistent kernels that gave up, as far as the host has seen them (pimhip_lstm_plan_fallbacks).  Such a
+    // forward is completed by the workgroups themselves; after kLstmEventsBeforeSafe events the plan stops choosing
+    // kernels whose workgroups wait for one another.
+    unsigned long long gave_up_events = 0;
+    bool safe_only = false;
 };
+
+namespace
+{
+constexpr unsigned long long kLstmEventsBeforeSafe = 3;
+}
 
 namespace
 {
@@ -380,18 +390,26 @@ extern "C" int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned in
 extern "C" int pimhip_lstm_plan_status(PimHipLstmPlan* plan)
 {
     if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
-    if (*plan->abort_host != 0u) {
-        // Reported once, here or by the next pimhip_lstm_forward, whichever comes first.  The caller has synchronised
-        // the stream, so the kernel that set the word has ended and nothing sets it again after it is cleared.
-        const bool misplaced = *plan->abort_host == 2u;
+    if (*plan->abort_host == 2u) {
+        // The one event that leaves a forward undefined: two workgroups of the per-XCD kernel with the same rank on one XCD
+        // (some units then belong to nobody).  Reported once, here or by the next pimhip_lstm_forward.  The caller has
+        // synchronised the stream, so the kernel that set the word has ended.
         *plan->abort_host = 0u;
         plan->reset_exchange = true;
-        if (misplaced) return xcd_placement_failure(plan);
-        return fail(PIMHIP_ERR_TIMEOUT, "a bounded wait of the persistent LSTM kernel gave up: the results of that forward are undefined");
+        return xcd_placement_failure(plan);
     }
+    // A wait that gave up is no error: the workgroups completed that forward by themselves (pimhip_lstm_plan_fallbacks
+    // counts such events; the next forward outside a capture re-initialises the exchange).
     return PIMHIP_OK;
 }
 
+extern "C" int pimhip_lstm_plan_fallbacks(PimHipLstmPlan* plan, uint64_t* events, int* exchanging)
+{
+    if (!plan || !events) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan and events must be non-null");
+    *events = plan->gave_up_events + (*plan->abort_host == 1u ? 1u : 0u);
+    if (exchanging) *exchanging = (plan->safe_only || *events >= kLstmEventsBeforeSafe) ? 0 : 1;
+    return PIMHIP_OK;
+}
 
 extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y,
                                    void* hn, void* cn, int64_t seq_len, void* stream)
@@ -435,6 +453,18 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
         PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
         capturing = capture != hipStreamCaptureStatusNone;
     }
+    if (*plan->abort_host != 0u && !capturing) {
+        // A wait of an earlier sequence kernel of this plan gave up.  That forward was completed by the workgroups
+        // themselves and every sequence launch since has run self-sufficient (the abort word stays up on the device); here,
+        // outside any capture, the exchange is put back in order.  The word is cleared only after the stream has drained
+        // (calls sharing a plan are ordered on one stream), so that no kernel sets it again.
+        PIMHIP_HIP_CHECK(hipStreamSynchronize(s));
+        const bool misplaced = *plan->abort_host == 2u;
+        *plan->abort_host = 0u;
+        plan->reset_exchange = true;
+        if (misplaced) return xcd_placement_failure(plan);  // (the one event that leaves a forward undefined)
+        if (++plan->gave_up_events >= kLstmEventsBeforeSafe) plan->safe_only = true;
+    }
     // One step: the fused step kernel in every mode (the persistent kernel's hand-over of its step count to the next
     // launch needs two super-steps).
     // Automatic choice: one recurrence per XCD where its groups have something to run side by side or nothing to gain
@@ -448,33 +478,19 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     // (a stack with residual sums needs the pipeline kernel that makes them; where that one is not resident the stack runs
     // layer by layer on the other paths)
     const bool res_pipeline_missing = D == 1 && L >= 2 && plan->first_residual_layer < L && !plan->xcd_res_ok;
-    const bool use_xcd = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && !res_pipeline_missing &&
+    // (a plan whose waits have given up kLstmEventsBeforeSafe times runs one launch per step from then on: no workgroup of
+    // those kernels waits for another)
+    const bool use_xcd = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && !res_pipeline_missing && !plan->safe_only &&
                          (plan->mode == 4 || (plan->mode == 0 && xcd_pays));
-    const bool use_seq = !use_xcd && T >= 2 && T + kSeqMaxChains <= kSeqMaxT &&
+    const bool use_seq = !use_xcd && T >= 2 && T + kSeqMaxChains <= kSeqMaxT && !plan->safe_only &&
                          (plan->mode == 2 || plan->mode == 3 || (plan->mode == 0 && plan->seq_kernel_ok));
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
-    if (*plan->abort_host != 0u) {
-        // An earlier sequence kernel of this plan gave up a wait and nobody has asked pimhip_lstm_plan_status since:
-        // the error is reported here instead of being dropped, and nothing is launched.  The word is cleared only
-        // after the stream has drained (calls sharing a plan are ordered on one stream), so that kernel cannot set
-        // it again; the next forward starts from a re-initialised exchange buffer.
-        if (capturing)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "an earlier forward of this plan gave up a wait; recovering from that is not for a "
-                                                "graph: call pimhip_lstm_plan_status or one forward outside the capture first");
-        PIMHIP_HIP_CHECK(hipStreamSynchronize(s));
-        const bool misplaced = *plan->abort_host == 2u;
-        *plan->abort_host = 0u;
-        plan->reset_exchange = true;
-        if (misplaced) return xcd_placement_failure(plan);
-        return fail(PIMHIP_ERR_TIMEOUT, "an earlier forward of this plan gave up a wait of the persistent LSTM kernel: its results "
-                                        "are undefined (this call was not launched; the next one starts from a re-initialised exchange buffer)");
-    }
     if ((use_seq || use_xcd) && plan->reset_exchange) {
         // After a time-out or a change of the entry layout: re-arm the flag and bring the exchange buffer and its step
         // counters back to their initial state.
         if (capturing)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's exchange buffer has to be re-initialised (after a time-out or a change of "
-                                                "mode), which a graph must not record: run one forward outside the capture first");
+            return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's exchange buffer has to be re-initialised (after a change of mode), which a "
+                                                "graph must not record: run one forward outside the capture first");
         launch_fill_u32(plan->abort_flag, 1, 0u, s);
         if (plan->hx) {
             const size_t words = plan->hx_region_words * kSeqMaxChains;

@@ -225,9 +225,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_generic_kernel(const h
 // XCD's reducing blocks (the last slice), and a reducing block on one XCD waits at most for the other XCDs to get
 // through the producers dealt to them.  When other work holds CUs of one XCD (a resident sequence kernel on another
 // stream) that wait grows by as much as that XCD is held up.  It is bounded all the same: after `spin_limit` polls
-// of one record (none at all with a limit of 0, which is how a test forces the condition from the host) the lane
-// sets *status (host-visible) and goes on with what it has; the host then reports the failure and re-initialises
-// the records.
+// of one record (none at all with a limit of 0, which is how a test forces the condition from the host), or one second,
+// the lane gives up on the record and computes that slice's sums for its eight columns itself, with the producer's own
+// order of operations, so the result has the bits it would have had.  The record may still arrive later and would then
+// sit in the workspace as if it belonged to the next launch: the lane raises *poison (a device word the reducing blocks
+// of every launch look at) and *status (for the host), and until the host has refilled the records and cleared both,
+// reducing blocks do not look at records at all and compute every slice themselves: slow, but right.
 // ---------------------------------------------------------------------------------------------
 // Destinations of a VM product: the same result is stored to `count` buffers (the GNMT attention context goes
 // straight into three concatenation buffers, runtime/source/executor/op_executor/aten_ops_executor.cpp:694-737).
@@ -259,7 +262,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
                                                                  const half_t* __restrict__ bias,
                                                                  GemvOuts outs, int K, int N, long lda,
                                                                  int relu, int k_per_slice, float* partial,
-                                                                 unsigned int* status, unsigned int spin_limit)
+                                                                 unsigned int* status, unsigned int* poison,
+                                                                 unsigned int spin_limit)
 {
     static_assert(LPR == 16 || LPR == 32 || LPR == 64, "lanes per weight row");
     constexpr int RPW = 64 / LPR;          // rows per wavefront and load instruction
@@ -276,6 +280,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
     const bool col_ok = col0 < N;
     const int k_begin = blockIdx.y * k_per_slice;
     const int k_end = min(K, k_begin + k_per_slice);
+
+    // (asked for now by the blocks that will reduce, needed when they start to: it travels behind the block's own rows)
+    unsigned int poisoned = 0u;
+    if (gridDim.y > 1 && blockIdx.y == gridDim.y - 1) poisoned = __hip_atomic_load(poison, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     float acc[8];
 #pragma unroll
@@ -357,11 +365,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
             float4_t lo, hi;
             unsigned int spins = 0;
             unsigned long long t_first = 0ull;
-            while (true) {
+            bool have = false;
+            while (poisoned == 0u) {
                 if (spins > 0u && (spins & 255u) == 0u && wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
                 if (spins++ >= spin_limit) {
+                    __hip_atomic_store(poison, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                    lo = hi = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
                     break;
                 }
                 load32_device_scope_one(rec, lo, hi);
@@ -369,16 +378,42 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     ok = ok && __builtin_bit_cast(unsigned int, lo[j]) != kVmEmpty && __builtin_bit_cast(unsigned int, hi[j]) != kVmEmpty;
-                if (ok) break;
+                if (ok) {
+                    have = true;
+                    break;
+                }
+            }
+            if (have) {
+                const float e = __builtin_bit_cast(float, kVmEmpty);
+                const float empty[8] = {e, e, e, e, e, e, e, e};
+                store32_device_scope(rec, empty);
+            } else {
+                // Slice sl's sums for these eight columns, as its own block makes them: every row group's rows in ascending
+                // order, then the groups in order.
+                const half_t* a = A + col0;
+                const int ks_begin = sl * k_per_slice, ks_end = min(K, ks_begin + k_per_slice);
+                float v[8];
+                for (int g = 0; g < GROUPS; ++g) {
+                    float part[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) part[j] = 0.0f;
+                    for (int k = ks_begin + g; k < ks_end; k += STEP) {
+                        const half8_t ar = *reinterpret_cast<const half8_t*>(a + (long)k * lda);
+                        const float xr = (float)x[k];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) part[j] = fmaf((float)ar[j], xr, part[j]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = g == 0 ? part[j] : v[j] + part[j];
+                }
+                lo = float4_t{v[0], v[1], v[2], v[3]};
+                hi = float4_t{v[4], v[5], v[6], v[7]};
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 acc[j] += lo[j];
                 acc[4 + j] += hi[j];
             }
-            const float e = __builtin_bit_cast(float, kVmEmpty);
-            const float empty[8] = {e, e, e, e, e, e, e, e};
-            store32_device_scope(rec, empty);
         }
     }
     __syncthreads();  // the first lanes have read `red` above before it is written again

@@ -18,6 +18,7 @@
 #pragma once
 
 #include "device_common.h"
+#include "lstm_solo.h"
 
 namespace pimhip
 {
@@ -158,9 +159,12 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
 // sequence of flag bits per slot stays alternating across launches.  After a time-out the host clears the buffer and
 // sets the counter back to 2.
 //
-// Every wait is bounded: after `spin_limit` polls a lane raises *abort_flag and stops waiting; lanes poll
-// the flag every 256 spins and stop waiting once it is set.  The kernel then runs to the end with
-// undefined results and the host reports a time-out.
+// Every wait is bounded: after `spin_limit` polls (or one second) a lane raises *abort_flag and stops waiting; lanes poll
+// the flag every 256 spins and stop waiting once it is set.  A block in which a lane stopped waiting publishes nothing
+// from then on (so that no other block takes values for real that were computed from stale ones), leaves the loop of
+// super-steps and computes its chains by itself (lstm_solo.h): slower, but the call's result is what it would have been.
+// The abort word stays up: later launches of the plan start in that self-sufficient mode until the host has re-initialised
+// the exchange buffer.
 // ---------------------------------------------------------------------------------------------
 static constexpr int kSeqUnits = 4;        // hidden units per block, one per wavefront
 static constexpr int kSeqMaxH = 1024;      // 64 lanes x 16 columns
@@ -234,6 +238,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
     static_assert(NC >= 1 && NC <= kSeqMaxChains && 2 * NW <= kSeqEntryWords, "an entry is 64 bytes");
     __shared__ __align__(16) half_t hbuf[2][NC][MAXH];       // published h per chain, double buffered by parity
     __shared__ __align__(16) unsigned short pub[NC][UNITS];  // this block's next entry: chain k, wavefront w
+    __shared__ int block_gave_up;                            // set by a lane whose wait gave up; read by all after the step's first barrier
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -249,6 +254,10 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
     // launch stored it from another XCD.  The value is first needed when super-step 0 publishes.
     const unsigned int g_base = __builtin_amdgcn_readfirstlane(
         __hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    // A wait of an earlier launch gave up and the host has not re-initialised the exchange buffer since (it may hold that
+    // launch's values): nothing is exchanged, every block computes its chains by itself.
+    const bool poisoned = __builtin_amdgcn_readfirstlane(__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) != 0u;
+    if (tid == 0) block_gave_up = poisoned ? 1 : 0;
 
     // ---- weights into registers: per chain the four gate rows of unit j, columns 16 * lane .. + 15 ----
     // Accumulator slot v holds gate {i, g, f, o}[v]: the transpose-sum below then leaves gate k in lane k.
@@ -309,6 +318,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
     }
     bool gave_up = false;
 
+    bool alone = poisoned;  // the block has to go on by itself (a wait gave up)
     auto super_step = [&](const int tau, float (&xp_slot)[NC]) __attribute__((always_inline)) {
         half_t(*hb)[MAXH] = hbuf[tau & 1];
 
@@ -344,6 +354,7 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
                         __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                         gave_up = true;
                     }
+                    if (gave_up) block_gave_up = 1;  // (its own wait or another block's: this block's h would be made from stale values)
                 }
             }
 #pragma unroll
@@ -370,6 +381,9 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             }
         }
         __syncthreads();
+        // Written only in front of this barrier: every thread reads the same value, and the block leaves together.
+        alone = block_gave_up != 0;
+        if (!alone) {
 
         // ---- 2. gates of all chains ----
         // Written without branches and phase by phase over the chains, so that the chains' dependency chains
@@ -483,14 +497,61 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             for (int k = 0; k + 1 < NW; k += 2) store16_device_scope(dst + k, src[k], src[k + 1]);
             if (NW & 1) __hip_atomic_store(dst + (NW - 1), src[NW - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        }  // (!alone)
     };
 
     int tau = 0;
-    for (; tau + 1 < n_super; tau += 2) {
+    for (; !alone && tau + 1 < n_super; tau += 2) {
         super_step(tau, xp_even);
-        super_step(tau + 1, xp_odd);
+        if (!alone) super_step(tau + 1, xp_odd);
     }
-    if (tau < n_super) super_step(tau, xp_even);
+    if (!alone && tau < n_super) super_step(tau, xp_even);
+    if (alone) {
+        // ---- self-sufficient: this block's units of every chain, from the call's inputs, by this block alone ----
+        SoloStack st;
+        st.y_stride = p.y_stride;
+        st.H = H;
+        st.T = T;
+        st.res_in0 = nullptr;
+        const int u_begin = min(blockIdx.x * UNITS, H), u_end = min(u_begin + UNITS, H);
+        auto layer_of = [&](int k) {
+            SoloLayer ly;
+            ly.w_hh = p.chain[k].w_hh;
+            ly.w_ih = nullptr;
+            ly.bsum = nullptr;
+            ly.h0 = p.chain[k].h0;
+            ly.c0 = p.chain[k].c0;
+            ly.y = p.chain[k].y;
+            ly.hn = p.chain[k].hn;
+            ly.cn = p.chain[k].cn;
+            ly.residual = 0;
+            ly.u_begin = u_begin;
+            ly.u_end = u_end;
+            return ly;
+        };
+        if (WAVEFRONT) {
+            st.n = NC;
+            st.xproj = p.chain[0].xproj;
+            st.reverse = 0;
+#pragma unroll
+            for (int k = 0; k < NC; ++k) {
+                st.layer[k] = layer_of(k);
+                if (k > 0) {
+                    st.layer[k].w_ih = p.chain[k].w_ih;
+                    st.layer[k].bsum = p.chain[k].bsum;
+                }
+            }
+            lstm_solo_stack<64 * UNITS, NC, MAXH>(st);
+        } else {
+            for (int k = 0; k < NC; ++k) {  // independent chains, one after the other
+                st.n = 1;
+                st.xproj = p.chain[k].xproj;
+                st.reverse = p.chain[k].reverse;
+                st.layer[0] = layer_of(k);
+                lstm_solo_stack<64 * UNITS, 1, MAXH>(st);
+            }
+        }
+    }
     // Block 0 has finished its last super-step, for which (n_super >= 2, the launcher's condition) it needed what every
     // block published one super-step earlier: every block has read the counter by now.  The next launch reads it after
     // this one has ended.

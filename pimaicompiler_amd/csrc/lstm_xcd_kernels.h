@@ -22,7 +22,8 @@
 // cache is write-through, so they land in the XCD's L2) and read with non-temporal loads (a line read that way is
 // dropped from the per-CU cache at once, so the next poll goes to the L2 again).  Nothing in the results depends on
 // that cache behaviour: a stale piece fails its flag check and is polled again; only the time a poll takes does.
-// Every wait is bounded (spin_limit polls, then the abort flag, as in lstm_seq_f16_kernel).
+// Every wait is bounded (spin_limit polls, then the abort flag, as in lstm_seq_f16_kernel), and as there a workgroup one
+// of whose waits gave up publishes nothing from then on and computes its units of the recurrence by itself at the end.
 //
 // A stack of unidirectional layers runs as a pipeline over the XCDs: layer k's recurrence (group R_k) on one XCD, and for
 // k >= 1 a second group P_k on another XCD that holds W_ih of layer k and turns every h of layer k - 1 into layer k's
@@ -45,6 +46,7 @@
 #include <type_traits>
 
 #include "lstm_kernels.h"
+#include "lstm_solo.h"
 
 namespace pimhip
 {
@@ -149,6 +151,9 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
     __shared__ __align__(16) float xring[kXcdWaves][32][4][4];  // per wavefront: [step & 31][gate][unit] projection terms
     __shared__ __align__(16) unsigned long long hout[2][kXcdWaves];  // the workgroup's 32 new h values, for the layer above
     __shared__ unsigned short in_ring[2][kXcdUnitsPerBlock];        // RES: the layer's own input of the last two steps, for the sums
+    // Raised by a wavefront one of whose waits gave up, always in front of a step's barrier, and read by all right behind
+    // it: the workgroup then leaves the loop of steps together, publishes nothing more and computes its units by itself.
+    __shared__ int block_gave_up;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -179,6 +184,10 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
     bool gave_up = false;
     const unsigned int g_base = __builtin_amdgcn_readfirstlane(
         __hip_atomic_load(p.g_counter + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    // A wait of an earlier launch gave up and the host has not re-initialised the exchange since: nothing is exchanged in
+    // this launch, every workgroup of a recurrence computes its units by itself.
+    const bool poisoned = __builtin_amdgcn_readfirstlane(__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) != 0u;
+    if (tid == 0) block_gave_up = poisoned ? 1 : 0;
     unsigned int* region = p.hx + (long)k * kXcdRegionWords;
     // This launch's mark on (XCD, rank): the counter value is new in every launch of the plan.  Found already there, two
     // workgroups of this launch share the rank, so another rank of the group is empty: not a rotation.
@@ -256,6 +265,7 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
 
     if (is_proj) {
         // ================= P group: xproj rows of layer k from the h of layer k - 1, step by step =================
+        if (poisoned) return;  // (the recurrence it feeds makes its own rows then)
         const float bias = pj.bsum[(long)my_gate * H + uc];
         float* dst = pj.xp_out + (long)my_gate * H + uc;
         unsigned long long lo = 0ull, hi = 0ull;  // this lane's piece of the step ahead
@@ -277,7 +287,9 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
                 const u64x2 both = {lo, hi};
                 *reinterpret_cast<half8_t*>(hb + piece * 8) = __builtin_bit_cast(half8_t, both);
             }
+            if (gave_up) block_gave_up = 1;
             lds_barrier();
+            if (block_gave_up) return;  // rows made from a stale h must not reach the recurrence: it will make its own
             if (polls && t + 1 < T) {
                 // the step ahead, in flight while this one is multiplied (tested at the top of the next iteration)
                 const unsigned long long* nxt = reinterpret_cast<const unsigned long long*>(pj.seq_in + (long)(t + 1) * H + piece * 8);
@@ -418,7 +430,9 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
             }
             *reinterpret_cast<half8_t*>(hb + piece * 8) = hv;
         }
+        if (gave_up) block_gave_up = 1;
         lds_barrier();
+        if (block_gave_up) break;  // (the same value in every thread: it is written in front of barriers only)
         if (polled && fetcher && s + 2 < T) {
             xp_ahead = xp_bits_at(s + 2);
             xp_ahead_other = __hip_atomic_load(xp_other + (long)(s + 2) * 4 * H, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -472,12 +486,15 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
             pw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)pb16, 16 * i) << (16 * i);
             if (emits) sw |= (unsigned long long)(unsigned int)__builtin_amdgcn_readlane((int)sb16, 16 * i) << (16 * i);
         }
+        // (a wavefront one of whose waits gave up after this step's barrier has made its h from stale values: it keeps them
+        // to itself, and the group's other members stop at their next wait)
+        const bool wave_gave_up = __builtin_amdgcn_ballot_w64(gave_up) != 0ull;
         if (lane == 0) {
             const unsigned int g = g_base + (unsigned int)s;
             const unsigned long long flag = ((g >> 1) & 1u) ? 0x4000400040004000ull : 0ull;
             // units past H publish zeros with the flag, so that every piece of a member's entry validates
             unsigned char* dst = reinterpret_cast<unsigned char*>(region + ((long)(g & 1u) * kXcdMembers + rank) * kXcdEntryWords) + wave * 8;
-            store8_plain(dst, (units_ok ? pw : 0ull) | flag);
+            if (!wave_gave_up) store8_plain(dst, (units_ok ? pw : 0ull) | flag);
             if (!res && units_ok && ch.y) *reinterpret_cast<unsigned long long*>(ch.y + (long)t * p.y_stride + u0) = yw;
             if (emits) hout[s & 1][wave] = sw;
         }
@@ -486,17 +503,22 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
             ch.cn[my_unit] = (half_t)c_new;
         }
     }
-    if (emits) {
-        if (sums) in_ring[(T - 1) & 1][lane & 31] = in_ahead;
-        lds_barrier();
+    if (emits && sums) in_ring[(T - 1) & 1][lane & 31] = in_ahead;
+    if (gave_up) block_gave_up = 1;
+    lds_barrier();
+    if (emits && !block_gave_up) {
         if (!res && wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) emit(T - 1);
         if (sums) emit_sum(T - 1);
+        if (gave_up) block_gave_up = 1;  // (the last sum's own wait)
     }
+    lds_barrier();
     };
     const bool polled_rt = PIPE && ch.xproj_polled != 0;
     const bool feeds_rt = PIPE && ch.seq_out != nullptr;
     const bool res_rt = RES && ch.res_in != nullptr;
-    if (RES && res_rt) {
+    if (poisoned) {
+        // (nothing is exchanged)
+    } else if (RES && res_rt) {
         if (!polled_rt && !feeds_rt) recurrence(std::false_type{}, std::false_type{}, std::true_type{});
         else if (!polled_rt) recurrence(std::false_type{}, std::true_type{}, std::true_type{});
         else if (!feeds_rt) recurrence(std::true_type{}, std::false_type{}, std::true_type{});
@@ -505,6 +527,39 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
     else if (!polled_rt) recurrence(std::false_type{}, std::true_type{}, std::false_type{});
     else if (!feeds_rt) recurrence(std::true_type{}, std::false_type{}, std::false_type{});
     else recurrence(std::true_type{}, std::true_type{}, std::false_type{});
+    if (block_gave_up) {
+        // ---- self-sufficient: this workgroup's units of chain k, from the call's inputs, by this workgroup alone: the layers
+        // below it in the launch are recomputed on the way (lstm_solo.h) ----
+        SoloStack st;
+        st.y_stride = p.y_stride;
+        st.H = H;
+        st.T = T;
+        const int first = PIPE ? 0 : k;  // independent chains (the two directions of a layer) have their own projection rows
+        st.n = k - first + 1;
+        st.xproj = p.chain[first].xproj;
+        st.res_in0 = RES ? p.chain[first].res_in : nullptr;
+        st.reverse = ch.reverse;
+#pragma unroll
+        for (int j = 0; j < kXcdMaxChains; ++j) {
+            if (first + j > k) break;
+            const XcdChain& cj = p.chain[first + j];
+            SoloLayer& ly = st.layer[j];
+            ly.w_hh = cj.w_hh;
+            ly.w_ih = j > 0 ? p.proj[first + j - 1].w_ih : nullptr;
+            ly.bsum = j > 0 ? p.proj[first + j - 1].bsum : nullptr;
+            ly.h0 = cj.h0;
+            ly.c0 = cj.c0;
+            ly.residual = (RES && cj.res_in != nullptr) ? 1 : 0;
+            const bool mine = first + j == k;
+            ly.y = mine ? cj.y : nullptr;
+            ly.hn = cj.hn;
+            ly.cn = cj.cn;
+            ly.u_begin = mine ? min(rank * kXcdUnitsPerBlock, H) : 0;
+            ly.u_end = mine ? min((rank + 1) * kXcdUnitsPerBlock, H) : 0;
+        }
+        lstm_solo_stack<kXcdThreads, PIPE ? kXcdMaxChains : 1, kXcdMaxH>(st);
+        return;
+    }
     // Rank 0 has finished its last step, for which (T >= 2) it needed what every member published one step earlier:
     // every member has read the counter by now.
     if (rank == 0 && tid == 0)

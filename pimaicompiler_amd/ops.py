@@ -85,24 +85,30 @@ def _stream_handle(stream):
 
 
 def gemv_status(stream=None):
-    """After the caller has synchronised `stream`: has a sliced I_X_W product given up waiting for partial sums since the
-    workspace was last re-initialised?  Returns (on_this_stream, static_entry_point).  The next sliced product on the
-    stream raises in any case; this is for a caller that wants to know before it uses the result."""
+    """After the caller has synchronised `stream`: has a reducing block of a sliced I_X_W product given up waiting for
+    partial sums since the workspace was last put in order?  Returns (on_this_stream, static_entry_point).  Such a product
+    is completed by the block itself; this is for a caller that wants to know."""
     flags = ctypes.c_int(0)
     _check(L.load().pimhip_gemv_status(_stream_handle(stream), ctypes.byref(flags)))
     return bool(flags.value & 1), bool(flags.value & 2)
 
 
+def gemv_fallbacks(stream=None):
+    """How many times a reducing block of a sliced I_X_W product has given up a wait so far, on `stream` plus through the
+    static entry point (pimhip_gemv_fallbacks).  Ask after synchronising the stream."""
+    n = ctypes.c_uint64(0)
+    _check(L.load().pimhip_gemv_fallbacks(_stream_handle(stream), ctypes.byref(n)))
+    return int(n.value)
+
+
 def synchronize_and_check(stream=None):
-    """Synchronises `stream` (torch's current one by default) and raises if a sliced I_X_W product on it gave up."""
+    """Synchronises `stream` (torch's current one by default).  Kept for callers of the earlier interface, where a sliced
+    I_X_W product that gave up a wait left an undefined result and this raised: nothing is left undefined any more."""
     s = stream if isinstance(stream, torch.cuda.Stream) else (torch.cuda.current_stream() if stream is None else None)
     if s is not None:
         s.synchronize()
     else:
         torch.cuda.synchronize()
-    on_stream, static = gemv_status(stream)
-    if on_stream or static:
-        raise NNRuntimeException("a sliced I_X_W product gave up waiting for partial sums: its result is undefined")
 
 
 def set_gemv_spin_limit(spin_limit):
@@ -568,9 +574,20 @@ class LstmPlan:
         _check(L.load().pimhip_lstm_plan_set_spin_limit(self._handle, limit))
 
     def status(self):
-        """Raises NNRuntimeException if the last forward's persistent kernel gave up a wait.  Synchronises."""
+        """Synchronises.  Raises NNRuntimeException only for the one event that leaves a forward undefined (the per-XCD
+        kernel's workgroups not dealt to the XCDs in rotation); a wait that gives up is made good inside the launch and
+        counted by fallbacks()."""
         torch.cuda.synchronize(self.device)
         _check(L.load().pimhip_lstm_plan_status(self._handle))
+
+    def fallbacks(self):
+        """(events, exchanging): waits of the persistent kernels that have given up in forwards of this plan so far, and
+        whether sequence calls still use those kernels (False once the plan runs one launch per step for good).
+        Synchronises (pimhip_lstm_plan_fallbacks)."""
+        torch.cuda.synchronize(self.device)
+        events, exchanging = ctypes.c_uint64(0), ctypes.c_int(0)
+        _check(L.load().pimhip_lstm_plan_fallbacks(self._handle, ctypes.byref(events), ctypes.byref(exchanging)))
+        return int(events.value), bool(exchanging.value)
 
     def forward(self, x2d, h0, c0, stream=None, out=None):
         """x2d [T, I]; h0, c0 [L*D, H] (any shape with those elements).  Returns y [T, D*H], hn, cn [L*D, H].
