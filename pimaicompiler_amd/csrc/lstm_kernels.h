@@ -381,9 +381,10 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             }
         }
         __syncthreads();
-        // Written only in front of this barrier: every thread reads the same value, and the block leaves together.
-        alone = block_gave_up != 0;
-        if (!alone) {
+        // Written only in front of this barrier: every thread reads the same value, and the block leaves together.  Asked
+        // for here, with the reads of h, and looked at where the block would publish: the step's arithmetic does not wait
+        // for it (a step that should not have been made is made on stale values and dropped).
+        const int gave_up_in_this_step = __builtin_amdgcn_readfirstlane(block_gave_up);
 
         // ---- 2. gates of all chains ----
         // Written without branches and phase by phase over the chains, so that the chains' dependency chains
@@ -489,7 +490,8 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             }
         }
         __syncthreads();
-        if (tid == 0) {
+        alone = gave_up_in_this_step != 0;
+        if (tid == 0 && !alone) {
             const unsigned int g = g_base + (unsigned int)tau;
             unsigned long long* dst = reinterpret_cast<unsigned long long*>(p.hx + ((long)(g & 1u) * nb + blockIdx.x) * kSeqEntryWords);
             const unsigned long long* src = reinterpret_cast<const unsigned long long*>(&pub[0][0]);
@@ -497,7 +499,6 @@ __global__ __launch_bounds__(64 * UNITS) void lstm_seq_f16_kernel(LstmSeqArgs p)
             for (int k = 0; k + 1 < NW; k += 2) store16_device_scope(dst + k, src[k], src[k + 1]);
             if (NW & 1) __hip_atomic_store(dst + (NW - 1), src[NW - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        }  // (!alone)
     };
 
     int tau = 0;

@@ -289,7 +289,7 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
             }
             if (gave_up) block_gave_up = 1;
             lds_barrier();
-            if (block_gave_up) return;  // rows made from a stale h must not reach the recurrence: it will make its own
+            const int dead = __builtin_amdgcn_readfirstlane(block_gave_up);  // (asked for with the reads of h, looked at where the row would leave)
             if (polls && t + 1 < T) {
                 // the step ahead, in flight while this one is multiplied (tested at the top of the next iteration)
                 const unsigned long long* nxt = reinterpret_cast<const unsigned long long*>(pj.seq_in + (long)(t + 1) * H + piece * 8);
@@ -305,6 +305,7 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
                 for (int g = 0; g < 4; ++g) acc[g] = dot8(w[g][c], hv, acc[g]);
             }
             const float v = row16_transpose_sum4(acc, lane) + bias;
+            if (dead) return;  // rows made from a stale h must not reach the recurrence: it will make its own
             if (units_ok && (lane & 3) == 0)
                 __hip_atomic_store(reinterpret_cast<unsigned int*>(dst + (long)t * 4 * H), __builtin_bit_cast(unsigned int, v), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
@@ -432,18 +433,20 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
         }
         if (gave_up) block_gave_up = 1;
         lds_barrier();
-        if (block_gave_up) break;  // (the same value in every thread: it is written in front of barriers only)
+        // (the same value in every thread: it is written in front of barriers only.  Asked for here, with the reads of h,
+        // and looked at where values would leave the workgroup: the step's arithmetic does not wait for it)
+        const int dead = __builtin_amdgcn_readfirstlane(block_gave_up);
         if (polled && fetcher && s + 2 < T) {
             xp_ahead = xp_bits_at(s + 2);
             xp_ahead_other = __hip_atomic_load(xp_other + (long)(s + 2) * 4 * H, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         // The previous step's h of the whole workgroup (gathered in LDS before the barrier) goes to the layer above, from a
         // wavefront that does not poll.
-        if (!res && feeds && s > 0 && wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H) emit(s - 1);
+        if (!res && feeds && s > 0 && wave == 4 && lane < 4 && rank * kXcdUnitsPerBlock + lane * 8 < H && !dead) emit(s - 1);
         if (sums) {
             in_ahead = __hip_atomic_load(reinterpret_cast<const unsigned short*>(ch.res_in) + (long)s * H + eu, __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
-            if (s > 0) emit_sum(s - 1);
+            if (s > 0 && !dead) emit_sum(s - 1);
         }
 
         // ---- 2. the four gate rows of this row of lanes' unit
@@ -494,7 +497,7 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
             const unsigned long long flag = ((g >> 1) & 1u) ? 0x4000400040004000ull : 0ull;
             // units past H publish zeros with the flag, so that every piece of a member's entry validates
             unsigned char* dst = reinterpret_cast<unsigned char*>(region + ((long)(g & 1u) * kXcdMembers + rank) * kXcdEntryWords) + wave * 8;
-            if (!wave_gave_up) store8_plain(dst, (units_ok ? pw : 0ull) | flag);
+            if (!wave_gave_up && !dead) store8_plain(dst, (units_ok ? pw : 0ull) | flag);
             if (!res && units_ok && ch.y) *reinterpret_cast<unsigned long long*>(ch.y + (long)t * p.y_stride + u0) = yw;
             if (emits) hout[s & 1][wave] = sw;
         }
@@ -502,6 +505,7 @@ __device__ __forceinline__ void lstm_xcd_body(const LstmXcdArgs& p)
             ch.hn[my_unit] = h;
             ch.cn[my_unit] = (half_t)c_new;
         }
+        if (dead) break;  // (a step made on stale values: nothing of it has left the workgroup)
     }
     if (emits && sums) in_ring[(T - 1) & 1][lane & 31] = in_ahead;
     if (gave_up) block_gave_up = 1;
