@@ -211,11 +211,24 @@ int pimhip_lstm_plan_set_spin_limit(PimHipLstmPlan* plan, unsigned int spin_limi
 /* Selects how pimhip_lstm_forward runs the recurrence: 0 = automatic, 1 = one fused launch per step,
  * 2 = persistent sequence kernel (hidden_size up to 2048; fails with PIMHIP_ERR_UNSUPPORTED otherwise), 3 = as 2 but with
  * four hidden units per block in every launch (2 runs a single unidirectional layer with eight), 4 = every recurrence
- * (layer and direction) on one XCD of the part, the two directions of a layer side by side on two (hidden_size up to
- * 1024 on a device of 8 XCDs x 32 CUs; PIMHIP_ERR_UNSUPPORTED otherwise).  Automatic takes 4 for bidirectional layers
- * and for a single unidirectional layer when the sequence is long enough to pay for it, 2 for unidirectional stacks
- * (a wavefront over the layers), 1 where neither fits.  A call with seq_len 1 runs the fused step launch in every mode. */
+ * (layer and direction) on one XCD of the part, the two directions of a layer side by side on two, the layers of a
+ * unidirectional stack as a pipeline (hidden_size up to 1024 on a device of 8 XCDs x 32 CUs; PIMHIP_ERR_UNSUPPORTED
+ * otherwise).  A call with seq_len 1 runs the fused step launch in every mode.
+ * Automatic mode measures: the first pimhip_lstm_forward of a plan with a sequence length in [2^b, 2^(b+1)) that is issued
+ * outside a graph capture runs the call under every mode that takes it (a few runs each, timed with HIP events: that
+ * call synchronises its stream and costs a few times its usual duration), and the plan keeps the fastest for that range of
+ * lengths; as the reference does with its two libraries on the first inference
+ * (runtime/source/executor/stream_executor.cpp:312-339).  Until then (calls inside a capture, or after
+ * pimhip_lstm_plan_set_measure(plan, 0)) thresholds measured once on MI355X choose: 4 for bidirectional layers and for a
+ * single unidirectional layer when the sequence is long enough to pay for it, 4 or 2 for unidirectional stacks, 1 where
+ * neither fits. */
 int pimhip_lstm_plan_set_mode(PimHipLstmPlan* plan, int mode);
+
+/* No counterpart in the reference beyond the above.  enabled == 0: automatic mode stops measuring and forgets what it
+ * measured (thresholds choose); != 0 (the default): it measures as described.  pimhip_lstm_plan_measured_mode: the mode
+ * automatic mode uses for sequences of seq_len (>= 2) steps, 0 if that range of lengths has not been measured yet. */
+int pimhip_lstm_plan_set_measure(PimHipLstmPlan* plan, int enabled);
+int pimhip_lstm_plan_measured_mode(PimHipLstmPlan* plan, int64_t seq_len, int* mode);
 
 /* No counterpart in aten::lstm.  Layers first_residual_layer .. num_layers - 1 of a unidirectional stack hand up and
  * return out_t = h_t + in_t (fp16, one rounding) instead of h_t, in_t being the layer's own input: the wiring of the GNMT

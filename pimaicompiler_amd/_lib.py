@@ -53,6 +53,8 @@ SIGNATURES = {
     "pimhip_lstm_plan_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), c_int_p]),
     "pimhip_lstm_plan_set_mode": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
     "pimhip_lstm_plan_set_residual": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "pimhip_lstm_plan_set_measure": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int]),
+    "pimhip_lstm_plan_measured_mode": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, c_int_p]),
     "pimhip_lstm_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "pimhip_decoder_plan_create": (ctypes.c_int, [c_void_pp, c_void_pp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,

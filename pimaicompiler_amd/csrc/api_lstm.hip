@@ -64,6 +64,11 @@ struct PimHipLstmPlan {
     // kernels whose workgroups wait for one another.
     unsigned long long gave_up_events = 0;
     bool safe_only = false;
+    // Automatic mode: the kernel family measured fastest on this plan for sequence lengths in [2^b, 2^(b+1)), 0 = not
+    // measured yet (pimhip_lstm_forward measures on the first eager call of a bucket; see measured_mode below).
+    unsigned char measured_mode[32] = {};
+    bool measure = true;             // pimhip_lstm_plan_set_measure
+    hipEvent_t tune_event[2] = {nullptr, nullptr};
 };
 
 namespace
@@ -96,6 +101,8 @@ int destroy_plan_locked(PimHipLstmPlan* plan)
     if (plan->xcd_pipe) hipFree(plan->xcd_pipe);
     if (plan->abort_flag) hipFree(plan->abort_flag);
     if (plan->abort_host) hipHostFree(plan->abort_host);
+    for (hipEvent_t e : plan->tune_event)
+        if (e) hipEventDestroy(e);
     if (prev >= 0) hipSetDevice(prev);
     for (size_t i = 0; i < g_plans.size(); ++i) {
         if (g_plans[i] == plan) {
@@ -376,6 +383,7 @@ extern "C" int pimhip_lstm_plan_set_residual(PimHipLstmPlan* plan, int first_res
                 return fail(PIMHIP_ERR_INVALID_ARGUMENT, "layer %d has input width %lld and hidden size %lld: its input cannot be added to its output",
                             l, (long long)plan->cells[(size_t)l].in_w, (long long)plan->hidden);
     }
+    if (plan->first_residual_layer != first_residual_layer) memset(plan->measured_mode, 0, sizeof(plan->measured_mode));
     plan->first_residual_layer = first_residual_layer;
     return PIMHIP_OK;
 }
@@ -411,8 +419,15 @@ extern "C" int pimhip_lstm_plan_fallbacks(PimHipLstmPlan* plan, uint64_t* events
     return PIMHIP_OK;
 }
 
-extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y,
-                                   void* hn, void* cn, int64_t seq_len, void* stream)
+namespace
+{
+int measure_modes(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn, void* cn,
+                  int64_t seq_len, void* stream, int bucket, bool xcd_takes_it, bool seq_takes_it);
+
+// pimhip_lstm_forward with the plan's mode replaced by `forced_mode` when that is not negative (the measurement of
+// automatic mode runs the call under every kernel family that takes it).
+int lstm_forward_impl(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn, void* cn,
+                      int64_t seq_len, void* stream, int forced_mode)
 {
     DeviceState* st = nullptr;
     int rc = current_device_state(&st);
@@ -480,10 +495,24 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
     const bool res_pipeline_missing = D == 1 && L >= 2 && plan->first_residual_layer < L && !plan->xcd_res_ok;
     // (a plan whose waits have given up kLstmEventsBeforeSafe times runs one launch per step from then on: no workgroup of
     // those kernels waits for another)
-    const bool use_xcd = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && !res_pipeline_missing && !plan->safe_only &&
-                         (plan->mode == 4 || (plan->mode == 0 && xcd_pays));
+    const bool xcd_takes_it = T >= 2 && T <= kSeqMaxT - 2 && plan->xcd_ok && !res_pipeline_missing && !plan->safe_only;
+    const bool seq_takes_it = T >= 2 && T + kSeqMaxChains <= kSeqMaxT && plan->seq_kernel_ok && !plan->safe_only;
+    int mode = forced_mode >= 0 ? forced_mode : plan->mode;
+    if (mode == 0 && T >= 2) {
+        // Automatic: what was measured fastest on this plan for sequences of about this length; failing that (nothing
+        // measured yet and no way to measure now) the thresholds above.
+        int bucket = 0;
+        while ((T >> (bucket + 1)) != 0 && bucket < 31) ++bucket;
+        if (plan->measured_mode[bucket] == 0 && plan->measure && !capturing && forced_mode < 0 && (xcd_takes_it || seq_takes_it)) {
+            rc = measure_modes(plan, x, h0, c0, y, hn, cn, seq_len, stream, bucket, xcd_takes_it, seq_takes_it);
+            if (rc != PIMHIP_OK) return rc;
+            return PIMHIP_OK;  // (the last of the measured runs was the call, under the mode that won)
+        }
+        if (plan->measured_mode[bucket] != 0) mode = plan->measured_mode[bucket];
+    }
+    const bool use_xcd = xcd_takes_it && (mode == 4 || (mode == 0 && xcd_pays));
     const bool use_seq = !use_xcd && T >= 2 && T + kSeqMaxChains <= kSeqMaxT && !plan->safe_only &&
-                         (plan->mode == 2 || plan->mode == 3 || (plan->mode == 0 && plan->seq_kernel_ok));
+                         (mode == 2 || mode == 3 || (mode == 0 && plan->seq_kernel_ok));
     if (use_seq && !plan->seq_kernel_ok) return fail(PIMHIP_ERR_UNSUPPORTED, "persistent sequence kernel not available for this plan");
     if ((use_seq || use_xcd) && plan->reset_exchange) {
         // After a time-out or a change of the entry layout: re-arm the flag and bring the exchange buffer and its step
@@ -725,7 +754,7 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
                     case 1:
                         // A single chain exchanges 2 bytes per unit: eight units per block still fit one 16-byte
                         // store and one 16-byte load per entry, and half as many blocks finish a round sooner.
-                        if (plan->seq_units8_ok && plan->mode != 3)
+                        if (plan->seq_units8_ok && mode != 3)
                             lstm_seq_f16_kernel<1, true, 8><<<dim3((unsigned)((H + 7) / 8)), dim3(512), 0, s>>>(a);
                         else
                             lstm_seq_f16_kernel<1, true><<<grid, block, 0, s>>>(a);
@@ -781,5 +810,70 @@ extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const vo
             layer_in = layer_out;
         }
     }
+    return PIMHIP_OK;
+}
+
+// Runs the call once under every kernel family that takes it and keeps, for sequence lengths of this bucket, the fastest:
+// the counterpart of the reference timing both of its libraries on the first inference and keeping the faster per layer
+// (runtime/source/executor/stream_executor.cpp:312-339).  Every run computes the same call into the same outputs; the last
+// one is made under the winner, so the caller gets that mode's bits.  Synchronises `stream` (HIP events).
+int measure_modes(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y, void* hn, void* cn,
+                  int64_t seq_len, void* stream, int bucket, bool xcd_takes_it, bool seq_takes_it)
+{
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (hipEvent_t& e : plan->tune_event)
+        if (!e) PIMHIP_HIP_CHECK(hipEventCreate(&e));
+    int candidates[3], n = 0;
+    if (xcd_takes_it) candidates[n++] = 4;
+    if (seq_takes_it) candidates[n++] = 2;
+    if (seq_len <= 8) candidates[n++] = 1;  // (one launch per step only ever wins on the shortest sequences)
+    int best = candidates[0];
+    float best_ms = -1.0f;
+    const unsigned long long events_before = plan->gave_up_events;
+    for (int i = 0; i < n && n > 1; ++i) {
+        float ms_min = -1.0f;
+        for (int rep = 0; rep < 3; ++rep) {  // the first run of a mode also loads its code and warms the weights
+            PIMHIP_HIP_CHECK(hipEventRecord(plan->tune_event[0], s));
+            const int rc = lstm_forward_impl(plan, x, h0, c0, y, hn, cn, seq_len, stream, candidates[i]);
+            if (rc != PIMHIP_OK) return rc;
+            PIMHIP_HIP_CHECK(hipEventRecord(plan->tune_event[1], s));
+            PIMHIP_HIP_CHECK(hipEventSynchronize(plan->tune_event[1]));
+            float ms = 0.0f;
+            PIMHIP_HIP_CHECK(hipEventElapsedTime(&ms, plan->tune_event[0], plan->tune_event[1]));
+            if (rep > 0 && (ms_min < 0.0f || ms < ms_min)) ms_min = ms;
+        }
+        // (a mode in which a wait gave up while it was measured is not a candidate)
+        const bool gave_up = *plan->abort_host != 0u || plan->gave_up_events != events_before;
+        if (!gave_up && (best_ms < 0.0f || ms_min < best_ms)) {
+            best_ms = ms_min;
+            best = candidates[i];
+        }
+    }
+    plan->measured_mode[bucket] = (unsigned char)best;
+    return lstm_forward_impl(plan, x, h0, c0, y, hn, cn, seq_len, stream, best);
+}
+}  // namespace
+
+extern "C" int pimhip_lstm_forward(PimHipLstmPlan* plan, const void* x, const void* h0, const void* c0, void* y,
+                                   void* hn, void* cn, int64_t seq_len, void* stream)
+{
+    return lstm_forward_impl(plan, x, h0, c0, y, hn, cn, seq_len, stream, -1);
+}
+
+extern "C" int pimhip_lstm_plan_set_measure(PimHipLstmPlan* plan, int enabled)
+{
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    plan->measure = enabled != 0;
+    if (!plan->measure) memset(plan->measured_mode, 0, sizeof(plan->measured_mode));
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_lstm_plan_measured_mode(PimHipLstmPlan* plan, int64_t seq_len, int* mode)
+{
+    if (!plan || !mode) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan and mode must be non-null");
+    if (seq_len < 2) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "seq_len=%lld: one step has one kernel", (long long)seq_len);
+    int bucket = 0;
+    while ((seq_len >> (bucket + 1)) != 0 && bucket < 31) ++bucket;
+    *mode = plan->measured_mode[bucket];
     return PIMHIP_OK;
 }

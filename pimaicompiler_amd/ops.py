@@ -565,6 +565,17 @@ class LstmPlan:
         4 one recurrence per XCD (pimhip_lstm_plan_set_mode)."""
         _check(L.load().pimhip_lstm_plan_set_mode(self._handle, mode))
 
+    def set_measure(self, enabled):
+        """Automatic mode times every kernel family on the first eager call of a range of sequence lengths and keeps the
+        fastest (the default); False: thresholds choose (pimhip_lstm_plan_set_measure)."""
+        _check(L.load().pimhip_lstm_plan_set_measure(self._handle, int(bool(enabled))))
+
+    def measured_mode(self, seq_len):
+        """The mode automatic mode uses for sequences of `seq_len` steps; 0 if not measured yet."""
+        m = ctypes.c_int(0)
+        _check(L.load().pimhip_lstm_plan_measured_mode(self._handle, int(seq_len), ctypes.byref(m)))
+        return int(m.value)
+
     def set_residual(self, first_residual_layer):
         """Layers from `first_residual_layer` on return and hand up h + their own input (the GNMT wiring: an aten::lstm and an
         aten::add per layer in the reference); None or >= num_layers switches it off (pimhip_lstm_plan_set_residual)."""

@@ -24,11 +24,12 @@ def maxabs(a, b):
     return float((a.detach().float().cpu().reshape(-1) - b.float().reshape(-1)).abs().max())
 
 
-def run_plan(ops, params, x, h0, c0, has_b, L, bidir, mode, T=None):
+def run_plan(ops, params, x, h0, c0, has_b, L, bidir, mode, T=None, measure=True):
     T = x.shape[0] if T is None else T
     plan = ops.LstmPlan([p.to(DEV) for p in params], has_b, L, bidir, max(T, 1))
     if mode:
         plan.set_mode(mode)
+    plan.set_measure(measure)
     y, hn, cn = plan.forward(x.reshape(x.shape[0], -1).to(DEV), h0.to(DEV), c0.to(DEV))
     plan.status()
     return y, hn, cn
@@ -341,19 +342,80 @@ def test_sequence_kernels_issued_on_two_streams_do_not_starve_each_other(ops):
         assert maxabs(y, want[0]) <= 2e-3 and maxabs(cn, want[2]) <= 2e-3
 
 
-def test_automatic_mode_takes_the_per_xcd_kernel_where_it_pays(ops):
-    """Bidirectional layers from 16 steps on, single unidirectional layers from 64 (16 at H <= 512) and unidirectional
-    stacks from 32 (16 with three layers and more) run one recurrence per XCD in automatic mode: the same bits as mode 4,
-    which sums in another order than mode 2."""
+def test_automatic_mode_without_measurement_follows_the_thresholds(ops):
+    """What automatic mode does where it cannot measure (inside a graph capture, or with measuring switched off): bidirectional
+    layers from 16 steps on, single unidirectional layers from 64 (16 at H <= 512) and unidirectional stacks from 32 (16 with
+    three layers and more) run one recurrence per XCD: the same bits as mode 4, which sums in another order than mode 2."""
     for I, H, L, bidir, T, same_as in [(32, 256, 2, True, 40, 4), (32, 1024, 1, False, 70, 4), (32, 1024, 1, False, 20, 2),
                                         (32, 256, 1, False, 20, 4), (32, 256, 3, False, 40, 4), (32, 256, 1, True, 9, 2),
                                         (32, 256, 2, False, 20, 2), (32, 256, 2, False, 33, 4), (32, 256, 3, False, 12, 2)]:
         params, x, h0, c0 = workloads.lstm_inputs(800 + T, I, H, L, bidir, T)
-        y0, _, c0n = run_plan(ops, params, x, h0, c0, True, L, bidir, 0)
+        y0, _, c0n = run_plan(ops, params, x, h0, c0, True, L, bidir, 0, measure=False)
         ym, _, cmn = run_plan(ops, params, x, h0, c0, True, L, bidir, same_as)
         assert torch.equal(y0, ym) and torch.equal(c0n, cmn), (I, H, L, bidir, T)
         want = oracle.torch_lstm(x, h0, c0, params, True, L, bidir)
         assert maxabs(y0, want[0]) <= 2e-3 and maxabs(c0n, want[2]) <= 2e-3
+
+
+def _call_us(plan, xd, hd, cd, reps=12):
+    """Shortest of `reps` forwards, each timed with events on torch's current stream, in microseconds."""
+    stream = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = None
+    for _ in range(reps):
+        e0.record(stream)
+        plan.forward(xd, hd, cd)
+        e1.record(stream)
+        e1.synchronize()
+        us = e0.elapsed_time(e1) * 1e3
+        best = us if best is None else min(best, us)
+    return best
+
+
+@pytest.mark.parametrize("name,I,H,L,bidir,T", [
+    ("rnnt_encoder", 240, 1024, 2, False, 200),                      # C3
+    ("gnmt_l0", 1024, 1024, 1, True, 50), ("gnmt_l1", 2048, 1024, 1, False, 50), ("gnmt_l2", 1024, 1024, 1, False, 50),   # C4's calls
+    ("prediction_net_T2", 320, 320, 2, False, 2), ("prediction_net_T5", 320, 320, 2, False, 5),
+    ("prediction_net_T16", 320, 320, 2, False, 16), ("prediction_net_T64", 320, 320, 2, False, 64),
+    ("wide", 256, 1536, 1, False, 40),
+])
+def test_automatic_mode_is_the_fastest_mode_the_plan_has(ops, name, I, H, L, bidir, T):
+    """Automatic mode measures: the first eager forward of a plan in a range of sequence lengths runs the call under every
+    kernel family that takes it and keeps the fastest (as the reference keeps the faster of its two libraries per layer on the
+    first inference).  Afterwards a call in automatic mode is not slower than the same call under any forced mode by more than
+    5 % (+ 4 us: two plans in the same mode differ by that much on the shortest calls, where the host's launches show in the
+    events), and its result is the oracle's."""
+    params, x, h0, c0 = workloads.lstm_inputs(900 + T, I, H, L, bidir, T)
+    pd = [p.to(DEV) for p in params]
+    xd, hd, cd = x.reshape(T, I).to(DEV), h0.to(DEV), c0.to(DEV)
+    auto = ops.LstmPlan(pd, True, L, bidir, T)
+    assert auto.measured_mode(T) == 0
+    y, hn, cn = auto.forward(xd, hd, cd)            # measures
+    auto.status()
+    chosen = auto.measured_mode(T)
+    assert chosen in (1, 2, 4)
+    want = oracle.torch_lstm(x, h0, c0, params, True, L, bidir)
+    assert maxabs(y, want[0]) <= LSTM_TOL and maxabs(hn, want[1]) <= LSTM_TOL and maxabs(cn, want[2]) <= LSTM_TOL
+    y2, _, _ = auto.forward(xd, hd, cd)             # the same mode from now on: the same bits
+    assert torch.equal(y, y2)
+    forced = {}
+    for mode in (1, 2, 4):
+        plan = ops.LstmPlan(pd, True, L, bidir, T)
+        try:
+            plan.set_mode(mode)
+        except ops.NNRuntimeException:
+            continue                                 # this hidden size does not fit that kernel
+        plan.forward(xd, hd, cd)
+        forced[mode] = plan
+    # (the plans take turns, three rounds: what the GPU ran just before shifts a call's time by several per cent)
+    times, t_auto = {m: float("inf") for m in forced}, float("inf")
+    for _ in range(3):
+        t_auto = min(t_auto, _call_us(auto, xd, hd, cd, reps=6))
+        for m, plan in forced.items():
+            times[m] = min(times[m], _call_us(plan, xd, hd, cd, reps=6))
+    print(f"{name}: automatic took mode {chosen}: {t_auto:.1f} us; forced {({m: round(t, 1) for m, t in times.items()})}", flush=True)
+    assert t_auto <= 1.05 * min(times.values()) + 4.0, (name, chosen, t_auto, times)
+    assert auto.fallbacks() == (0, True)
 
 
 def test_per_xcd_kernel_finds_its_groups_on_any_queue(ops):
