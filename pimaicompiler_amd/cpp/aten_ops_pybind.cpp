@@ -1,9 +1,11 @@
 // Python access to the C++ operator bodies of aten_ops_pimhip.cpp, so that the GPU tests can drive the exact code a
 // maintainer of the reference would link.
 #include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
 
 #include <chrono>
 
+#include "../../include/pimhip.h"
 #include "aten_ops_pimhip.h"
 
 namespace ops = nn_compiler::runtime::op_executor;
@@ -24,12 +26,15 @@ PYBIND11_MODULE(_aten_ops_pimhip, m)
     //   "addmm": t = {self, mat1, mat2}    "matmul": t = {self, other}    "linear": t = {input, weight[, bias]}
     //   "lstm1": t = {input, h0, c0}, params in LibTorch order with biases, unidirectional, num_layers = params / 4
     //   "lstm1_into": the same through atenLstm1Into with t = {input, h0, c0, output, hy, cy}
+    //   "c_abi_gemv": pimhip_execute_gemv itself (the call under the three GEMV operators) with t = {y[N], x[K], w[N, K], b[N]}:
+    //   what of an operator's host time is the library's launch and what the operator layer adds on top
     m.def("opHostMicroseconds", [](const std::string& op, std::vector<at::Tensor> t, std::vector<at::Tensor> params, int iters) {
         torch::jit::IValue out;
         std::vector<at::Tensor> hx;
         if (op == "lstm1" || op == "lstm1_into") hx = {t.at(1), t.at(2)};
         const int64_t layers = (int64_t)params.size() / 4;
         const c10::optional<at::Tensor> bias = (op == "linear" && t.size() > 2) ? c10::optional<at::Tensor>(t[2]) : c10::nullopt;
+        void* c_abi_stream = op == "c_abi_gemv" ? (void*)c10::hip::getCurrentHIPStream().stream() : nullptr;
         const auto t0 = std::chrono::steady_clock::now();
         for (int i = 0; i < iters; ++i) {
             if (op == "addmm")
@@ -42,6 +47,11 @@ PYBIND11_MODULE(_aten_ops_pimhip, m)
                 ops::atenLstm1(t.at(0), hx, params, true, layers, 0.0, false, false, false);
             else if (op == "lstm1_into")
                 ops::atenLstm1Into(t.at(0), hx, params, true, layers, 0.0, false, false, false, t.at(3), t.at(4), t.at(5));
+            else if (op == "c_abi_gemv") {
+                if (pimhip_execute_gemv(t.at(0).data_ptr(), t.at(1).data_ptr(), t.at(2).data_ptr(), t.at(3).data_ptr(), t.at(2).size(1),
+                                        t.at(2).size(0), 0, PIMHIP_ACT_NONE, PIMHIP_W_X_I, c_abi_stream) != PIMHIP_OK)
+                    throw utils::NNRuntimeException(pimhip_last_error());
+            }
             else
                 throw utils::NNRuntimeException("unknown operator " + op);
         }
