@@ -590,6 +590,43 @@ def main():
         other["rnnt_joint_step"] = {"three_launches_us": round(graph_timed_us(joint_three, 32), 3),
                                     "two_launches_us": round(graph_timed_us(joint_two, 32), 3),
                                     "max_abs_diff": round(float((jout.float() - ref_out.float()).abs().max()), 6)}
+        # A whole (t, u) step of the transducer's greedy loop: the prediction network (2 LSTM layers, H = I = 320, seq_len 1) and
+        # the joint network, as ONE launch (pimhip_rnnt_step) and as the four launches it replaces (two cells, cat2 product,
+        # 512 -> 29 product), all replayed from graphs; and the step after a blank, where only the joint network runs.
+        rn_prm, rn_x, rn_h, rn_c = workloads.lstm_inputs(4301, 320, 320, 2, False, 1)
+        rn_prm = [q.to(dev) for q in rn_prm]
+        rn_x = rn_x.reshape(320).to(dev)
+        rn_h, rn_c = (0.1 * torch.randn(2, 320, device=dev)).half(), (0.1 * torch.randn(2, 320, device=dev)).half()
+        rn_hn, rn_cn = torch.empty_like(rn_h), torch.empty_like(rn_c)
+        rn_logits = torch.empty(29, dtype=torch.float16, device=dev)
+        rn_plan = P.RnntPlan(rn_prm, True, 2, (jw1, jb1, jw2, jb2))
+        rn_full = rn_plan.bind(rn_x, rn_h, rn_c, jf, rn_hn, rn_cn, rn_logits)
+        rn_blank = rn_plan.bind(None, rn_hn, None, jf, None, None, rn_logits, run_prediction=False)
+        rn_lstm = P.LstmPlan(rn_prm, True, 2, False, 1)
+        rn_y, rn_hn2, rn_cn2 = torch.empty(1, 320, dtype=torch.float16, device=dev), torch.empty_like(rn_h), torch.empty_like(rn_c)
+
+        def rnnt_four(s_h=sh):
+            lib.pimhip_lstm_forward(rn_lstm._handle, rn_x.data_ptr(), rn_h.data_ptr(), rn_c.data_ptr(), rn_y.data_ptr(), rn_hn2.data_ptr(),
+                                    rn_cn2.data_ptr(), 1, s_h)
+            lib.pimhip_execute_gemv_cat2(jhid.data_ptr(), jf.data_ptr(), 1024, rn_y.data_ptr(), 320, jw1.data_ptr(), jb1.data_ptr(), 512, 0,
+                                         L.PIMHIP_ACT_RELU, s_h)
+            lib.pimhip_execute_gemv(jout.data_ptr(), jhid.data_ptr(), jw2.data_ptr(), jb2.data_ptr(), 512, 29, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_W_X_I, s_h)
+        rn_full()
+        rnnt_four()
+        torch.cuda.synchronize()
+        rn_events = rn_plan.fallbacks()[0]
+        other["rnnt_step_one_launch"] = {
+            "us": round(graph_timed_us(lambda s_: rn_full(s_), 32), 3),
+            "issued_from_python_us": round(timed_us(rn_full, 200), 3),
+            "four_launches_us": round(graph_timed_us(rnnt_four, 32), 3),
+            "four_launches_issued_from_python_us": round(timed_us(rnnt_four, 200), 3),
+            "after_a_blank_us": round(graph_timed_us(lambda s_: rn_blank(s_), 32), 3),
+            "after_a_blank_two_launches_us": other["rnnt_joint_step"]["two_launches_us"],
+            "bytes": 2 * (2 * 4 * 320 * 640 + 512 * 1344 + 29 * 512),
+            "max_abs_diff_of_states_to_the_four_launches": round(max(float((rn_hn.float() - rn_hn2.float()).abs().max()),
+                                                                      float((rn_cn.float() - rn_cn2.float()).abs().max())), 6),
+            "max_abs_diff_of_logits_to_the_four_launches": round(float((rn_logits.float() - jout.float()).abs().max()), 6),
+            "waits_that_gave_up": rn_plan.fallbacks()[0] - rn_events}
         # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
         big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
         big_c = torch.empty_like(big_a)

@@ -372,6 +372,53 @@ int pimhip_moe_plan_fallbacks(PimHipMoePlan* plan, uint64_t* events, int* exchan
  * fails gives up at once: every kernel still ends by itself. */
 int pimhip_moe_plan_set_spin_limit(PimHipMoePlan* plan, unsigned int spin_limit);
 
+/* ---- RNN-transducer decoding step --------------------------------------------------------------- */
+
+typedef struct PimHipRnntPlan PimHipRnntPlan;
+
+/* One launch for one (t, u) step of an RNN-transducer's greedy decoding loop: the prediction network's LSTM cells at
+ * seq_len 1 and the joint network.  Replaces, per iteration of that loop, executeAtenLSTM1 with seq_len == 1
+ * (aten_ops_executor.cpp:2135-2307) and the joint network's executeAtenAddmm calls (aten_ops_executor.cpp:181-216), the
+ * first of which RemoveCatForAddmm has split into two dependent products over the two halves of the concatenated input
+ * (compiler/source/frontend/optimizer/remove_cat_for_addmm.cpp:46-191):
+ *
+ *     h_l, c_l = lstm_cell_l(l == 0 ? x : h_{l-1}; h_prev_l, c_prev_l)                    l < num_layers
+ *     hidden   = relu(joint_w1[joint_size, enc_size + H] . cat(f, g) + joint_b1)          g = h of the last layer
+ *     logits   = joint_w2[vocab, joint_size] . hidden + joint_b2
+ *
+ *   params: host array of device pointers in LibTorch order per layer (w_ih [4H, in_w], w_hh [4H, H], then b_ih, b_hh
+ *           [4H] when has_biases), gate order (i, f, g, o); in_w = input_size for the first layer, H above it.
+ *   num_layers 1..4; hidden_size and input_size multiples of 8 up to 1024; enc_size and joint_size multiples of 8 up to
+ *   2048; one workgroup per eight hidden units of a layer, per eight joint units and per eight symbols, at most 256 in all
+ *   (RNNT: 2 x 40 + 64 + 4 = 148); PIMHIP_ERR_UNSUPPORTED otherwise (pimhip_lstm_forward, pimhip_execute_gemv_cat2 and
+ *   pimhip_execute_gemv serve any size).  Weights row-major, dense, fp16, 16-byte aligned.
+ * The plan keeps the weight pointers (they must outlive it), pre-adds the biases and owns a small exchange buffer.  Runs
+ * on `stream` and synchronises it. */
+int pimhip_rnnt_plan_create(PimHipRnntPlan** plan, const void* const* params, int n_params, int has_biases, int num_layers,
+                            int64_t input_size, int64_t hidden_size, const void* joint_w1, const void* joint_b1,
+                            int64_t joint_size, int64_t enc_size, const void* joint_w2, const void* joint_b2, int64_t vocab,
+                            void* stream);
+int pimhip_rnnt_plan_destroy(PimHipRnntPlan* plan);
+
+/* One step.  x [input_size] (the embedding of the last symbol), h_prev, c_prev, hn, cn [num_layers, H], f [enc_size] (the
+ * encoder's output for frame t), logits [vocab]; joint_hidden [joint_size] or null.  run_prediction == 0 is the step after
+ * a blank, where only the frame has changed: the prediction network does not run, g = h_prev of the last layer, and x,
+ * c_prev, hn, cn are not touched (they may be null).  hn / cn must not overlap h_prev / c_prev (keep two state buffers and
+ * swap them).
+ * Records one kernel, so steps can be recorded into a HIP graph.  All workgroups of the launch have to be resident at
+ * once: the call is ordered like a sequence call of pimhip_lstm_forward against the device's other such launches, and
+ * steps sharing a plan must be ordered on one stream.  Every wait inside is bounded, and a wait that gives up costs time,
+ * not the result: the workgroup that waited in vain computes the vector it waited for by itself, inside the same launch,
+ * with the same sums, and the outputs are what they would have been.  Later steps do the same from the start until a step
+ * issued outside a graph capture has put the exchange back in order (it synchronises the stream then); after the third
+ * such event the plan stops exchanging for good (slower, still one launch). */
+int pimhip_rnnt_step(PimHipRnntPlan* plan, const void* x, const void* h_prev, const void* c_prev, const void* f, void* hn,
+                     void* cn, void* logits, void* joint_hidden, int run_prediction, void* stream);
+
+/* No counterpart in the reference.  As pimhip_moe_plan_fallbacks / pimhip_moe_plan_set_spin_limit. */
+int pimhip_rnnt_plan_fallbacks(PimHipRnntPlan* plan, uint64_t* events, int* exchanging);
+int pimhip_rnnt_plan_set_spin_limit(PimHipRnntPlan* plan, unsigned int spin_limit);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,6 +28,7 @@ from .ops import (  # noqa: F401
     LstmPlan,
     DecoderPlan,
     MoePlan,
+    RnntPlan,
     prepare_lstm,
     invalidate_lstm_plans,
     gemv_status,

@@ -75,6 +75,13 @@ SIGNATURES = {
     "pimhip_moe_plan_status": (ctypes.c_int, [ctypes.c_void_p]),
     "pimhip_moe_plan_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), c_int_p]),
     "pimhip_moe_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
+    "pimhip_rnnt_plan_create": (ctypes.c_int, [c_void_pp, c_void_pp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+                                               ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                                               ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
+    "pimhip_rnnt_plan_destroy": (ctypes.c_int, [ctypes.c_void_p]),
+    "pimhip_rnnt_step": (ctypes.c_int, [ctypes.c_void_p] * 9 + [ctypes.c_int, ctypes.c_void_p]),
+    "pimhip_rnnt_plan_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), c_int_p]),
+    "pimhip_rnnt_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "pimhip_input_projection": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
     "pimhip_projection_packed_bytes": (ctypes.c_int, [ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_uint64)]),

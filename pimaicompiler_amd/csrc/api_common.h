@@ -100,5 +100,6 @@ void launch_lstm_bias_sum(const half_t* b_ih, const half_t* b_hh, float* bsum, i
 void destroy_all_lstm_plans_locked();
 void destroy_all_decoder_plans_locked();
 void destroy_all_moe_plans_locked();
+void destroy_all_rnnt_plans_locked();
 
 }  // namespace pimhip

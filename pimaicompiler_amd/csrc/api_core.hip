@@ -135,6 +135,7 @@ extern "C" int pimhip_deinitialize(void)
     destroy_all_lstm_plans_locked();
     destroy_all_decoder_plans_locked();
     destroy_all_moe_plans_locked();
+    destroy_all_rnnt_plans_locked();
     int prev = -1;
     hipGetDevice(&prev);
     for (auto& kv : g_devices) {

@@ -15,7 +15,7 @@ struct PimHipMoePlan {
     const half_t* router_b = nullptr;
     const half_t** tables = nullptr;       // device: [4][E] pointers (W1, b1, W2, b2 of every expert)
     unsigned long long* hx = nullptr;      // [2][kMoeMaxBlocks][kMoeEntryWords], all ones = empty
-    unsigned int* g_counter = nullptr;
+    unsigned int* g_counter = nullptr;     // [kMoeMaxBlocks][kMoeCounterStride]: every block's copy of the launch count
     unsigned int* abort_flag = nullptr;
     unsigned int* abort_host = nullptr;
     unsigned int* abort_host_dev = nullptr;
@@ -131,8 +131,8 @@ extern "C" int pimhip_moe_plan_create(PimHipMoePlan** plan_out, const void* rout
     MOE_HIP_CHECK(hipMemcpyAsync(plan->tables, host_tables.data(), host_tables.size() * sizeof(const half_t*), hipMemcpyHostToDevice, s));
     MOE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&plan->hx), kMoeExchangeWords32 * sizeof(unsigned int)));
     launch_fill_u32(reinterpret_cast<unsigned int*>(plan->hx), kMoeExchangeWords32, ~0u, s);
-    MOE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&plan->g_counter), sizeof(unsigned int)));
-    launch_fill_u32(plan->g_counter, 1, 0u, s);
+    MOE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&plan->g_counter), sizeof(unsigned int) * kMoeMaxBlocks * kMoeCounterStride));
+    launch_fill_u32(plan->g_counter, (size_t)kMoeMaxBlocks * kMoeCounterStride, 0u, s);
     MOE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&plan->abort_flag), sizeof(unsigned int)));
     launch_fill_u32(plan->abort_flag, 1, 0u, s);
     MOE_HIP_CHECK(hipGetLastError());
@@ -209,7 +209,7 @@ extern "C" int pimhip_moe_ffn_step(PimHipMoePlan* plan, const void* x, void* y, 
         ++plan->gave_up_events;
         if (plan->gave_up_events >= kMoeEventsBeforeAlone) plan->alone = true;
         launch_fill_u32(reinterpret_cast<unsigned int*>(plan->hx), kMoeExchangeWords32, ~0u, s);
-        launch_fill_u32(plan->g_counter, 1, 0u, s);
+        launch_fill_u32(plan->g_counter, (size_t)kMoeMaxBlocks * kMoeCounterStride, 0u, s);
         launch_fill_u32(plan->abort_flag, 1, 0u, s);
         PIMHIP_HIP_CHECK(hipGetLastError());
     }
@@ -234,6 +234,8 @@ extern "C" int pimhip_moe_ffn_step(PimHipMoePlan* plan, const void* x, void* y, 
     a.wpb = plan->wpb;
     a.rpb2 = plan->rpb2;
     a.alone = plan->alone ? 1 : 0;
+    // (every block publishes a word of hidden values unless the second matrix needs more blocks than there are words)
+    a.count_stride = (int64_t)(plan->blocks - 1) * plan->wpb < plan->d_ff / 8 ? 0 : kMoeCounterStride;
     a.spin_limit = plan->spin_limit;
     // All blocks have to be resident at once, like the sequence kernel's: ordered after it on other streams.
     if (!capturing) {

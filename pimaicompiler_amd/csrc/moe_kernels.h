@@ -27,8 +27,11 @@
 //
 // Exchange: hx[2][blocks] entries of 64 bytes, a block's words in the first 16 * wpb bytes.  An empty 8-byte half is all
 // ones, which no four fp16 values written here can be (a NaN is written as 0x7e00).  The two sets alternate by the launch
-// count g (a device word read at the start and advanced by block 0 at the end): a launch uses set g & 1 and marks its own
-// entry of the other set empty for the launch after it.
+// count g (a device word read at the start): a launch uses set g & 1 and marks its own entry of the other set empty for the
+// launch after it.  Where every block publishes a word, block 0 advances the count at its end: it has seen everybody's word
+// by then, so everybody has read the count.  A block that publishes nothing could start so late that it reads the count
+// after block 0 has advanced it, and would look into the wrong set; grids with such blocks (d_model > d_ff / 2) keep one copy
+// of the count per block, each in a line of its own, read and advanced by its block (0.3 us slower per step).
 //
 // A wait that gives up does not leave the result undefined.  Every wait is bounded (`spin_limit` polls, one second); a block
 // in which a lane gave up computes every hidden value itself from W1[e] (no other block is needed for that: it is only
@@ -54,6 +57,7 @@ constexpr int kMoeMaxWordsPerBlock = 2;               // wpb
 constexpr int kMoeMaxRows2 = kMoeWaves;               // W2 rows per block: one per wavefront
 constexpr int kMoeEntryWords = 8;                     // 8-byte words per entry (64 bytes); the first 2 * wpb carry values
 constexpr unsigned long long kMoeEmpty = ~0ull;
+constexpr int kMoeCounterStride = 16;                // 32-bit words between the blocks' copies of the launch count: a 64-byte line each
 static_assert(kMoeMaxFf / 8 <= kMoeThreads, "thread t of a block polls word t");
 static_assert(kMoeMaxWordsPerBlock * kMoeMaxBlocks * 8 >= kMoeMaxFf, "every hidden value has a producer");
 static_assert(2 * kMoeMaxWordsPerBlock <= kMoeEntryWords, "a block's words fit its entry");
@@ -67,7 +71,7 @@ struct MoeStepArgs {
     half_t* router_logits;           // [E] or null
     int* expert;                     // [1] or null
     unsigned long long* hx;          // [2][blocks][kMoeEntryWords]
-    unsigned int* g_counter;
+    unsigned int* g_counter;         // [blocks][kMoeCounterStride]: every block's copy of the launch count in word 0 of its line
     unsigned int* abort_flag;        // device word: non-zero from the first wait that gave up until the host clears it
     unsigned int* abort_host;        // the same event for the host to see
     int d_model, d_ff, E, act, scale_by_prob;
@@ -75,6 +79,7 @@ struct MoeStepArgs {
     int rpb2;                        // rows of W2 per block
     unsigned int spin_limit;
     int alone;                       // non-zero: every block computes all hidden values itself, nothing is exchanged
+    int count_stride;                // 0: one launch count, advanced by block 0; kMoeCounterStride: one per block
 };
 
 // What the kernel's first instructions need comes as plain arguments in front of the struct: those arrive in scalar
@@ -96,6 +101,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
     __shared__ const half_t* table_s[4][kMoeMaxExperts];
     __shared__ __align__(16) unsigned short mine[8 * kMoeMaxWordsPerBlock];  // this block's hidden values (bits)
     __shared__ int someone_gave_up;
+    __shared__ int block_poisoned;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int b = blockIdx.x, nb = gridDim.x;
@@ -104,7 +110,10 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
 #pragma unroll
     for (int e = 0; e < 8; ++e) zero8[e] = (half_t)0.0f;
 
-    if (tid == 0) someone_gave_up = 0;
+    if (tid == 0) {
+        someone_gave_up = 0;
+        block_poisoned = 0;
+    }
     // the experts' pointers, while the router's rows travel
     for (int i = tid; i < 4 * p.E; i += kMoeThreads) table_s[i / p.E][i % p.E] = p.tables[i];
 
@@ -197,7 +206,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
     // The launch count (which set of slots this launch uses) and the abort word are device-scope loads, which take longer
     // than the cached ones above and would hold those up if they stood in front of them (a wavefront's loads return in
     // order).  Asked for here, they travel with the rows of W1 and are needed when the block publishes.
-    const unsigned int g = __hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned int g = __hip_atomic_load(p.g_counter + p.count_stride * b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const unsigned int poisoned = __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- hidden = act(W1[e] . x + b1[e]): this block's words (asked for whether or not they will be published) ----
     const int row0 = 8 * p.wpb * b + wave * p.wpb;  // this wavefront's first row
@@ -221,10 +230,14 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
         a = wave_sum(a);
         if (lane == 0 && s < p.wpb) mine[wave * p.wpb + s] = r < p.d_ff ? hidden_bits(a, r) : (unsigned short)0;
     }
-    const bool alone = p.alone != 0 || poisoned != 0u;
+    // Whether the abort word is up is decided for the block as a whole, through LDS: wavefronts look at it at slightly
+    // different times and can see different values when it is raised while the launch starts; they would then disagree
+    // about the barriers that follow.  (The flags were set to 0 in front of the barrier behind the router.)
+    if (poisoned != 0u) block_poisoned = 1;
+    __syncthreads();
+    const bool alone = p.alone != 0 || block_poisoned != 0;
     const unsigned int set = g & 1u;
     if (!alone) {
-        __syncthreads();
         if (tid < p.wpb && b * p.wpb + tid < nf) {
             const unsigned long long* src = reinterpret_cast<const unsigned long long*>(&mine[8 * tid]);
             store16_device_scope(p.hx + ((long)set * nb + b) * kMoeEntryWords + 2 * tid, src[0], src[1]);
@@ -292,7 +305,8 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
     // this block's entry of the other set is empty for the next launch (nobody reads that set during this one)
     if (tid < 2 * kMoeMaxWordsPerBlock)
         __hip_atomic_store(p.hx + ((long)(set ^ 1u) * nb + b) * kMoeEntryWords + tid, kMoeEmpty, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (b == 0 && tid == 0) __hip_atomic_store(p.g_counter, g + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0 && (b == 0 || p.count_stride != 0))
+        __hip_atomic_store(p.g_counter + p.count_stride * b, g + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace pimhip

@@ -954,3 +954,102 @@ def aten_lstm2(data, batch_sizes, hx, params, has_biases, num_layers, dropout, t
     y, hn, cn = plan.forward(data, hx[0], hx[1], stream)
     D, H = plan.num_dirs, plan.hidden
     return y, hn.view(num_layers * D, 1, H), cn.view(num_layers * D, 1, H)
+
+
+class RnntPlan:
+    """One launch per (t, u) step of an RNN-transducer's greedy decoding loop (pimhip_rnnt_step): the prediction network's
+    LSTM cells at seq_len 1 and the joint network relu(W1 . cat(f, g) + b1) -> W2 . + b2.  The reference runs
+    executeAtenLSTM1 (aten_ops_executor.cpp:2135-2307) and three executeAtenAddmm per iteration, the joint network's first
+    layer split in two by RemoveCatForAddmm (remove_cat_for_addmm.cpp:46-191).
+
+    params: the prediction network's LSTM parameters in LibTorch order; joint = (W1 [J, F + H], b1 [J] or None,
+    W2 [V, J], b2 [V] or None)."""
+
+    def __init__(self, params, has_biases, num_layers, joint, stream=None):
+        lib = L.load()
+        w1, b1, w2, b2 = joint
+        ts = list(params) + [w1, w2] + [t for t in (b1, b2) if t is not None]
+        _require_half_cuda(*ts)
+        _ensure_init(w1)
+        per_layer = 4 if has_biases else 2
+        if len(params) != per_layer * num_layers:
+            raise NNRuntimeException(f"{len(params)} parameters for {num_layers} layers (expected {per_layer * num_layers})")
+        self.hidden, self.input_size = params[1].size(1), params[0].size(1)
+        self.num_layers = num_layers
+        self.joint_size, self.vocab = w1.size(0), w2.size(0)
+        self.enc_size = w1.size(1) - self.hidden
+        for l in range(num_layers):
+            in_w = self.input_size if l == 0 else self.hidden
+            if tuple(params[l * per_layer].shape) != (4 * self.hidden, in_w) or tuple(params[l * per_layer + 1].shape) != (4 * self.hidden, self.hidden):
+                raise NNRuntimeException(f"layer {l}: w_ih must be [{4 * self.hidden}, {in_w}] and w_hh [{4 * self.hidden}, {self.hidden}]")
+        if self.enc_size < 8 or tuple(w2.shape) != (self.vocab, self.joint_size):
+            raise NNRuntimeException("joint: W1 must be [J, F + H] and W2 [V, J]")
+        if (b1 is not None and b1.numel() != self.joint_size) or (b2 is not None and b2.numel() != self.vocab):
+            raise NNRuntimeException("joint: b1 must have J and b2 V elements")
+        self.device = w1.device
+        self._keep = [t.contiguous() for t in ts]   # the plan reads the weights where they lie: keep them alive
+        k = iter(self._keep)
+        prm = [next(k) for _ in range(len(params))]
+        w1_c, w2_c = next(k), next(k)
+        b1_c = next(k) if b1 is not None else None
+        b2_c = next(k) if b2 is not None else None
+        arr = (ctypes.c_void_p * len(prm))(*[t.data_ptr() for t in prm])
+        ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+        handle = ctypes.c_void_p()
+        _check(lib.pimhip_rnnt_plan_create(ctypes.byref(handle), arr, len(prm), int(bool(has_biases)), num_layers, self.input_size,
+                                           self.hidden, w1_c.data_ptr(), ptr(b1_c), self.joint_size, self.enc_size, w2_c.data_ptr(),
+                                           ptr(b2_c), self.vocab, _stream_handle(stream)))
+        self._handle = handle
+        self._finalizer = weakref.finalize(self, RnntPlan._destroy, handle.value)
+
+    @staticmethod
+    def _destroy(handle_value):
+        try:
+            L.load().pimhip_rnnt_plan_destroy(ctypes.c_void_p(handle_value))
+        except Exception:  # interpreter shutdown
+            pass
+
+    def set_spin_limit(self, limit):
+        _check(L.load().pimhip_rnnt_plan_set_spin_limit(self._handle, limit))
+
+    def fallbacks(self):
+        """(events, exchanging): waits that have given up inside steps of this plan so far, and whether steps still exchange
+        vectors between workgroups.  Synchronises (pimhip_rnnt_plan_fallbacks)."""
+        torch.cuda.synchronize(self.device)
+        events, exchanging = ctypes.c_uint64(0), ctypes.c_int(0)
+        _check(L.load().pimhip_rnnt_plan_fallbacks(self._handle, ctypes.byref(events), ctypes.byref(exchanging)))
+        return int(events.value), bool(exchanging.value)
+
+    def bind(self, x, h_prev, c_prev, f, hn, cn, logits, joint_hidden=None, run_prediction=True):
+        """Fixes the buffers of a step and returns a callable step(stream=None): what a decoding loop or a graph capture calls.
+        x [I], h_prev / c_prev / hn / cn [L, H], f [F], logits [V], joint_hidden [J] or None; with run_prediction False (the
+        step after a blank) x, c_prev, hn, cn may be None."""
+        lib = L.load()
+        given = [t for t in (x, h_prev, c_prev, f, hn, cn, logits, joint_hidden) if t is not None]
+        _require_half_cuda(*given)
+        for t in given:
+            if not t.is_contiguous():
+                raise NNRuntimeException("step buffers must be contiguous")
+        n_state = self.num_layers * self.hidden
+        sizes = ((x, self.input_size, "x"), (h_prev, n_state, "h_prev"), (c_prev, n_state, "c_prev"), (f, self.enc_size, "f"),
+                 (hn, n_state, "hn"), (cn, n_state, "cn"), (logits, self.vocab, "logits"), (joint_hidden, self.joint_size, "joint_hidden"))
+        for t, n, name in sizes:
+            if t is not None and t.numel() != n:
+                raise NNRuntimeException(f"{name} must have {n} elements")
+        ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+        args = (self._handle, ptr(x), ptr(h_prev), ptr(c_prev), ptr(f), ptr(hn), ptr(cn), ptr(logits), ptr(joint_hidden),
+                int(bool(run_prediction)))
+
+        def step(stream=None, _keep=tuple(given)):
+            _check(lib.pimhip_rnnt_step(*args, _stream_handle(stream)))
+        return step
+
+    def forward(self, x, h_prev, c_prev, f, run_prediction=True, stream=None):
+        """logits [V], hn, cn [L, H] for one step (new tensors; with run_prediction False hn, cn are h_prev, c_prev)."""
+        logits = torch.empty(self.vocab, dtype=torch.float16, device=self.device)
+        if run_prediction:
+            hn, cn = torch.empty_like(h_prev.contiguous()), torch.empty_like(c_prev.contiguous())
+            self.bind(x.contiguous(), h_prev.contiguous(), c_prev.contiguous(), f.contiguous(), hn, cn, logits)(stream)
+            return logits, hn, cn
+        self.bind(None, h_prev.contiguous(), None, f.contiguous(), None, None, logits, run_prediction=False)(stream)
+        return logits, h_prev, c_prev
