@@ -27,10 +27,11 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix rate
 SWEEP = [(4096, 4096), (16384, 4096), (4096, 16384), (32000, 1024)]
 POOL_BYTES_PER_SHAPE = 512 << 20
-# HBM bytes per launch of the dominant kernel, mean over its three shapes, from two rocprofv3 --pmc runs of this
-# script (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch, factors from --calibration-copy); the figures and the
-# commands are in profiles/gemv_sweep_pmc.md.  A counter reading, not something this script can measure itself.
-DOMINANT_KERNEL_TRAFFIC_BYTES = int((131431.0 + 131431.0 + 32935.0) / 3 * 1024 + (256.0 + 64.0 + 64.0) / 3 * 1024)
+# HBM bytes per launch of the dominant kernel, mean over its three shapes, from rocprofv3 --pmc runs of this script, one
+# shape and one counter per run (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch, factors from --calibration-copy);
+# the per-shape figures and the commands are in profiles/gemv_sweep_pmc.md, and tests/test_profiles.py recomputes this
+# number from that file.  A counter reading, not something this script can measure itself.
+DOMINANT_KERNEL_TRAFFIC_BYTES = 101094400
 
 
 def gemv_bytes(n, k, bias=True):
