@@ -107,6 +107,15 @@ int pimhip_get_gemm_type(const int64_t* self_shape4, const int64_t* other_shape4
 int pimhip_execute_gemv(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
                         int64_t out_w, int64_t ld_weight, int act, int order, void* stream);
 
+/* The same with the alpha and beta of the reference's own HIP launchers (rocblas_gemv_template_xAy / _Axy,
+ * rocblas_addmv_template_xAy / _Axy, runtime/include/executor/op_executor/custom_ops.h:123-139, 198-214, 281-298, 364-381):
+ * out[out_w] = act(alpha * sum_k weight * in[k] + beta * out[out_w] + bias[out_w]); out is not read when beta == 0.
+ * alpha == 1, beta == 0 (the only values the reference passes, aten_ops.cpp:627-628, custom_op_ut.cpp:26-27) is
+ * pimhip_execute_gemv itself; other values take plain kernels (2-byte loads, any size, pitch and alignment) that run at a
+ * fraction of its rate. */
+int pimhip_execute_gemv_scaled(void* out, const void* in, const void* weight, const void* bias, int64_t in_w,
+                               int64_t out_w, int64_t ld_weight, int act, int order, float alpha, float beta, void* stream);
+
 /* out[out_w] = act(weight[out_w, in1_w + in2_w] . cat(in1, in2) + bias) without the concatenation (order W_X_I): in1 and
  * in2 lie apart, as the encoder frame and the prediction that the RNNT joint network's first layer reads do.  Replaces the
  * pair of dependent products RemoveCatForAddmm makes of such a layer

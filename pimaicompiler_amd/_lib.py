@@ -26,6 +26,9 @@ SIGNATURES = {
     "pimhip_execute_gemv_static": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                                   ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                                   ctypes.c_int, ctypes.c_void_p]),
+    "pimhip_execute_gemv_scaled": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                                                  ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float,
+                                                  ctypes.c_void_p]),
     "pimhip_execute_gemv_cat2": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64,
                                                 ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                                 ctypes.c_void_p]),

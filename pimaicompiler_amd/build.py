@@ -32,7 +32,7 @@ def hipcc():
 
 
 # One translation unit per kernel family (each kernel header is compiled once); api_common.h is what they share.
-SOURCES = ["api_core.hip", "api_gemv.hip", "api_xproj.hip", "api_lstm.hip", "api_decoder.hip", "api_moe.hip", "api_rnnt.hip"]
+SOURCES = ["api_core.hip", "api_gemv.hip", "api_xproj.hip", "api_lstm.hip", "api_decoder.hip", "api_moe.hip", "api_rnnt.hip", "api_blas.hip"]
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 
 

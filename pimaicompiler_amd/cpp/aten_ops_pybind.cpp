@@ -7,6 +7,7 @@
 
 #include "../../include/pimhip.h"
 #include "aten_ops_pimhip.h"
+#include "custom_ops_pimhip.h"
 
 namespace ops = nn_compiler::runtime::op_executor;
 namespace utils = nn_compiler::runtime::utils;
@@ -87,5 +88,32 @@ PYBIND11_MODULE(_aten_ops_pimhip, m)
         return std::make_pair(a, b);
     });
     m.def("getGemmType", [](std::vector<int64_t> a, std::vector<int64_t> b) { return (int)utils::getGemmType(a, b); });
+    // The launchers with the signatures of the reference's custom_ops.h, called as its own code calls them: raw pointers to 16-bit
+    // floating-point elements (the reference's are _Float16*, which this host compiler does not have; at::Half has the same
+    // bits), sizes, alpha / beta; `stream` 0 is the null stream, as the reference passes it.
+    auto f16 = [](const at::Tensor& t) { return static_cast<at::Half*>(t.data_ptr()); };
+    auto hs = [](uintptr_t stream) { return reinterpret_cast<hipStream_t>(stream); };
+    m.def("rocblas_gemv_template_xAy", [f16, hs](uintptr_t stream, at::Tensor x, at::Tensor A, at::Tensor y, int mm, int n, int k, float alpha, float beta) {
+        ops::rocblas_gemv_template_xAy(hs(stream), (const at::Half*)f16(x), (const at::Half*)f16(A), f16(y), mm, n, k, alpha, beta);
+    });
+    m.def("rocblas_gemv_template_Axy", [f16, hs](uintptr_t stream, at::Tensor A, at::Tensor x, at::Tensor y, int mm, int n, int k, float alpha, float beta) {
+        ops::rocblas_gemv_template_Axy(hs(stream), (const at::Half*)f16(A), (const at::Half*)f16(x), f16(y), mm, n, k, alpha, beta);
+    });
+    m.def("rocblas_addmv_template_xAy", [f16, hs](uintptr_t stream, at::Tensor b, at::Tensor x, at::Tensor A, at::Tensor y, int mm, int n, int k,
+                                                   float alpha, float beta, bool relu) {
+        ops::rocblas_addmv_template_xAy(hs(stream), (const at::Half*)f16(b), (const at::Half*)f16(x), (const at::Half*)f16(A), f16(y), mm, n, k, alpha,
+                                        beta, relu);
+    });
+    m.def("rocblas_addmv_template_Axy", [f16, hs](uintptr_t stream, at::Tensor b, at::Tensor A, at::Tensor x, at::Tensor y, int mm, int n, int k,
+                                                   float alpha, float beta, bool relu) {
+        ops::rocblas_addmv_template_Axy(hs(stream), (const at::Half*)f16(b), (const at::Half*)f16(A), (const at::Half*)f16(x), f16(y), mm, n, k, alpha,
+                                        beta, relu);
+    });
+    m.def("custom_add", [f16, hs](uintptr_t stream, at::Tensor A, at::Tensor B, at::Tensor C, int mm, int n, float alpha, bool sym) {
+        ops::custom_add(hs(stream), f16(A), f16(B), f16(C), mm, n, alpha, sym, 1, 1, 1, 1);
+    });
+    m.def("rocblas_bmm_template_xAy", [f16, hs](uintptr_t stream, at::Tensor x, at::Tensor A, at::Tensor y, int mm, int n, int k) {
+        ops::rocblas_bmm_template_xAy(hs(stream), (const at::Half*)f16(x), (const at::Half*)f16(A), f16(y), mm, n, k);
+    });
     py::register_exception<utils::NNRuntimeException>(m, "NNRuntimeException");
 }

@@ -1,8 +1,8 @@
 """Tables from rocprofv3's CSV output for the kernels of libpimhip.so: durations per kernel and grid from a kernel trace
 (`*_kernel_trace.csv`), counter values per dispatch from a counter run (`*_counter_collection.csv`).
 
-    python -m pimaicompiler_amd.profile_tables trace gpurun_out/prof/bench_kernel_trace.csv
-    python -m pimaicompiler_amd.profile_tables pmc gpurun_out/pmc/p_counter_collection.csv
+    python -m pimaicompiler_amd.profile_tables trace out/bench_kernel_trace.csv
+    python -m pimaicompiler_amd.profile_tables pmc out/p_counter_collection.csv
 
 The summaries under profiles/ are made of these tables."""
 import collections

@@ -87,3 +87,15 @@ def test_hot_path_declarations_of_the_reference_header_are_the_ones_the_shim_hea
     shim = open(os.path.join(ROOT, "pimaicompiler_amd/cpp/aten_ops_pimhip.h")).read()
     for name in ("atenLinear", "atenLstm1", "atenLstm2", "customAtenAddmm", "customAtenMatmul"):
         assert types_only(decl(ref, name)) == types_only(decl(shim, name)), name
+
+
+@needs_reference
+def test_custom_ops_launchers_compile_where_the_references_do():
+    """cpp/custom_ops_pimhip.h against the reference's custom_ops.h: one source holding the calls the reference's own code
+    makes of the six launchers (custom_op_ut.cpp:42, :64; aten_ops_executor.cpp:159, :735) and their explicit instantiations
+    is compiled once against each header (oracle/Makefile sigcheck); the control asks for an argument list neither declares."""
+    ok = subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "sigcheck"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert ok.returncode == 0 and "6 launchers compile against both headers" in ok.stdout, ok.stdout
+    bad = subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "sigcheck", "SIGCHECK_DEFS=-DSIGCHECK_DRIFT"], stdout=subprocess.PIPE,
+                         stderr=subprocess.STDOUT, text=True)
+    assert bad.returncode != 0 and "6 launchers compile" not in bad.stdout

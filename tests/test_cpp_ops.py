@@ -246,3 +246,97 @@ def test_cpp_lstm_into_fills_the_callers_buffers(cpp_gpu):
     assert maxabs(ys, ws[0]) <= 5e-3 and maxabs(hs, ws[1]) <= 5e-3
     y4 = cpp_gpu.atenLstm1(xd, [h0d, c0d], pd, True, 2, 0.0, False, False, False)[0]
     assert torch.equal(y4, y)
+
+
+# ---- the launchers with the signatures of the reference's custom_ops.h (cpp/custom_ops_pimhip.h) ---------------------
+def _ulp_f16(v):
+    v = np.maximum(np.abs(np.asarray(v, dtype=np.float64)), 2.0 ** -14)
+    return 2.0 ** (np.floor(np.log2(v)) - 10)
+
+
+def _within(y, exact, atol=1e-3, rtol=1e-5):
+    """The reference's comparator (ut_utils.h:24-26: allclose(atol 1e-3, rtol 1e-5)) where it is meaningful for fp16 results:
+    the result is the rounding of a value within that tolerance of the exact one."""
+    exact = np.asarray(exact, dtype=np.float64)
+    err = np.abs(y.double().cpu().numpy().reshape(exact.shape) - exact)
+    return bool(np.all(err <= 0.5 * _ulp_f16(exact) + atol + rtol * np.abs(exact)))
+
+
+@pytest.mark.gpu
+def test_custom_gemv_unit_test_of_the_reference_through_its_own_launchers(cpp_gpu):
+    """runtime/unit-tests/custom_op_ut.cpp:20-69 statement by statement: U[0, 1) operands, alpha = 1, beta = 0, the null
+    stream, output buffers from at::zeros, rocblas_gemv_template_xAy on [1,1,1,1024] x [1024,4096] and
+    rocblas_gemv_template_Axy on [4096,1024] x [1,1,1024,1], against the matrix product."""
+    g = torch.Generator().manual_seed(5)
+    alpha, beta = 1.0, 0.0
+    self, other = torch.rand(1, 1, 1, 1024, generator=g).half(), torch.rand(1024, 4096, generator=g).half()
+    m, n, k = 1, other.size(-1), other.size(-2)
+    out = torch.zeros(1, 1, 1, n, dtype=torch.float16, device=DEV)
+    cpp_gpu.rocblas_gemv_template_xAy(0, self.to(DEV), other.to(DEV), out, m, n, k, alpha, beta)
+    torch.cuda.synchronize()
+    assert _within(out, torch.matmul(self.double(), other.double()).numpy())
+    self, other = torch.rand(4096, 1024, generator=g).half(), torch.rand(1, 1, 1024, 1, generator=g).half()
+    m, n, k = self.size(-2), 1, self.size(-1)
+    out = torch.zeros(1, 1, m, 1, dtype=torch.float16, device=DEV)
+    cpp_gpu.rocblas_gemv_template_Axy(0, self.to(DEV), other.to(DEV), out, m, n, k, alpha, beta)
+    torch.cuda.synchronize()
+    assert _within(out, torch.matmul(self.double(), other.double()).numpy())
+    # a matrix-matrix product does nothing, as in the reference ("found gemm, unsupported")
+    out.fill_(3.0)
+    cpp_gpu.rocblas_gemv_template_Axy(0, self.to(DEV), other.to(DEV), out, m, 2, k, alpha, beta)
+    torch.cuda.synchronize()
+    assert bool((out == 3.0).all())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 0.0), (1.0, 1.0), (-2.0, 0.25)])
+@pytest.mark.parametrize("n,k", [(512, 320), (29, 512), (1000, 77)])
+def test_gemv_and_addmv_launchers_with_alpha_and_beta(cpp_gpu, alpha, beta, n, k):
+    """y = relu?(alpha * product + beta * y + b) in both operand orders (custom_ops.h:66-108, 142-183, 216-259, 300-342),
+    against float64 on the same fp16 operands; tolerance 2e-3 on values of order one, as for every GEMV here."""
+    g = torch.Generator().manual_seed(n + k)
+    x = (2 * torch.rand(k, generator=g) - 1).half()
+    a_kn = (torch.randn(k, n, generator=g) / k ** 0.5).half()          # xAy: A [k, n]
+    a_nk = a_kn.t().contiguous()                                        # Axy: A [n, k]
+    b = (0.1 * torch.randn(n, generator=g)).half()
+    y0 = torch.randn(n, generator=g).half()
+    prod = x.double() @ a_kn.double()
+    for relu in (False, True):
+        want_gemv = alpha * prod + beta * y0.double()
+        want_addmv = want_gemv + b.double()
+        if relu:
+            want_addmv = want_addmv.clamp(min=0)
+        ya = y0.clone().to(DEV)
+        cpp_gpu.rocblas_addmv_template_xAy(0, b.to(DEV), x.to(DEV), a_kn.to(DEV), ya, 1, n, k, alpha, beta, relu)
+        yb = y0.clone().to(DEV)
+        cpp_gpu.rocblas_addmv_template_Axy(0, b.to(DEV), a_nk.to(DEV), x.to(DEV), yb, n, 1, k, alpha, beta, relu)
+        torch.cuda.synchronize()
+        assert maxabs(ya, want_addmv.float()) <= 2e-3 * max(1.0, abs(alpha) + abs(beta)) and maxabs(yb, want_addmv.float()) <= 2e-3 * max(1.0, abs(alpha) + abs(beta))
+    yc = y0.clone().to(DEV)
+    cpp_gpu.rocblas_gemv_template_xAy(0, x.to(DEV), a_kn.to(DEV), yc, 1, n, k, alpha, beta)
+    yd = y0.clone().to(DEV)
+    cpp_gpu.rocblas_gemv_template_Axy(0, a_nk.to(DEV), x.to(DEV), yd, n, 1, k, alpha, beta)
+    torch.cuda.synchronize()
+    assert maxabs(yc, want_gemv.float()) <= 2e-3 * max(1.0, abs(alpha) + abs(beta)) and maxabs(yd, want_gemv.float()) <= 2e-3 * max(1.0, abs(alpha) + abs(beta))
+
+
+@pytest.mark.gpu
+def test_custom_add_and_bmm_launchers_as_the_executors_call_them(cpp_gpu):
+    """custom_add as executeAtenAdd calls it (aten_ops_executor.cpp:148-159: m, n the last two sizes, sym when the ranks
+    agree, strides 1) and rocblas_bmm_template_xAy as executeAtenBmm does (aten_ops_executor.cpp:725-735), against the oracle's
+    add (bit for bit) and the float64 product."""
+    g = torch.Generator().manual_seed(9)
+    a, bsym, brow = (torch.randn(50, 1024, generator=g).half(), torch.randn(50, 1024, generator=g).half(), torch.randn(1024, generator=g).half())
+    c = torch.empty(50, 1024, dtype=torch.float16, device=DEV)
+    cpp_gpu.custom_add(0, a.to(DEV), bsym.to(DEV), c, 50, 1024, 1.0, True)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint16), oracle.add(a.numpy(), bsym.numpy()).view(np.uint16))
+    cpp_gpu.custom_add(0, a.to(DEV), brow.to(DEV), c, 50, 1024, 1.0, False)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint16), oracle.add(a.numpy(), brow.numpy()).view(np.uint16))
+    p = torch.softmax(torch.randn(1, 1, 50, generator=g), -1).half()
+    enc = torch.randn(1, 50, 1024, generator=g).half()
+    y = torch.zeros(1, 1, 1024, dtype=torch.float16, device=DEV)
+    cpp_gpu.rocblas_bmm_template_xAy(0, p.to(DEV), enc.to(DEV), y, 1, 1024, 50)
+    torch.cuda.synchronize()
+    assert maxabs(y, torch.matmul(p.double(), enc.double()).float()) <= 2e-3
