@@ -22,6 +22,33 @@
 
 namespace pimhip
 {
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov_f32(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
+// Sum over all lanes that share (lane & 3); every lane receives the total of its class.
+__device__ __forceinline__ float wave_sum_mod4(float v)
+{
+    v += dpp_mov_f32<0x124>(v);  // row_ror:4
+    v += dpp_mov_f32<0x128>(v);  // row_ror:8  -> total over the four quads of a row of 16 lanes
+    // v_permlane16_swap a, b exchanges rows 1 and 3 of a with rows 0 and 2 of b; v_permlane32_swap a, b exchanges the
+    // upper 32 lanes of a with the lower 32 lanes of b.  With a == b == v on entry, a + b is the pairwise sum in
+    // every lane.  (Written as asm: the compiler's builtin returns the first result twice.)
+    {
+        float a = v, b = v;
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        v = a + b;
+    }
+    {
+        float a = v, b = v;
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        v = a + b;
+    }
+    return v;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Single step.  One wavefront per hidden unit j: its four gate rows j, H+j, 2H+j, 3H+j.
 //   xproj  != nullptr : a = xproj[4H] (fp32, biases included) + W_hh h
@@ -94,20 +121,32 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
             for (int g = 0; g < 4; ++g) acc[g] = dot8(wr[g], x0, acc[g]);
         }
     }
-#pragma unroll
-    for (int g = 0; g < 4; ++g) acc[g] = wave_sum(acc[g]);
-
+    // The four gate sums are folded into one reduction: two halving exchanges leave gate l & 3 (i, f, g, o), summed over
+    // its quad, in lane l, and the rest of the tree adds the sixteen quads.  Lanes 0..3 of every quad then activate one gate
+    // each (sigmoid, and tanh(a) = 2 sigmoid(2a) - 1, on the hardware exp2 and reciprocal: absolute error below 1e-6) and
+    // quad broadcasts hand the four gates round: a few dozen instructions where four separate sums and five activations
+    // with full divisions in one lane took a tenth of a short launch.
+    const bool b0 = lane & 1, b1 = lane & 2;
+    const float a0 = (b0 ? acc[1] : acc[0]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[0] : acc[1]);
+    const float a1 = (b0 ? acc[3] : acc[2]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[2] : acc[3]);
+    float a = (b1 ? a1 : a0) + dpp_mov_f32<kDppQuadXor2>(b1 ? a0 : a1);
+    a = wave_sum_mod4(a);
+    const int gate = lane & 3;
+    if (xproj)
+        a += xproj[(long)gate * H + j];
+    else if (bsum)
+        a += bsum[(long)gate * H + j];
+    const bool is_g = gate == 2;
+    const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
+    const float act = is_g ? 2.0f * sg - 1.0f : sg;
+    const float g_i = dpp_mov_f32<0x00>(act);  // quad_perm broadcasts of lanes 0, 1, 2, 3 of the quad
+    const float g_f = dpp_mov_f32<0x55>(act);
+    const float g_g = dpp_mov_f32<0xAA>(act);
+    const float g_o = dpp_mov_f32<0xFF>(act);
+    const float c_prev = c_in_f16 ? (float)c_in_f16[j] : c_state[j];
+    const float c_new = g_f * c_prev + g_i * g_g;
+    const half_t h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
     if (lane == 0) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            if (xproj)
-                acc[g] += xproj[(long)g * H + j];
-            else if (bsum)
-                acc[g] += bsum[(long)g * H + j];
-        }
-        const float c_prev = c_in_f16 ? (float)c_in_f16[j] : c_state[j];
-        const float c_new = sigmoid_f32(acc[1]) * c_prev + sigmoid_f32(acc[0]) * tanh_f32(acc[2]);
-        const half_t h_new = (half_t)(sigmoid_f32(acc[3]) * tanh_f32(c_new));
         c_state[j] = c_new;
         h_out[j] = h_new;
         if (hn_f16) hn_f16[j] = h_new;
@@ -172,33 +211,6 @@ static constexpr int kSeqMaxHWide = 2048;  // 64 lanes x 32 columns (eight units
 static constexpr int kSeqEntryWords = 16;  // 32-bit words between the entries of consecutive blocks (64 bytes)
 static constexpr int kSeqMaxT = 1 << 30;    // super-steps per launch (the counters are 32-bit)
 static constexpr int kSeqMaxChains = 4;
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_mov_f32(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-
-// Sum over all lanes that share (lane & 3); every lane receives the total of its class.
-__device__ __forceinline__ float wave_sum_mod4(float v)
-{
-    v += dpp_mov_f32<0x124>(v);  // row_ror:4
-    v += dpp_mov_f32<0x128>(v);  // row_ror:8  -> total over the four quads of a row of 16 lanes
-    // v_permlane16_swap a, b exchanges rows 1 and 3 of a with rows 0 and 2 of b; v_permlane32_swap a, b exchanges the
-    // upper 32 lanes of a with the lower 32 lanes of b.  With a == b == v on entry, a + b is the pairwise sum in
-    // every lane.  (Written as asm: the compiler's builtin returns the first result twice.)
-    {
-        float a = v, b = v;
-        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-        v = a + b;
-    }
-    {
-        float a = v, b = v;
-        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-        v = a + b;
-    }
-    return v;
-}
 
 struct LstmSeqChain {
     const half_t* w_hh;   // [4H, H]
