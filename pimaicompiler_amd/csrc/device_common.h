@@ -58,8 +58,19 @@ __device__ __forceinline__ float wave_sum(float v)
     v += dpp_f32<kDppQuadXor2>(v);
     v += dpp_f32<kDppRowHalfMirror>(v);
     v += dpp_f32<kDppRowMirror>(v);
-    v += __shfl_xor(v, 16, kWave);
-    v += __shfl_xor(v, 32, kWave);
+    // The two steps across rows of 16 lanes: v_permlane16_swap a, b exchanges rows 1 and 3 of a with rows 0 and 2 of b,
+    // v_permlane32_swap a, b the upper 32 lanes of a with the lower 32 of b; with a == b == v on entry, a + b is the
+    // pairwise sum in every lane.  (No trip through the LDS crossbar, which the generic shuffle takes.)
+    {
+        float a = v, b = v;
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        v = a + b;
+    }
+    {
+        float a = v, b = v;
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        v = a + b;
+    }
     return v;
 }
 
