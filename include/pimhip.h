@@ -424,6 +424,33 @@ int pimhip_rnnt_plan_destroy(PimHipRnntPlan* plan);
 int pimhip_rnnt_step(PimHipRnntPlan* plan, const void* x, const void* h_prev, const void* c_prev, const void* f, void* hn,
                      void* cn, void* logits, void* joint_hidden, int run_prediction, void* stream);
 
+/* The whole greedy decoding loop over one utterance in one launch: what the reference interprets operator by operator per
+ * iteration of prim::Loop (runtime/source/executor/op_executor/prim_ops_executor.cpp:820-875: executeAtenLSTM1 with
+ * seq_len == 1, the joint network's executeAtenAddmm calls and executeAtenArgmax, aten_ops_executor.cpp:520-560, whose
+ * result the host reads before the next iteration).
+ *
+ *     t = 0; g, state = prediction(x0, (h0, c0))          (run_prediction_first == 0: g = h0 of the last layer as it is)
+ *     while t < n_frames and fewer than max_symbols emitted:
+ *         k = argmax(logits(enc[t], g))                    (fp16 logits; the first maximum, a NaN counting as the largest)
+ *         if k == blank: t += 1
+ *         else: symbols[n++] = k; g, state = prediction(embedding[k], state);
+ *               after max_symbols_per_frame symbols of one frame: t += 1
+ *
+ *   enc [n_frames, enc_size], embedding [embedding_rows >= vocab, input_size] (row k: the prediction network's input after
+ *   symbol k), x0 [input_size] (its input before any symbol), h0 / c0 [num_layers, H] or null (zeros), hn / cn the same
+ *   shape or null, not overlapping h0 / c0; symbols [max_symbols] int32; result [8] int32: symbols emitted, frames
+ *   consumed, steps taken, 1 if one workgroup had to decode alone, 1 if the last symbol has not been fed to the prediction
+ *   network yet (hn / cn are the state before it), the last symbol (-1: none), 0, 0.  All device memory; fp16 tensors
+ *   dense and 16-byte aligned.  vocab <= 64 (PIMHIP_ERR_UNSUPPORTED otherwise: drive pimhip_rnnt_step from the host).
+ * Symbols and final state equal, bit for bit, those of the same loop driven from the host through pimhip_rnnt_step.
+ * Asynchronous; records three kernels, so it can be recorded into a HIP graph.  Residency, ordering and the plan's stream
+ * as for pimhip_rnnt_step.  Every wait inside is bounded; when one gives up, one workgroup decodes the utterance again from
+ * its start by itself inside the same launch (slower, the same result), and the event counts for the plan like a step's. */
+int pimhip_rnnt_greedy_decode(PimHipRnntPlan* plan, const void* enc, int64_t n_frames, const void* embedding, int64_t embedding_rows,
+                              const void* x0, const void* h0, const void* c0, int run_prediction_first, int blank,
+                              int max_symbols_per_frame, int64_t max_symbols, int32_t* symbols, int32_t* result, void* hn, void* cn,
+                              void* stream);
+
 /* No counterpart in the reference.  As pimhip_moe_plan_fallbacks / pimhip_moe_plan_set_spin_limit. */
 int pimhip_rnnt_plan_fallbacks(PimHipRnntPlan* plan, uint64_t* events, int* exchanging);
 int pimhip_rnnt_plan_set_spin_limit(PimHipRnntPlan* plan, unsigned int spin_limit);

@@ -83,6 +83,10 @@ SIGNATURES = {
                                                ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]),
     "pimhip_rnnt_plan_destroy": (ctypes.c_int, [ctypes.c_void_p]),
     "pimhip_rnnt_step": (ctypes.c_int, [ctypes.c_void_p] * 9 + [ctypes.c_int, ctypes.c_void_p]),
+    "pimhip_rnnt_greedy_decode": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64,
+                                                 ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                 ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                                 ctypes.c_void_p]),
     "pimhip_rnnt_plan_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), c_int_p]),
     "pimhip_rnnt_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "pimhip_input_projection": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

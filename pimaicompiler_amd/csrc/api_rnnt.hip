@@ -1,7 +1,8 @@
-// The RNN-transducer step of the C ABI (include/pimhip.h): the prediction network's LSTM cells at seq_len 1 and the joint
-// network's two products in one launch.
+// The RNN-transducer entry points of the C ABI (include/pimhip.h): one step of the greedy decoding loop (the prediction
+// network's LSTM cells at seq_len 1 and the joint network's two products) in one launch, and the whole loop over an
+// utterance in one launch.
 #include "api_common.h"
-#include "rnnt_kernels.h"
+#include "rnnt_greedy_kernels.h"
 
 using namespace pimhip;
 
@@ -18,6 +19,10 @@ struct PimHipRnntPlan {
     float* bsum = nullptr;                 // [num_layers][4H], or null without biases
     unsigned long long* hx = nullptr;      // [2][blocks][kRnntEntryWords], all ones = empty
     unsigned int* g_counter = nullptr;     // [blocks][kRnntCounterStride]
+    unsigned int* greedy = nullptr;        // what the loop kernel exchanges through, refilled before every launch of it:
+                                           // [kRnntGreedySets][blocks][kRnntEntryWords] 8-byte words (all ones), then
+                                           // seen [blocks][kRnntSeenStride] and solo_owner (zero)
+    bool greedy_resident = false;          // all workgroups of the loop kernel fit on the device together
     unsigned int* abort_flag = nullptr;
     unsigned int* abort_host = nullptr;
     unsigned int* abort_host_dev = nullptr;
@@ -34,6 +39,8 @@ std::vector<PimHipRnntPlan*> g_rnnt_plans;
 constexpr unsigned long long kRnntEventsBeforeAlone = 3;  // waits given up before a plan stops exchanging for good
 
 size_t exchange_words32(const PimHipRnntPlan* plan) { return (size_t)2 * plan->blocks * kRnntEntryWords * 2; }
+size_t greedy_exchange_words32(const PimHipRnntPlan* plan) { return (size_t)kRnntGreedySets * plan->blocks * kRnntEntryWords * 2; }
+size_t greedy_count_words32(const PimHipRnntPlan* plan) { return (size_t)plan->blocks * kRnntSeenStride + kRnntSeenStride; }
 
 int destroy_rnnt_plan_locked(PimHipRnntPlan* plan)
 {
@@ -45,6 +52,7 @@ int destroy_rnnt_plan_locked(PimHipRnntPlan* plan)
     if (plan->bsum) hipFree(plan->bsum);
     if (plan->hx) hipFree(plan->hx);
     if (plan->g_counter) hipFree(plan->g_counter);
+    if (plan->greedy) hipFree(plan->greedy);
     if (plan->abort_flag) hipFree(plan->abort_flag);
     if (plan->abort_host) hipHostFree(plan->abort_host);
     if (prev >= 0) hipSetDevice(prev);
@@ -145,6 +153,12 @@ extern "C" int pimhip_rnnt_plan_create(PimHipRnntPlan** plan_out, const void* co
     launch_fill_u32(reinterpret_cast<unsigned int*>(plan->hx), exchange_words32(plan), ~0u, s);
     RNNT_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&plan->g_counter), sizeof(unsigned int) * (size_t)plan->blocks * kRnntCounterStride));
     launch_fill_u32(plan->g_counter, (size_t)plan->blocks * kRnntCounterStride, 0u, s);
+    RNNT_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&plan->greedy), sizeof(unsigned int) * (greedy_exchange_words32(plan) + greedy_count_words32(plan))));
+    {
+        int greedy_per_cu = 0;
+        RNNT_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&greedy_per_cu, rnnt_greedy_f16_kernel, kRnntThreads, 0));
+        plan->greedy_resident = (int64_t)greedy_per_cu * st->num_cus >= blocks;
+    }
     RNNT_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&plan->abort_flag), sizeof(unsigned int)));
     launch_fill_u32(plan->abort_flag, 1, 0u, s);
     RNNT_HIP_CHECK(hipGetLastError());
@@ -213,7 +227,7 @@ extern "C" int pimhip_rnnt_step(PimHipRnntPlan* plan, const void* x, const void*
     PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
     const bool capturing = capture != hipStreamCaptureStatusNone;
     if (*plan->abort_host != 0u && !capturing) {
-        // A wait of an earlier step gave up.  That step's result was completed by the blocks themselves, and every step
+        // A wait of an earlier launch gave up.  That step's result was completed by the blocks themselves, and every step
         // since has run self-sufficient (the abort word stays up on the device); here, outside any capture, the exchange is
         // put back in order: drain the stream (steps sharing a plan are ordered on one stream), refill the entries, clear
         // the words.  A plan that has needed this kRnntEventsBeforeAlone times stops exchanging for good.
@@ -259,6 +273,107 @@ extern "C" int pimhip_rnnt_step(PimHipRnntPlan* plan, const void* x, const void*
     rnnt_step_f16_kernel<<<dim3((unsigned)plan->blocks), dim3(kRnntThreads), 0, s>>>(
         (const half_t*)x, (const half_t*)h_prev, (const half_t*)c_prev, (const half_t*)f, plan->num_layers, (int)plan->hidden,
         (int)plan->joint_size, run_prediction ? 1 : 0, a);
+    PIMHIP_HIP_CHECK(hipGetLastError());
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_rnnt_greedy_decode(PimHipRnntPlan* plan, const void* enc, int64_t n_frames, const void* embedding,
+                                         int64_t embedding_rows, const void* x0, const void* h0, const void* c0, int run_prediction_first,
+                                         int blank, int max_symbols_per_frame, int64_t max_symbols, int32_t* symbols, int32_t* result,
+                                         void* hn, void* cn, void* stream)
+{
+    DeviceState* st = nullptr;
+    int rc = current_device_state(&st);
+    if (rc != PIMHIP_OK) return rc;
+    if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
+    int dev = -1;
+    PIMHIP_HIP_CHECK(hipGetDevice(&dev));
+    if (dev != plan->device) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan belongs to device %d, current device is %d", plan->device, dev);
+    if (!embedding || !result || (!enc && n_frames > 0) || (!symbols && max_symbols > 0))
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "enc, embedding, symbols and result must be non-null");
+    if (n_frames < 0 || n_frames > INT32_MAX || max_symbols < 0 || max_symbols > INT32_MAX || max_symbols_per_frame < 1)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "n_frames=%lld, max_symbols=%lld, max_symbols_per_frame=%d", (long long)n_frames,
+                    (long long)max_symbols, max_symbols_per_frame);
+    if (plan->vocab > kRnntGreedyMaxVocab)
+        return fail(PIMHIP_ERR_UNSUPPORTED, "the one-launch loop takes up to %d symbols (the plan has %lld): drive pimhip_rnnt_step from the host",
+                    kRnntGreedyMaxVocab, (long long)plan->vocab);
+    if (blank < 0 || blank >= plan->vocab) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "blank=%d not in [0, %lld)", blank, (long long)plan->vocab);
+    if (embedding_rows < plan->vocab)
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "embedding has %lld rows, the joint network emits %lld symbols", (long long)embedding_rows,
+                    (long long)plan->vocab);
+    if (run_prediction_first && !x0) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "x0 must be non-null when the first step runs the prediction network");
+    if (!aligned16(enc) || !aligned16(embedding) || !aligned16(x0) || !aligned16(h0))
+        return fail(PIMHIP_ERR_UNSUPPORTED, "enc, embedding, x0 and h0 must be 16-byte aligned");
+    const size_t state_bytes = sizeof(half_t) * (size_t)plan->num_layers * plan->hidden;
+    // A workgroup that has to decode alone starts again from h0 / c0.
+    if ((hn && h0 && overlap(hn, state_bytes, h0, state_bytes)) || (hn && c0 && overlap(hn, state_bytes, c0, state_bytes)) ||
+        (cn && h0 && overlap(cn, state_bytes, h0, state_bytes)) || (cn && c0 && overlap(cn, state_bytes, c0, state_bytes)))
+        return fail(PIMHIP_ERR_INVALID_ARGUMENT, "hn / cn must not overlap h0 / c0");
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
+    const bool capturing = capture != hipStreamCaptureStatusNone;
+    if (*plan->abort_host != 0u && !capturing) {
+        // as in pimhip_rnnt_step: a wait of an earlier launch gave up (its result was completed all the same)
+        PIMHIP_HIP_CHECK(hipStreamSynchronize(s));
+        *plan->abort_host = 0u;
+        ++plan->gave_up_events;
+        if (plan->gave_up_events >= kRnntEventsBeforeAlone) plan->alone = true;
+        launch_fill_u32(reinterpret_cast<unsigned int*>(plan->hx), exchange_words32(plan), ~0u, s);
+        launch_fill_u32(plan->g_counter, (size_t)plan->blocks * kRnntCounterStride, 0u, s);
+        launch_fill_u32(plan->abort_flag, 1, 0u, s);
+        PIMHIP_HIP_CHECK(hipGetLastError());
+    }
+    RnntGreedyArgs a;
+    memset(&a, 0, sizeof(a));
+    const int n4 = (int)(4 * plan->hidden);
+    for (int l = 0; l < plan->num_layers; ++l) {
+        a.layer[l].w_ih = plan->w_ih[l];
+        a.layer[l].w_hh = plan->w_hh[l];
+        a.layer[l].bsum = plan->bsum ? plan->bsum + (size_t)l * n4 : nullptr;
+        a.layer[l].in_w = (int)(l == 0 ? plan->input_size : plan->hidden);
+    }
+    a.w1 = plan->w1;
+    a.b1 = plan->b1;
+    a.w2 = plan->w2;
+    a.b2 = plan->b2;
+    a.enc = (const half_t*)enc;
+    a.embedding = (const half_t*)embedding;
+    a.x0 = (const half_t*)x0;
+    a.h0 = (const half_t*)h0;
+    a.c0 = (const half_t*)c0;
+    a.hn = (half_t*)hn;
+    a.cn = (half_t*)cn;
+    a.symbols = symbols;
+    a.result = result;
+    a.hx = reinterpret_cast<unsigned long long*>(plan->greedy);
+    a.seen = plan->greedy + greedy_exchange_words32(plan);
+    a.solo_owner = a.seen + (size_t)plan->blocks * kRnntSeenStride;
+    a.abort_flag = plan->abort_flag;
+    a.abort_host = plan->abort_host_dev;
+    a.L = plan->num_layers;
+    a.H = (int)plan->hidden;
+    a.F = (int)plan->enc_size;
+    a.J = (int)plan->joint_size;
+    a.V = (int)plan->vocab;
+    a.T = (int)n_frames;
+    a.emb_rows = (int)embedding_rows;
+    a.emb_in_lds = (embedding_rows + 1) * plan->input_size <= kRnntGreedyEmbHalfs ? 1 : 0;
+    a.blank = blank;
+    a.max_symbols = (int)max_symbols;
+    a.max_per_frame = max_symbols_per_frame;
+    a.run_pred_first = run_prediction_first ? 1 : 0;
+    a.spin_limit = plan->spin_limit;
+    a.alone = (plan->alone || !plan->greedy_resident) ? 1 : 0;
+    if (!capturing) {
+        rc = order_after_previous_sequence_launch(st, s);
+        if (rc != PIMHIP_OK) return rc;
+    }
+    // fill kernels, not memsets: the call can be recorded into a HIP graph
+    launch_fill_u32(plan->greedy, greedy_exchange_words32(plan), ~0u, s);
+    launch_fill_u32(plan->greedy + greedy_exchange_words32(plan), greedy_count_words32(plan), 0u, s);
+    rnnt_greedy_f16_kernel<<<dim3(a.alone ? 1u : (unsigned)plan->blocks), dim3(kRnntThreads), 0, s>>>(a);
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
 }

@@ -105,10 +105,19 @@ struct RnntStepArgs {
 // which nothing here depends on.
 __device__ __forceinline__ void rnnt_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// An fp32 value rounded to fp16 in a step of its own.  Where the rounding is the only use of a multiply-add's result the
+// compiler folds it into that instruction (v_fma_mixlo_f16), which rounds once instead of twice and differs in the last bit
+// now and then; whoever computes a unit, in whatever surrounding code, has to get the same bits.
+__device__ __forceinline__ half_t rnnt_round(float v)
+{
+    asm volatile("" : "+v"(v));
+    return (half_t)v;
+}
+
 // The bits a value travels as: a NaN in its canonical form (an all-ones half word means "empty").
 __device__ __forceinline__ unsigned short rnnt_bits(float a)
 {
-    unsigned short bits = __builtin_bit_cast(unsigned short, (half_t)a);
+    unsigned short bits = __builtin_bit_cast(unsigned short, rnnt_round(a));
     if (a != a) bits = 0x7e00u;
     return bits;
 }
@@ -175,7 +184,7 @@ __device__ __forceinline__ void rnnt_unit(const float acc[4], float bias, float 
     const float g_g = rnnt_dpp<0xAA>(act);
     const float g_o = rnnt_dpp<0xFF>(act);
     c_new = __builtin_fmaf(g_f, c_prev, g_i * g_g);
-    h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
+    h_new = rnnt_round(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
 }
 
 // The chain of the step up to `upto` by this workgroup alone: upto < L gives h of layer `upto`, upto == L the joint
@@ -390,7 +399,7 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_step_f16_kernel(const half_
         publish(set);
         if (lane == 0) {  // (behind the word the next role waits for)
             p.hn[(long)l * H + u] = h_new;
-            p.cn[(long)l * H + u] = (half_t)c_new;
+            p.cn[(long)l * H + u] = rnnt_round(c_new);
         }
     } else if (b < n_lstm + nwj) {
         // ---- the joint network's first layer: row r of W1 over cat(f, g) ----
@@ -458,7 +467,7 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_step_f16_kernel(const half_
         for (int k = 0; k < kRnntJC; ++k)
             if (lane + 64 * k < njp) a = dot8(wv[k], in[lane + 64 * k], a);
         a = rnnt_sum(a);
-        if (lane == 0 && v < p.V) p.logits[v] = (half_t)(a + bias);
+        if (lane == 0 && v < p.V) p.logits[v] = rnnt_round(a + bias);
     }
     // this block's entry of the other set is empty for the next launch (nobody reads that set during this one)
     const unsigned int set = g & 1u;

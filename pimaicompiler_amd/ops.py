@@ -1044,6 +1044,38 @@ class RnntPlan:
             _check(lib.pimhip_rnnt_step(*args, _stream_handle(stream)))
         return step
 
+    def greedy_decode(self, enc, embedding, x0, blank, max_symbols_per_frame=30, max_symbols=None, h0=None, c0=None,
+                      run_prediction_first=True, stream=None):
+        """The greedy decoding loop over the frames enc [T, F] in one launch (pimhip_rnnt_greedy_decode): returns
+        (symbols int32 [max_symbols], result int32 [8], hn, cn [L, H]), all on the device and not synchronised; result[0] is
+        the number of symbols.  embedding [rows >= V, I]: row k is the prediction network's input after symbol k; x0 [I] its
+        input before any symbol."""
+        lib = L.load()
+        enc, embedding = enc.contiguous(), embedding.contiguous()
+        given = [t for t in (enc, embedding, x0, h0, c0) if t is not None]
+        _require_half_cuda(*given)
+        if enc.dim() != 2 or enc.size(1) != self.enc_size:
+            raise NNRuntimeException(f"enc must be [T, {self.enc_size}]")
+        if embedding.dim() != 2 or embedding.size(1) != self.input_size:
+            raise NNRuntimeException(f"embedding must be [rows, {self.input_size}]")
+        n_state = self.num_layers * self.hidden
+        for t, n, name in ((x0, self.input_size, "x0"), (h0, n_state, "h0"), (c0, n_state, "c0")):
+            if t is not None and (t.numel() != n or not t.is_contiguous()):
+                raise NNRuntimeException(f"{name} must be contiguous with {n} elements")
+        n_frames = enc.size(0)
+        if max_symbols is None:
+            max_symbols = n_frames * max_symbols_per_frame
+        symbols = torch.empty(max(int(max_symbols), 1), dtype=torch.int32, device=self.device)
+        result = torch.zeros(8, dtype=torch.int32, device=self.device)
+        hn = torch.empty(self.num_layers, self.hidden, dtype=torch.float16, device=self.device)
+        cn = torch.empty_like(hn)
+        ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+        _check(lib.pimhip_rnnt_greedy_decode(self._handle, enc.data_ptr(), n_frames, embedding.data_ptr(), embedding.size(0), ptr(x0),
+                                             ptr(h0), ptr(c0), int(bool(run_prediction_first)), int(blank), int(max_symbols_per_frame),
+                                             int(max_symbols), symbols.data_ptr(), result.data_ptr(), hn.data_ptr(), cn.data_ptr(),
+                                             _stream_handle(stream)))
+        return symbols[:int(max_symbols)], result, hn, cn
+
     def forward(self, x, h_prev, c_prev, f, run_prediction=True, stream=None):
         """logits [V], hn, cn [L, H] for one step (new tensors; with run_prediction False hn, cn are h_prev, c_prev)."""
         logits = torch.empty(self.vocab, dtype=torch.float16, device=self.device)

@@ -1,0 +1,211 @@
+"""The one-launch greedy decoding loop (pimhip_rnnt_greedy_decode) against the same loop driven from the host through
+pimhip_rnnt_step (which tests/test_rnnt_gpu.py holds against LibTorch CPU): symbols, counts and final state bit for bit, as
+both sum in the same order and round the state to fp16 between runs of the prediction network.  Integer outputs and fp16
+bits: no tolerance."""
+import pytest
+import torch
+
+from test_rnnt_gpu import DEV, dev, make
+
+pytestmark = pytest.mark.gpu
+
+
+def model(seed, L, I, H, F, J, V, T, blank, blank_bias, biases=True, w2_scale=0.1):
+    """A transducer with random weights whose joint network prefers `blank` by `blank_bias` (a real model emits mostly
+    blanks; with plain random weights every frame would emit symbols up to the per-frame limit)."""
+    g, params, joint = make(seed, L, I, H, F, J, V, biases)
+    w1, b1, w2, b2 = joint
+    w2 = (w2.float() * w2_scale).half()
+    if b2 is not None:
+        b2 = b2.clone()
+        b2[blank] += blank_bias
+    enc = torch.randn(T, F, generator=g).half().to(DEV)
+    embedding = torch.randn(V, I, generator=g).half().to(DEV)
+    x0 = torch.zeros(I, dtype=torch.float16, device=DEV)
+    return params, (w1, b1, w2, b2), enc, embedding, x0
+
+
+def argmax_like_torch(logits):
+    """torch.argmax of the fp16 logits: the first maximum, a NaN counting as the largest."""
+    nan = torch.isnan(logits)
+    if bool(nan.any()):
+        return int(nan.float().argmax())
+    return int(torch.argmax(logits.float()))
+
+
+def loop_driven_from_the_host(plan, enc, embedding, x0, blank, per_frame, max_symbols, h0=None, c0=None, run_prediction_first=True):
+    """The loop of pimhip_rnnt_greedy_decode, one pimhip_rnnt_step and one read of the logits per iteration."""
+    L, H = plan.num_layers, plan.hidden
+    h = torch.zeros(L, H, dtype=torch.float16, device=DEV) if h0 is None else h0.clone()
+    c = torch.zeros(L, H, dtype=torch.float16, device=DEV) if c0 is None else c0.clone()
+    t, symbols, in_frame, run_prediction, label, steps = 0, [], 0, run_prediction_first, -1, 0
+    while t < enc.size(0) and len(symbols) < max_symbols:
+        if run_prediction:
+            logits, h, c = plan.forward(x0 if label < 0 else embedding[label], h, c, enc[t], True)
+        else:
+            logits, _, _ = plan.forward(None, h, None, enc[t], False)
+        k = argmax_like_torch(logits)
+        steps += 1
+        if k == blank:
+            t, in_frame, run_prediction = t + 1, 0, False
+        else:
+            symbols.append(k)
+            label, in_frame, run_prediction = k, in_frame + 1, True
+            if in_frame >= per_frame:
+                t, in_frame = t + 1, 0
+    return symbols, t, steps, h, c, run_prediction, label
+
+
+def check(got, want):
+    symbols, result, hn, cn = got
+    torch.cuda.synchronize()
+    r = result.cpu().tolist()
+    w_symbols, w_t, w_steps, w_h, w_c, w_pending, w_label = want
+    assert r[0] == len(w_symbols) and symbols[: r[0]].cpu().tolist() == w_symbols
+    assert (r[1], r[2], r[4], r[5]) == (w_t, w_steps, int(w_pending), w_label)
+    assert torch.equal(hn, w_h) and torch.equal(cn, w_c)
+    return r
+
+
+CASES = [
+    # L, I, H, F, J, V, T, blank, per_frame, max_symbols, blank_bias, biases
+    (2, 320, 320, 1024, 512, 29, 120, 28, 30, None, 0.62, True),     # the RNNT shapes, mostly blanks
+    (2, 320, 320, 1024, 512, 29, 60, 28, 7, None, 0.7, True),
+    (2, 320, 320, 1024, 512, 29, 40, 28, 30, None, 0.3, True),       # mostly symbols: frames end at the per-frame limit
+    (2, 320, 320, 1024, 512, 29, 50, 28, 2, 37, 0.4, True),          # ends at max_symbols
+    (1, 64, 32, 128, 64, 5, 12, 0, 3, None, 0.3, True),
+    (3, 72, 136, 200, 1024, 8, 40, 3, 4, None, 0.2, False),
+    (4, 1024, 256, 2048, 512, 64, 25, 63, 5, None, 0.5, True),       # widest x and f, embedding rows read from memory
+    (1, 64, 32, 128, 64, 5, 0, 0, 3, None, 0.3, True),               # no frames
+]
+
+
+@pytest.mark.parametrize("L,I,H,F,J,V,T,blank,per_frame,max_symbols,blank_bias,biases", CASES)
+def test_one_launch_gives_what_the_loop_driven_from_the_host_gives(ops, L, I, H, F, J, V, T, blank, per_frame, max_symbols, blank_bias, biases):
+    params, joint, enc, embedding, x0 = model(900 + L + H + T, L, I, H, F, J, V, T, blank, blank_bias, biases)
+    plan = ops.RnntPlan(dev(params), biases, L, tuple(dev(joint)))
+    cap = T * per_frame if max_symbols is None else max_symbols
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, per_frame, cap)
+    r = check(plan.greedy_decode(enc, embedding, x0, blank, per_frame, max_symbols), want)
+    assert r[3] == 0 and plan.fallbacks() == (0, True)
+    # again on the same plan (the exchange is refilled by every call), now with a state to start from
+    h0 = (0.3 * torch.randn(L, H)).half().to(DEV)
+    c0 = torch.randn(L, H).half().to(DEV)
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, per_frame, cap, h0, c0)
+    check(plan.greedy_decode(enc, embedding, x0, blank, per_frame, max_symbols, h0=h0, c0=c0), want)
+    assert plan.fallbacks() == (0, True)
+
+
+def test_the_mix_of_blanks_and_symbols_is_a_real_one(ops):
+    """The cases here are meant to mix the two kinds of step: many frames pass with a blank, some emit symbols."""
+    L, I, H, F, J, V, T, blank = 2, 320, 320, 1024, 512, 29, 60, 28
+    params, joint, enc, embedding, x0 = model(6161, L, I, H, F, J, V, T, blank, 0.75)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    _, result, _, _ = plan.greedy_decode(enc, embedding, x0, blank)
+    torch.cuda.synchronize()
+    n, frames, steps = result.cpu().tolist()[:3]
+    assert frames == T and n >= 30 and steps >= n + T // 2
+
+
+def test_decoding_goes_on_where_a_chunk_of_frames_ended(ops):
+    """Frames arrive in chunks: the second call starts from the first one's state, with the last symbol still to be fed to
+    the prediction network or not as result[4] says.  Together they give what one call over all frames gives."""
+    L, I, H, F, J, V, T, blank = 2, 320, 320, 1024, 512, 29, 90, 28
+    params, joint, enc, embedding, x0 = model(4242, L, I, H, F, J, V, T, blank, 0.6)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    whole = plan.greedy_decode(enc, embedding, x0, blank, 1000)
+    torch.cuda.synchronize()
+    want_n = int(whole[1][0])
+    want = whole[0][:want_n].cpu().tolist()
+    for cut in (1, 37, 60):
+        s1, r1, h1, c1 = plan.greedy_decode(enc[:cut], embedding, x0, blank, 1000)
+        torch.cuda.synchronize()
+        r1 = r1.cpu().tolist()
+        assert r1[1] == cut
+        x_next = x0 if r1[5] < 0 else embedding[r1[5]]
+        s2, r2, h2, c2 = plan.greedy_decode(enc[cut:], embedding, x_next, blank, 1000, h0=h1, c0=c1, run_prediction_first=bool(r1[4]))
+        torch.cuda.synchronize()
+        r2 = r2.cpu().tolist()
+        assert s1[: r1[0]].cpu().tolist() + s2[: r2[0]].cpu().tolist() == want, cut
+        assert torch.equal(h2, whole[2]) and torch.equal(c2, whole[3])
+    assert plan.fallbacks() == (0, True)
+
+
+def test_a_loop_whose_waits_give_up_still_gives_the_right_result(ops):
+    """Forced from the host with a spin limit of 0: the workgroups leave the loop at their first wait and one of them
+    decodes the utterance by itself, inside the same launch, to the same bits.  The events count for the plan; after the
+    third every launch is that one workgroup from the start."""
+    L, I, H, F, J, V, T, blank = 2, 320, 320, 1024, 512, 29, 30, 28
+    params, joint, enc, embedding, x0 = model(5151, L, I, H, F, J, V, T, blank, 0.55)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, 30, T * 30)
+    assert len(want[0]) >= 10
+    plan.set_spin_limit(0)
+    for i in range(4):
+        r = check(plan.greedy_decode(enc, embedding, x0, blank), want)
+        assert r[3] == 1, i
+    events, exchanging = plan.fallbacks()
+    assert events >= 3 and not exchanging
+    plan.set_spin_limit(1 << 22)
+    r = check(plan.greedy_decode(enc, embedding, x0, blank), want)
+    assert r[3] == 1 and plan.fallbacks() == (events, False)
+    # a fresh plan is a team again
+    plan2 = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    r = check(plan2.greedy_decode(enc, embedding, x0, blank), want)
+    assert r[3] == 0 and plan2.fallbacks() == (0, True)
+
+
+def test_the_loop_recorded_into_a_graph_replays_like_the_eager_call(ops):
+    L, I, H, F, J, V, T, blank = 2, 320, 320, 1024, 512, 29, 60, 28
+    params, joint, enc, embedding, x0 = model(6161, L, I, H, F, J, V, T, blank, 0.75)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, 30, T * 30)
+    from pimaicompiler_amd import _lib
+    from pimaicompiler_amd.ops import _check
+    lib = _lib.load()
+    symbols = torch.empty(T * 30, dtype=torch.int32, device=DEV)
+    result = torch.zeros(8, dtype=torch.int32, device=DEV)
+    hn = torch.empty(L, H, dtype=torch.float16, device=DEV)
+    cn = torch.empty_like(hn)
+
+    def call(stream):
+        _check(lib.pimhip_rnnt_greedy_decode(plan._handle, enc.data_ptr(), T, embedding.data_ptr(), V, x0.data_ptr(), None, None, 1,
+                                                 blank, 30, T * 30, symbols.data_ptr(), result.data_ptr(), hn.data_ptr(), cn.data_ptr(),
+                                                 stream))
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(4):
+        for t in (symbols, result, hn, cn):
+            t.fill_(7)
+        graph.replay()
+        check((symbols, result, hn, cn), want)
+        check(plan.greedy_decode(enc, embedding, x0, blank), want)      # eager calls between the replays
+    assert plan.fallbacks() == (0, True)
+
+
+def test_arguments_the_loop_refuses(ops):
+    L, I, H, F, J, V, T = 2, 320, 320, 1024, 512, 29, 8
+    params, joint, enc, embedding, x0 = model(7171, L, I, H, F, J, V, T, 28, 0.5)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    with pytest.raises(ops.NNRuntimeException, match="blank"):
+        plan.greedy_decode(enc, embedding, x0, 29)
+    with pytest.raises(ops.NNRuntimeException, match="rows"):
+        plan.greedy_decode(enc, embedding[:20], x0, 28)
+    with pytest.raises(ops.NNRuntimeException, match="max_symbols_per_frame"):
+        plan.greedy_decode(enc, embedding, x0, 28, 0)
+    with pytest.raises(ops.NNRuntimeException, match="x0"):
+        plan.greedy_decode(enc, embedding, None, 28)
+    with pytest.raises(ops.NNRuntimeException, match=r"\[T, 1024\]"):
+        plan.greedy_decode(enc[:, :512], embedding, x0, 28)
+    # more symbols than one wavefront's ballot takes
+    g2, params2, joint2 = make(7272, 1, 64, 32, 128, 64, 130, True)
+    plan2 = ops.RnntPlan(dev(params2), True, 1, tuple(dev(joint2)))
+    with pytest.raises(ops.NNRuntimeException, match="symbols"):
+        plan2.greedy_decode(torch.zeros(4, 128, dtype=torch.float16, device=DEV), torch.zeros(130, 64, dtype=torch.float16, device=DEV),
+                            torch.zeros(64, dtype=torch.float16, device=DEV), 0)
