@@ -628,6 +628,43 @@ def main():
                                                                       float((rn_cn.float() - rn_cn2.float()).abs().max())), 6),
             "max_abs_diff_of_logits_to_the_four_launches": round(float((rn_logits.float() - jout.float()).abs().max()), 6),
             "waits_that_gave_up": rn_plan.fallbacks()[0] - rn_events}
+        # The whole greedy loop over an utterance in one launch (pimhip_rnnt_greedy_decode), timed on its two kinds of step:
+        # with the joint network's bias pushed towards the blank every frame passes with one step of the joint network alone;
+        # pushed away from it every step emits a symbol and runs the prediction network (30 per frame).  Beside them the same
+        # loop driven from the host: one pimhip_rnnt_step and one read of the argmax per iteration.
+        progress("other: RNNT greedy decoding loop in one launch")
+        gd_T, gd_blank = 400, 28
+        gd_enc = torch.randn(gd_T, 1024, device=dev).half()
+        gd_emb, gd_x0 = torch.randn(29, 320, device=dev).half(), torch.zeros(320, dtype=torch.float16, device=dev)
+        greedy = {}
+        for kind, push, frames in (("after_a_blank", 20.0, gd_T), ("with_a_symbol", -20.0, 40)):
+            b2 = jb2.clone()
+            b2[gd_blank] += push
+            gd_plan = P.RnntPlan(rn_prm, True, 2, (jw1, jb1, jw2, b2))
+            enc_k = gd_enc[:frames]
+            _, gd_res, _, _ = gd_plan.greedy_decode(enc_k, gd_emb, gd_x0, gd_blank)
+            torch.cuda.synchronize()
+            steps_k = int(gd_res[2])
+            us = timed_us(lambda: gd_plan.greedy_decode(enc_k, gd_emb, gd_x0, gd_blank), 10)
+            # the host's loop over the first frames of the same utterance
+            h_, c_ = torch.zeros(2, 320, dtype=torch.float16, device=dev), torch.zeros(2, 320, dtype=torch.float16, device=dev)
+            hn_, cn_ = torch.empty_like(h_), torch.empty_like(c_)
+            lg_ = torch.empty(29, dtype=torch.float16, device=dev)
+            n_host = 200
+            first = gd_plan.bind(gd_x0, h_, c_, enc_k[0], hn_, cn_, lg_)
+            full_ = gd_plan.bind(gd_emb[3], h_, c_, enc_k[0], hn_, cn_, lg_)
+            blank_ = gd_plan.bind(None, hn_, None, enc_k[1], None, None, lg_, run_prediction=False)
+            first()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n_host):
+                (blank_ if kind == "after_a_blank" else full_)()
+                k_ = int(torch.argmax(lg_))          # the read that decides the next iteration
+            host_us = (time.perf_counter() - t0) / n_host * 1e6
+            greedy[kind] = {"steps": steps_k, "us_per_step": round(us / max(steps_k, 1), 3),
+                            "driven_from_the_host_us_per_step": round(host_us, 2),
+                            "one_workgroup_decoded_alone": int(gd_res[3]), "waits_that_gave_up": gd_plan.fallbacks()[0]}
+        other["rnnt_greedy_decode_one_launch"] = greedy
         # residual add (fp16, c = a + b): 32 Mi elements (6 bytes each) and the decoder's 1024-element case
         big_a, big_b = torch.randn(32 << 20, device=dev).half().view(-1, 1024), torch.randn(32 << 20, device=dev).half().view(-1, 1024)
         big_c = torch.empty_like(big_a)

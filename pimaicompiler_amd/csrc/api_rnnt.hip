@@ -39,7 +39,11 @@ std::vector<PimHipRnntPlan*> g_rnnt_plans;
 constexpr unsigned long long kRnntEventsBeforeAlone = 3;  // waits given up before a plan stops exchanging for good
 
 size_t exchange_words32(const PimHipRnntPlan* plan) { return (size_t)2 * plan->blocks * kRnntEntryWords * 2; }
-size_t greedy_exchange_words32(const PimHipRnntPlan* plan) { return (size_t)kRnntGreedySets * plan->blocks * kRnntEntryWords * 2; }
+size_t greedy_exchange_words32(const PimHipRnntPlan* plan)
+{
+    const size_t n_lstm = (size_t)plan->num_layers * (plan->hidden / 8), n_joint = plan->joint_size / 8, n_vocab = (plan->vocab + 7) / 8;
+    return (kRnntGreedyVersions * n_lstm + kRnntGreedyRing * (n_joint + n_vocab)) * kRnntEntryWords * 2;
+}
 size_t greedy_count_words32(const PimHipRnntPlan* plan) { return (size_t)plan->blocks * kRnntSeenStride + kRnntSeenStride; }
 
 int destroy_rnnt_plan_locked(PimHipRnntPlan* plan)

@@ -41,7 +41,11 @@
 namespace pimhip
 {
 
-constexpr int kRnntGreedySets = 4;
+constexpr int kRnntGreedyVersions = 4;             // h of a layer: one entry per block and version of g, modulo this
+constexpr int kRnntGreedyRing = 16;                // hidden vectors and logits: one entry per block and step, modulo this
+constexpr int kRnntGreedyAhead = 8;                // steps the joint network runs ahead of the decisions
+constexpr int kRnntGreedyLook = 4;                 // steps whose logits one pass looks at
+static_assert(kRnntGreedyAhead < kRnntGreedyRing && (kRnntGreedyRing & (kRnntGreedyRing - 1)) == 0, "ring");
 constexpr int kRnntGreedyMaxVocab = 64;            // the argmax is one wavefront's ballot
 constexpr int kRnntGreedyEmbHalfs = 16384;         // embedding rows kept in LDS by the first layer's blocks (32 KB)
 constexpr int kRnntSeenStride = 16;                // 32-bit words between the blocks' `seen` counts
@@ -209,21 +213,22 @@ __device__ __forceinline__ void rnnt_greedy_solo(const RnntGreedyArgs& p, half_t
 
 __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const RnntGreedyArgs p)
 {
-    __shared__ __align__(16) half_t buf0[kRnntMaxVec];            // the vector a role waits for
-    __shared__ __align__(16) half_t own[kRnntMaxH];               // a layer's blocks: h of their layer; joint blocks: g
-    __shared__ __align__(16) half_t lg[kRnntGreedyMaxVocab];      // the step's logits
-    __shared__ __align__(16) half_t emb[kRnntGreedyEmbHalfs];     // first layer: the embedding rows and x0 behind them
-    __shared__ __align__(16) unsigned short mine[8];
+    typedef unsigned long long u64;
+    __shared__ __align__(16) half_t buf0[kRnntMaxVec];                              // the vector a role waits for
+    __shared__ __align__(16) half_t own[kRnntMaxH];                                 // a layer's blocks: h of their layer; joint blocks: g
+    __shared__ __align__(16) half_t lgs[2][kRnntGreedyLook][kRnntGreedyMaxVocab];   // the logits of the next steps, alternating per pass
+    __shared__ __align__(16) half_t emb[kRnntGreedyEmbHalfs];                       // first layer: the embedding rows and x0 behind them
+    __shared__ __align__(16) unsigned short mine[2][12];                            // this block's eight values, alternating per publish
+    __shared__ int missing[3][2 + kRnntGreedyLook];                                 // per pass (rotating): something of the vector / of step j is not
+                                                                                    // there yet; last: a wait has given up
     __shared__ int someone_gave_up;
     __shared__ int i_decode_alone;
+    __shared__ int min_seen_lds;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nb = gridDim.x, b = blockIdx.x;
     const int H = p.H, nhp = H >> 3, nwh = H >> 3, nwj = p.J >> 3, nwv = (p.V + 7) >> 3;
     const int n_lstm = p.L * nwh;
-    half8_t zero8;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) zero8[e] = (half_t)0.0f;
 
     // The solo decoder's arrays lie where the embedding rows lay (the team's loop is over by then).
     half_t* solo_hs = emb;
@@ -234,72 +239,173 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
         someone_gave_up = (p.alone || __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) ? 1 : 0;
         i_decode_alone = 0;
     }
+    if (tid < 3 * (2 + kRnntGreedyLook)) (&missing[0][0])[tid] = 0;
+    if (tid < 24) (&mine[0][0])[tid] = 0;
     __syncthreads();
 
     RnntGreedyState s = {0, 0, 0, -1, p.run_pred_first};
-    int n_pred = 0, step = 0;
+    int n_pred = 0, step = 0;          // runs of the prediction network and steps so far
+    unsigned int n_pass = 0, n_publish = 0, waited = 0;
+    bool dead = false;                 // a wait of this block has given up (the same in every thread)
+    unsigned long long t_first = 0ull;
 
-    // Thread t takes word t of the vector that blocks first .. first + nwords published in `set`; it lands in dst.
-    // Returns whether the block has to leave the loop (uniform).
-    auto gather = [&](int first, int nwords, int set, half_t* dst) {
-        if (tid < nwords) {
-            const unsigned long long* slot = p.hx + ((long)set * nb + first + tid) * kRnntEntryWords;
-            unsigned long long lo = kRnntEmpty, hi = kRnntEmpty;
-            unsigned int spins = 0;
-            unsigned long long t_first = 0ull;
-            bool gave_up = false;
-            while (true) {
-                load16_device_scope(slot, lo, hi);
-                if (lo != kRnntEmpty && hi != kRnntEmpty) break;
-                if (spins > 0u && (spins & 255u) == 0u) {
-                    if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
-                    if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;
-                }
-                if (spins >= p.spin_limit) {
-                    __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                    gave_up = true;
-                }
-                if (gave_up) break;
-                if (spins != 0xffffffffu) ++spins;
+    auto running = [&]() { return s.t < p.T && s.emitted < p.max_symbols; };
+    // The version of g that the current step's joint network sees: runs of the prediction network started, less one.
+    auto g_version = [&]() { return n_pred + s.run_pred - 1; };
+    auto h_tag = [](int version) { return (unsigned int)(version & 0x7fff); };
+    auto step_tag = [](int st, int version) { return (unsigned int)(((version & 0x7f) << 8) | (st & 0xff)); };
+    auto h_entry = [&](int version, int block) { return p.hx + ((long)(version & (kRnntGreedyVersions - 1)) * n_lstm + block) * kRnntEntryWords; };
+    auto hid_entry = [&](int st, int j) {
+        return p.hx + ((long)kRnntGreedyVersions * n_lstm + (long)(st & (kRnntGreedyRing - 1)) * nwj + j) * kRnntEntryWords;
+    };
+    auto lg_entry = [&](int st, int j) {
+        return p.hx + ((long)kRnntGreedyVersions * n_lstm + (long)kRnntGreedyRing * nwj + (long)(st & (kRnntGreedyRing - 1)) * nwv + j) * kRnntEntryWords;
+    };
+
+    // mine[] of this publish goes out as three 8-byte words of three values and the tag each.
+    auto publish = [&](u64* entry, unsigned int tag) {
+        rnnt_barrier();
+        if (tid < 3) {
+            const unsigned short* m = mine[n_publish & 1u] + 3 * tid;
+            const u64 w = (u64)m[0] | ((u64)m[1] << 16) | ((u64)m[2] << 32) | ((u64)tag << 48);
+            __hip_atomic_store(entry + tid, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        ++n_publish;
+    };
+    auto my_values = [&]() { return mine[n_publish & 1u]; };
+
+    // One 8-byte word: looked at once, or (blocks) polled until it carries `tag` or the wait's limits are reached, in which
+    // case the thread raises the abort words and this pass's "gave up" flag.  Returns whether the tag is there.
+    auto fetch = [&](const u64* slot, unsigned int tag, bool blocks, int* miss, u64& w) {
+        unsigned int spins = 0;
+        unsigned long long first = 0ull;
+        while (true) {
+            w = __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((unsigned int)(w >> 48) == tag) return true;
+            if (!blocks) return false;
+            bool give_up = false;
+            if (spins > 0u && (spins & 255u) == 0u) {
+                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) give_up = true;
+                if (wait_clock_expired(spins, first)) spins = 0xffffffffu;
             }
-            if (gave_up) someone_gave_up = 1;
-            typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
-            const u64x2 v = {lo, hi};
-            *reinterpret_cast<u64x2*>(&dst[8 * tid]) = v;
+            if (spins >= p.spin_limit) {
+                __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                give_up = true;
+            }
+            if (give_up) {
+                miss[1 + kRnntGreedyLook] = 1;
+                someone_gave_up = 1;
+                return false;
+            }
+            if (spins != 0xffffffffu) ++spins;
+        }
+    };
+    auto unpack = [&](u64 w, half_t* dst, int prod, int part) {
+        unsigned short* d = reinterpret_cast<unsigned short*>(dst) + 8 * prod + 3 * part;
+        d[0] = (unsigned short)w;
+        d[1] = (unsigned short)(w >> 16);
+        if (part < 2) d[2] = (unsigned short)(w >> 32);
+    };
+    // One round over everything this block waits for: the 8-byte words of a vector (n_vec producers from `vec`, tagged
+    // vec_tag, values to vec_dst) by the first six wavefronts, and with want_steps the logits of the steps step .. step + 3
+    // under the current version by the last two.  What the block cannot go on without is polled until it is there
+    // (vec_blocks; step_blocks: the logits of `step`), the rest is looked at once.  Returns bit 0: the vector is complete;
+    // bit 1 + j: the logits of step + j are.
+    auto pass = [&](const u64* vec, int n_vec, unsigned int vec_tag, half_t* vec_dst, bool vec_blocks, bool want_steps, bool step_blocks) -> int {
+        int* miss = missing[n_pass % 3u];
+        u64 w;
+        if (tid < 384) {
+            for (int i = tid; i < 3 * n_vec; i += 384) {
+                const int prod = i / 3, part = i - 3 * prod;
+                if (fetch(vec + (long)prod * kRnntEntryWords + part, vec_tag, vec_blocks, miss, w))
+                    unpack(w, vec_dst, prod, part);
+                else
+                    miss[0] = 1;
+            }
+        } else if (want_steps) {
+            const int j = (tid - 384) >> 5, i = (tid - 384) & 31;
+            if (i < 3 * nwv) {
+                const int prod = i / 3, part = i - 3 * prod;
+                if (fetch(lg_entry(step + j, prod) + part, step_tag(step + j, g_version()), step_blocks && j == 0, miss, w))
+                    unpack(w, lgs[n_pass & 1u][j], prod, part);
+                else
+                    miss[1 + j] = 1;
+            }
         }
         rnnt_barrier();
-        return someone_gave_up != 0;
+        int r = (n_vec > 0 && miss[0] == 0) ? 1 : 0;
+        if (want_steps) {
+#pragma unroll
+            for (int j = 0; j < kRnntGreedyLook; ++j)
+                if (miss[1 + j] == 0) r |= 2 << j;
+        }
+        if (miss[1 + kRnntGreedyLook] != 0) dead = true;
+        // the flags of the pass after the next are cleared now: their last readers passed this barrier, their next
+        // writers come after the next one
+        if (tid < 2 + kRnntGreedyLook) missing[(n_pass + 2u) % 3u][tid] = 0;
+        ++n_pass;
+        return r;
     };
-    // This block's entry of the set after `round`'s becomes empty (it holds round - 3).
-    auto empty_next = [&](int round) {
-        if (tid < 2)
-            __hip_atomic_store(p.hx + ((long)((round + 1) & 3) * nb + b) * kRnntEntryWords + tid, kRnntEmpty, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-    };
-    // mine[] goes out as this block's word of `round`.  The store that emptied this entry's successor, issued a round's work
-    // ago, is acknowledged first: whoever sees this word and moves on to the next set finds it emptied.
-    auto publish = [&](int round) {
-        rnnt_barrier();
+    // After a pass that brought nothing: counts, and gives up when the limits are reached.  Everybody learns of it behind the
+    // next pass's barrier, through that pass's flags (a word that thread 0 wrote now could be read by some threads of this
+    // round and not by others).
+    auto nothing_came = [&]() {
         if (tid == 0) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            const unsigned long long* src = reinterpret_cast<const unsigned long long*>(mine);
-            store16_device_scope(p.hx + ((long)(round & 3) * nb + b) * kRnntEntryWords, src[0], src[1]);
+            bool give_up = false;
+            if (waited > 0u && (waited & 255u) == 0u) {
+                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) give_up = true;
+                if (wait_clock_expired(waited, t_first)) waited = 0xffffffffu;
+            }
+            if (waited >= p.spin_limit) {
+                __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                give_up = true;
+            }
+            if (give_up) {
+                someone_gave_up = 1;
+                missing[n_pass % 3u][1 + kRnntGreedyLook] = 1;
+            }
+            if (waited != 0xffffffffu) ++waited;
         }
     };
-    // The end of a step for every role: the logits arrive, everybody takes the same decision.  Returns false when the block
-    // has to leave the loop.
-    auto decide = [&]() {
-        if (gather(n_lstm + nwj, nwv, step & 3, lg)) return false;
-        if (tid == 0) __hip_atomic_store(p.seen + (long)kRnntSeenStride * b, (unsigned int)(step + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int k = rnnt_argmax(lg, p.V, lane);
-        const int at = s.emitted;
-        n_pred += s.run_pred;
-        ++step;
-        if (rnnt_greedy_advance(s, k, p.blank, p.max_per_frame) && b == 0 && tid == 0) p.symbols[at] = k;
+    auto something_came = [&]() {
+        if (tid == 0) waited = 0u;
+    };
+    // Takes the decisions whose logits a pass found (bits 1.. of mask), in order, up to and including the first that emits a
+    // symbol (what lies behind it was computed for a g that is no longer the current one).  Returns how many.
+    auto take_decisions = [&](int mask) {
+        int taken = 0;
+#pragma unroll
+        for (int j = 0; j < kRnntGreedyLook; ++j) {
+            if (!(mask & (2 << j)) || !running()) break;
+            const int k = rnnt_argmax(lgs[(n_pass - 1u) & 1u][j], p.V, lane);
+            const int at = s.emitted;
+            n_pred += s.run_pred;
+            ++step;
+            ++taken;
+            if (rnnt_greedy_advance(s, k, p.blank, p.max_per_frame)) {
+                if (b == 0 && tid == 0) p.symbols[at] = k;
+                break;
+            }
+        }
+        if (taken > 0 && tid == 0)
+            __hip_atomic_store(p.seen + (long)kRnntSeenStride * b, (unsigned int)step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return taken;
+    };
+    // Waits for a vector.  Returns false when the block has to leave the loop.
+    auto wait_for_vector = [&](const u64* vec, int n_vec, unsigned int tag, half_t* dst) {
+        pass(vec, n_vec, tag, dst, true, false, false);
+        return !dead;
+    };
+    // Waits until the decision of `step` can be taken, and takes those behind it too if their logits are there already.
+    // Returns false when the block has to leave the loop.
+    auto wait_for_decisions = [&]() {
+        const int r = pass(nullptr, 0, 0u, nullptr, false, true, true);
+        if (dead) return false;
+        take_decisions(r);
         return true;
     };
-    auto running = [&]() { return s.t < p.T && s.emitted < p.max_symbols; };
 
     if (someone_gave_up == 0 && b < n_lstm) {
         // ---- a layer of the prediction network: unit u, gate rows u, H + u, 2H + u, 3H + u ----
@@ -329,16 +435,15 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
         half_t c_half = p.c0 ? p.c0[(long)l * H + u] : (half_t)0.0f;
         half_t h_last = p.h0 ? p.h0[(long)l * H + u] : (half_t)0.0f;
         for (int i = tid; i < H; i += kRnntThreads) own[i] = p.h0 ? p.h0[(long)l * H + i] : (half_t)0.0f;
-        if (l == 0) {
+        if (l == 0 && p.emb_in_lds) {
             // the rows the first layer will be asked for: embedding[0 .. emb_rows) and, behind them, x0
-            if (p.emb_in_lds) {
-                const half8_t* e8 = reinterpret_cast<const half8_t*>(p.embedding);
-                half8_t* d8 = reinterpret_cast<half8_t*>(emb);
-                const int n8 = p.emb_rows * nxp;
-                for (int i = tid; i < n8; i += kRnntThreads) d8[i] = e8[i];
-                const half8_t* x8 = reinterpret_cast<const half8_t*>(p.x0);
+            const half8_t* e8 = reinterpret_cast<const half8_t*>(p.embedding);
+            half8_t* d8 = reinterpret_cast<half8_t*>(emb);
+            const int n8 = p.emb_rows * nxp;
+            for (int i = tid; i < n8; i += kRnntThreads) d8[i] = e8[i];
+            const half8_t* x8 = reinterpret_cast<const half8_t*>(p.x0);
+            if (x8)  // (null when the first step does not run the prediction network: never asked for then)
                 for (int i = tid; i < nxp; i += kRnntThreads) d8[n8 + i] = x8[i];
-            }
         }
         __syncthreads();
         // W_hh . h of the layer, summed as soon as h is known
@@ -356,16 +461,15 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
         sum_hh();
         bool ok = true;
         while (ok && running()) {
-            rnnt_barrier();
             if (s.run_pred) {
-                empty_next(n_pred);
+                const int version = n_pred;
                 const half8_t* in;
                 if (l == 0) {
                     const int row = s.label < 0 ? p.emb_rows : s.label;
                     in = p.emb_in_lds ? reinterpret_cast<const half8_t*>(emb) + (long)row * nxp
                                       : reinterpret_cast<const half8_t*>(s.label < 0 ? p.x0 : p.embedding + (long)s.label * ly.in_w);
                 } else {
-                    if (gather((l - 1) * nwh, nwh, n_pred & 3, buf0)) {
+                    if (!wait_for_vector(h_entry(version, (l - 1) * nwh), nwh, h_tag(version), buf0)) {
                         ok = false;
                         break;
                     }
@@ -385,24 +489,25 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
                 c_half = rnnt_round(c_new);
                 const unsigned short bits = rnnt_bits((float)h_new);
                 h_last = __builtin_bit_cast(half_t, bits);
-                if (lane == 0) mine[wave] = bits;
-                publish(n_pred);
+                if (lane == 0) my_values()[wave] = bits;
+                publish(h_entry(version, b), h_tag(version));
                 // h of this layer, for W_hh at the next symbol
-                if (gather(l * nwh, nwh, n_pred & 3, own)) {
+                if (!wait_for_vector(h_entry(version, l * nwh), nwh, h_tag(version), own)) {
                     ok = false;
                     break;
                 }
                 sum_hh();
             }
-            ok = decide();
+            ok = wait_for_decisions();
         }
         if (ok && lane == 0) {
             if (p.hn) p.hn[(long)l * H + u] = h_last;
             if (p.cn) p.cn[(long)l * H + u] = c_half;
         }
     } else if (someone_gave_up == 0 && b < n_lstm + nwj) {
-        // ---- the joint network's first layer: row r of W1 over cat(f, g) ----
-        const int r = 8 * (b - n_lstm) + wave;
+        // ---- the joint network's first layer: row r of W1 over cat(f, g), for the current step and, while nothing else
+        // is to do, for the steps behind it should they all be blanks ----
+        const int jb = b - n_lstm, r = 8 * jb + wave;
         const int nfp = p.F >> 3;
         const half8_t* row = reinterpret_cast<const half8_t*>(p.w1 + (long)r * (p.F + H));
         half8_t wf[kRnntFC], wg[kRnntHC];
@@ -418,10 +523,11 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
         }
         const float bias = (lane == 0 && p.b1) ? (float)p.b1[r] : 0.0f;
         for (int i = tid; i < H; i += kRnntThreads) own[i] = p.h0 ? p.h0[(long)(p.L - 1) * H + i] : (half_t)0.0f;  // g before the first run
-        // this lane's part of the row's sum over frame `frame` (zero past the last frame: never used)
+        __syncthreads();
+        // this lane's part of the row's sum over a frame (nothing is read for a frame the utterance does not have)
         auto sum_f = [&](int frame) {
             float a = 0.0f;
-            if (frame < p.T) {
+            if (frame >= 0 && frame < p.T) {
                 const half8_t* f8 = reinterpret_cast<const half8_t*>(p.enc + (long)frame * p.F);
 #pragma unroll
                 for (int k = 0; k < kRnntFC; ++k)
@@ -429,37 +535,57 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
             }
             return a;
         };
-        float af_cur = sum_f(0), af_nxt = sum_f(1);
-        int t_cur = 0;
+        // The sums over the frames around the current one are kept (per thread, in the LDS that the first layer's blocks
+        // use for the embedding rows): frames [af_lo, af_hi) in slots frame mod 16.  A frame is summed once, ahead of its
+        // turn, whatever the number of symbols it then emits.
+        float* af_ring = reinterpret_cast<float*>(emb) + tid;
+        static_assert(kRnntGreedyRing * kRnntThreads * sizeof(float) <= kRnntGreedyEmbHalfs * sizeof(half_t), "the ring of frame sums fits");
+        int af_lo = 0, af_hi = 0;
+        auto frame_sum = [&](int frame) {
+            if (frame >= af_lo && frame < af_hi) return af_ring[(frame & (kRnntGreedyRing - 1)) * kRnntThreads];
+            const float a = sum_f(frame);
+            if (frame != af_hi) af_lo = frame;
+            af_hi = frame + 1;
+            if (af_hi - af_lo > kRnntGreedyRing) af_lo = af_hi - kRnntGreedyRing;
+            af_ring[(frame & (kRnntGreedyRing - 1)) * kRnntThreads] = a;
+            return a;
+        };
+        int have_g = -1;          // the version of g in `own`
+        int pub = 0;              // the next step to publish a hidden vector for
+        frame_sum(0);
         bool ok = true;
         while (ok && running()) {
-            rnnt_barrier();
-            empty_next(step);
-            if (s.t != t_cur) af_cur = af_nxt;
-            if (s.run_pred) {
-                if (gather((p.L - 1) * nwh, nwh, n_pred & 3, own)) {
+            const int version = g_version();
+            if (version != have_g) {
+                if (!wait_for_vector(h_entry(version, (p.L - 1) * nwh), nwh, h_tag(version), own)) {
                     ok = false;
                     break;
                 }
+                have_g = version;
+                pub = step;
             }
-            const half8_t* gv = reinterpret_cast<const half8_t*>(own);
-            float a = af_cur;
+            if (pub < step) pub = step;
+            // the current step first, then up to kRnntGreedyAhead behind it, two per round
+            for (int i = 0; i < 2; ++i) {
+                const int frame = s.t + (pub - step);
+                if (frame >= p.T || pub > step + kRnntGreedyAhead) break;
+                const half8_t* gv = reinterpret_cast<const half8_t*>(own);
+                float a = frame_sum(frame);
 #pragma unroll
-            for (int k = 0; k < kRnntHC; ++k)
-                if (lane + 64 * k < nhp) a = dot8(wg[k], gv[lane + 64 * k], a);
-            a = rnnt_sum(a);
-            if (lane == 0) mine[wave] = rnnt_bits(fmaxf(a + bias, 0.0f));
-            publish(step);
-            // while the symbol blocks work: the row's sum over the frame after this one
-            if (s.t != t_cur) {
-                t_cur = s.t;
-                af_nxt = sum_f(t_cur + 1);
+                for (int k = 0; k < kRnntHC; ++k)
+                    if (lane + 64 * k < nhp) a = dot8(wg[k], gv[lane + 64 * k], a);
+                a = rnnt_sum(a);
+                if (lane == 0) my_values()[wave] = rnnt_bits(fmaxf(a + bias, 0.0f));
+                publish(hid_entry(pub, jb), step_tag(pub, version));
+                ++pub;
+                // the frame that comes next, while the symbol blocks work
+                if (frame + 1 < p.T) frame_sum(frame + 1);
             }
-            ok = decide();
+            ok = wait_for_decisions();
         }
     } else if (someone_gave_up == 0) {
-        // ---- the joint network's second layer: row v of W2 ----
-        const int v = 8 * (b - n_lstm - nwj) + wave;
+        // ---- the joint network's second layer: row v of W2, for every hidden vector that arrives ----
+        const int vb = b - n_lstm - nwj, v = 8 * vb + wave;
         const int njp = p.J >> 3;
         const half8_t* row = reinterpret_cast<const half8_t*>(p.w2 + (long)min(v, p.V - 1) * p.J);
         half8_t wv[kRnntJC];
@@ -469,53 +595,52 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
             wv[k] = row[min(lane + 64 * k, njp - 1)];
         }
         const float bias = (lane == 0 && p.b2 && v < p.V) ? (float)p.b2[v] : 0.0f;
+        int pub = 0;              // the next step to publish logits for
+        int have_version = g_version();
+        int min_seen = 0;         // no block has taken in fewer decisions than this
         bool ok = true;
         while (ok && running()) {
-            rnnt_barrier();
-            empty_next(step);
-            // how far everybody has come (asked for now, looked at before this step's logits go out)
-            unsigned int sv = 0u;
-            if (tid < nb) sv = __hip_atomic_load(p.seen + (long)kRnntSeenStride * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (gather(n_lstm, nwj, step & 3, buf0)) {
+            const int version = g_version();
+            if (version != have_version) {
+                have_version = version;
+                pub = step;
+            }
+            if (pub < step) pub = step;
+            const int frame = s.t + (pub - step);
+            bool want = frame < p.T && pub <= step + kRnntGreedyAhead;
+            if (want && pub - kRnntGreedyRing >= min_seen) {
+                // The entry for step `pub` still holds step pub - ring: has everybody taken that decision in?
+                if (tid == 0) min_seen_lds = 0x7fffffff;
+                rnnt_barrier();
+                if (tid < nb)
+                    atomicMin(&min_seen_lds, (int)__hip_atomic_load(p.seen + (long)kRnntSeenStride * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                rnnt_barrier();
+                min_seen = min_seen_lds;
+                want = pub - kRnntGreedyRing < min_seen;
+            }
+            // the hidden vector of `step` itself is what everybody waits for (no decision can come before it): polled; one
+            // of a later step is looked for once per round, between looks at the decisions
+            const int r = pass(hid_entry(pub, 0), want ? nwj : 0, step_tag(pub, version), buf0, pub == step, true, false);
+            if (dead) {
                 ok = false;
                 break;
             }
-            const half8_t* in = reinterpret_cast<const half8_t*>(buf0);
-            float a = 0.0f;
+            if (r & 1) {
+                const half8_t* in = reinterpret_cast<const half8_t*>(buf0);
+                float a = 0.0f;
 #pragma unroll
-            for (int k = 0; k < kRnntJC; ++k)
-                if (lane + 64 * k < njp) a = dot8(wv[k], in[lane + 64 * k], a);
-            a = rnnt_sum(a);
-            if (lane == 0) mine[wave] = v < p.V ? rnnt_bits(a + bias) : (unsigned short)0xfc00u;  // (-inf past the last symbol)
-            if (tid < nb) {
-                // nobody is still to take in the decision of step - 2 (whose words the next step's start empties)
-                unsigned int spins = 0;
-                unsigned long long t_first = 0ull;
-                while ((int)sv < step - 1) {
-                    bool gave_up = false;
-                    if (spins > 0u && (spins & 255u) == 0u) {
-                        if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
-                        if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;
-                    }
-                    if (spins >= p.spin_limit) {
-                        __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                        gave_up = true;
-                    }
-                    if (gave_up) {
-                        someone_gave_up = 1;
-                        break;
-                    }
-                    if (spins != 0xffffffffu) ++spins;
-                    sv = __hip_atomic_load(p.seen + (long)kRnntSeenStride * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
+                for (int k = 0; k < kRnntJC; ++k)
+                    if (lane + 64 * k < njp) a = dot8(wv[k], in[lane + 64 * k], a);
+                a = rnnt_sum(a);
+                if (lane == 0) my_values()[wave] = v < p.V ? rnnt_bits(a + bias) : (unsigned short)0xfc00u;  // (-inf past the last symbol)
+                publish(lg_entry(pub, vb), step_tag(pub, version));
+                ++pub;
             }
-            publish(step);  // (its barrier also carries someone_gave_up to everybody)
-            if (someone_gave_up != 0) {
-                ok = false;
-                break;
-            }
-            ok = decide();
+            const int taken = take_decisions(r);
+            if ((r & 1) || taken > 0)
+                something_came();
+            else
+                nothing_came();
         }
     }
 
@@ -524,7 +649,7 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
     if (someone_gave_up != 0) {
         if (tid == 0) i_decode_alone = (p.alone || atomicCAS(p.solo_owner, 0u, 1u) == 0u) ? 1 : 0;
         __syncthreads();
-        if (i_decode_alone) rnnt_greedy_solo(p, solo_hs, solo_cs, buf0, lg);
+        if (i_decode_alone) rnnt_greedy_solo(p, solo_hs, solo_cs, buf0, lgs[0][0]);
         return;
     }
     if (b == 0 && tid == 0) {
