@@ -18,14 +18,27 @@
 //   * the argmax is taken by every workgroup for itself from the logits that the symbol blocks publish, so the decision
 //     travels with the hand-over that ends the step and every workgroup keeps the same loop state (t, symbols so far, ..);
 //   * a layer's blocks also collect their own layer's h (what W_hh multiplies at the next symbol) and sum W_hh . h right
-//     then, long before the next symbol is known; the joint blocks sum their rows over the NEXT frame while they wait.
+//     then, long before the next symbol is known;
+//   * most steps of a real utterance are blanks, after which only the frame changes: the joint blocks do not wait for the
+//     decision but publish the hidden vectors of the next steps as well, up to eight ahead, as if every decision in
+//     between were a blank (the frames' columns are asked for a round earlier and their sums kept), and the symbol blocks
+//     turn every hidden vector that arrives into logits, two per round.  When a symbol is emitted, g gets a new version
+//     and what was computed ahead under the old one is simply never looked at.  A run of blanks then costs what the symbol
+//     blocks' round costs, not two hand-overs per step.
 //
-// Exchange: 16-byte words in 128-byte entries as in the step kernel, in FOUR sets.  A producer's n-th word (n counts the
-// prediction network's runs for the layers' blocks, steps for the joint and symbol blocks) goes to set n mod 4; at the start
-// of round n it empties its entry of set (n + 1) mod 4, which holds round n - 3.  Everybody who reads that word has long
-// done so: readers on the chain of a round cannot fall a round behind, and for the one exception, blocks of the prediction
-// network, which nobody waits for in steps after a blank, the symbol blocks look at a count that every block keeps of the
-// decisions it has taken in (`seen`) and do not publish step s before all have taken in step s - 2.
+// Exchange: 8-byte words of three fp16 values and a 16-bit tag, three words per producing block in a 128-byte entry of its
+// own, written and read with device-scope accesses.  The tag says what the word belongs to: h of a layer carries the
+// version of g (the count of the prediction network's runs), hidden vectors and logits carry the step and the version they
+// were computed under; a word with another tag is "not there yet", so nothing is ever cleared and a stale word cannot be
+// taken for a fresh one.  h lives in four sets by version, hidden vectors and logits in rings of sixteen by step.  A
+// producer may overwrite what is sixteen steps old: for the joint blocks' entries that follows from the order of things
+// (they run at most eight steps ahead of decisions that the symbol blocks have already published); the symbol blocks, whom
+// a slow reader could fall sixteen steps behind (nobody waits for the layers' blocks during a run of blanks), look at a
+// count that every block keeps of the decisions it has taken in (`seen`) before they reuse an entry.
+//
+// Waiting: a block looks at everything it waits for in one round ("pass"): the words of a vector by the first six
+// wavefronts, the logits of the next four steps by the last two.  What the block cannot go on without is polled until it
+// is there, the rest is looked at once; one barrier ends the round, and a pass can take several decisions at once.
 //
 // Sums run in the order of the step kernel, c is rounded to fp16 after every run of the prediction network as it is when
 // the state travels between launches: symbols and final state equal, bit for bit, those of a loop of pimhip_rnnt_step
@@ -103,34 +116,46 @@ __device__ __forceinline__ bool rnnt_greedy_advance(RnntGreedyState& s, int k, i
     return true;
 }
 
-__device__ __forceinline__ float rnnt_max(float v)
+template <int CTRL>
+__device__ __forceinline__ unsigned int rnnt_dpp_u32(unsigned int v)
 {
-    v = fmaxf(v, rnnt_dpp<kDppQuadXor1>(v));
-    v = fmaxf(v, rnnt_dpp<kDppQuadXor2>(v));
-    v = fmaxf(v, rnnt_dpp<0x124>(v));
-    v = fmaxf(v, rnnt_dpp<0x128>(v));
+    return (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+
+// The maximum over the 64 lanes; every lane returns it.
+__device__ __forceinline__ unsigned int rnnt_max_u32(unsigned int v)
+{
+    v = max(v, rnnt_dpp_u32<kDppQuadXor1>(v));
+    v = max(v, rnnt_dpp_u32<kDppQuadXor2>(v));
+    v = max(v, rnnt_dpp_u32<0x124>(v));
+    v = max(v, rnnt_dpp_u32<0x128>(v));
     {
-        float a = v, b = v;
+        unsigned int a = v, b = v;
         asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-        v = fmaxf(a, b);
+        v = max(a, b);
     }
     {
-        float a = v, b = v;
+        unsigned int a = v, b = v;
         asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-        v = fmaxf(a, b);
+        v = max(a, b);
     }
     return v;
 }
 
-// torch.argmax over V <= 64 fp16 values: the first maximum, a NaN counting as the largest.  Every lane returns it.
+// torch.argmax over V <= 64 fp16 values: the first maximum, a NaN counting as the largest.  Every lane returns it.  One
+// integer maximum over keys: the value's bits made monotonic (-0 as +0, a NaN above everything) in front of the lane counted
+// from the top, so that of equal values the first wins.
 __device__ __forceinline__ int rnnt_argmax(const half_t* lg, int V, int lane)
 {
-    const bool mine = lane < V;
-    const float v = mine ? (float)lg[lane] : -__builtin_inff();
-    const unsigned long long nan_mask = __ballot(mine && v != v);
-    if (nan_mask) return __builtin_ctzll(nan_mask);
-    const float m = rnnt_max(v);
-    return __builtin_ctzll(__ballot(mine && v == m));
+    unsigned int key = 0u;
+    if (lane < V) {
+        unsigned int bits = __builtin_bit_cast(unsigned short, lg[lane]);
+        if (bits == 0x8000u) bits = 0u;
+        unsigned int order = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
+        if ((bits & 0x7fffu) > 0x7c00u) order = 0xffffu;
+        key = (order << 8) | (unsigned int)(255 - lane);
+    }
+    return 255 - (int)(rnnt_max_u32(key) & 0xffu);
 }
 
 // The whole loop by one workgroup.  LDS: hs [L * H] (h of every layer), cs [L * H], tmp [max(H, J)], lg [64].
@@ -219,8 +244,8 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
     __shared__ __align__(16) half_t lgs[2][kRnntGreedyLook][kRnntGreedyMaxVocab];   // the logits of the next steps, alternating per pass
     __shared__ __align__(16) half_t emb[kRnntGreedyEmbHalfs];                       // first layer: the embedding rows and x0 behind them
     __shared__ __align__(16) unsigned short mine[2][12];                            // this block's eight values, alternating per publish
-    __shared__ int missing[3][2 + kRnntGreedyLook];                                 // per pass (rotating): something of the vector / of step j is not
-                                                                                    // there yet; last: a wait has given up
+    __shared__ int missing[3][3 + kRnntGreedyLook];                                 // per pass (rotating): something of the vector / of step j is not
+                                                                                    // there yet; a wait has given up; something of a second vector is not there
     __shared__ int someone_gave_up;
     __shared__ int i_decode_alone;
     __shared__ int min_seen_lds;
@@ -239,7 +264,7 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
         someone_gave_up = (p.alone || __hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) ? 1 : 0;
         i_decode_alone = 0;
     }
-    if (tid < 3 * (2 + kRnntGreedyLook)) (&missing[0][0])[tid] = 0;
+    if (tid < 3 * (3 + kRnntGreedyLook)) (&missing[0][0])[tid] = 0;
     if (tid < 24) (&mine[0][0])[tid] = 0;
     __syncthreads();
 
@@ -312,16 +337,27 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
     // under the current version by the last two.  What the block cannot go on without is polled until it is there
     // (vec_blocks; step_blocks: the logits of `step`), the rest is looked at once.  Returns bit 0: the vector is complete;
     // bit 1 + j: the logits of step + j are.
-    auto pass = [&](const u64* vec, int n_vec, unsigned int vec_tag, half_t* vec_dst, bool vec_blocks, bool want_steps, bool step_blocks) -> int {
+    // A second vector (vec2, looked at once) is taken along where the first leaves threads free; bit 30 says it is complete.
+    auto pass = [&](const u64* vec, int n_vec, unsigned int vec_tag, half_t* vec_dst, bool vec_blocks, bool want_steps, bool step_blocks,
+                    const u64* vec2 = nullptr, int n_vec2 = 0, unsigned int vec2_tag = 0u, half_t* vec2_dst = nullptr) -> int {
         int* miss = missing[n_pass % 3u];
         u64 w;
         if (tid < 384) {
-            for (int i = tid; i < 3 * n_vec; i += 384) {
-                const int prod = i / 3, part = i - 3 * prod;
-                if (fetch(vec + (long)prod * kRnntEntryWords + part, vec_tag, vec_blocks, miss, w))
-                    unpack(w, vec_dst, prod, part);
-                else
-                    miss[0] = 1;
+            for (int i = tid; i < 3 * (n_vec + n_vec2); i += 384) {
+                const bool second = i >= 3 * n_vec;
+                const int i2 = second ? i - 3 * n_vec : i;
+                const int prod = i2 / 3, part = i2 - 3 * prod;
+                if (!second) {
+                    if (fetch(vec + (long)prod * kRnntEntryWords + part, vec_tag, vec_blocks, miss, w))
+                        unpack(w, vec_dst, prod, part);
+                    else
+                        miss[0] = 1;
+                } else {
+                    if (fetch(vec2 + (long)prod * kRnntEntryWords + part, vec2_tag, false, miss, w))
+                        unpack(w, vec2_dst, prod, part);
+                    else
+                        miss[2 + kRnntGreedyLook] = 1;
+                }
             }
         } else if (want_steps) {
             const int j = (tid - 384) >> 5, i = (tid - 384) & 31;
@@ -340,10 +376,11 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
             for (int j = 0; j < kRnntGreedyLook; ++j)
                 if (miss[1 + j] == 0) r |= 2 << j;
         }
+        if (n_vec2 > 0 && miss[2 + kRnntGreedyLook] == 0) r |= 1 << 30;
         if (miss[1 + kRnntGreedyLook] != 0) dead = true;
         // the flags of the pass after the next are cleared now: their last readers passed this barrier, their next
         // writers come after the next one
-        if (tid < 2 + kRnntGreedyLook) missing[(n_pass + 2u) % 3u][tid] = 0;
+        if (tid < 3 + kRnntGreedyLook) missing[(n_pass + 2u) % 3u][tid] = 0;
         ++n_pass;
         return r;
     };
@@ -541,13 +578,16 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
         float* af_ring = reinterpret_cast<float*>(emb) + tid;
         static_assert(kRnntGreedyRing * kRnntThreads * sizeof(float) <= kRnntGreedyEmbHalfs * sizeof(half_t), "the ring of frame sums fits");
         int af_lo = 0, af_hi = 0;
-        auto frame_sum = [&](int frame) {
-            if (frame >= af_lo && frame < af_hi) return af_ring[(frame & (kRnntGreedyRing - 1)) * kRnntThreads];
-            const float a = sum_f(frame);
+        auto frame_keep = [&](int frame, float a) {
             if (frame != af_hi) af_lo = frame;
             af_hi = frame + 1;
             if (af_hi - af_lo > kRnntGreedyRing) af_lo = af_hi - kRnntGreedyRing;
             af_ring[(frame & (kRnntGreedyRing - 1)) * kRnntThreads] = a;
+        };
+        auto frame_sum = [&](int frame) {
+            if (frame >= af_lo && frame < af_hi) return af_ring[(frame & (kRnntGreedyRing - 1)) * kRnntThreads];
+            const float a = sum_f(frame);
+            frame_keep(frame, a);
             return a;
         };
         int have_g = -1;          // the version of g in `own`
@@ -565,8 +605,10 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
                 pub = step;
             }
             if (pub < step) pub = step;
-            // the current step first, then up to kRnntGreedyAhead behind it, two per round
-            for (int i = 0; i < 2; ++i) {
+            // the current step first, then up to kRnntGreedyAhead behind it: two per round while symbols come (the next g is
+            // what matters then), more in a run of blanks, where running ahead is all there is to do
+            const int per_round = s.run_pred ? 2 : 5;
+            for (int i = 0; i < per_round; ++i) {
                 const int frame = s.t + (pub - step);
                 if (frame >= p.T || pub > step + kRnntGreedyAhead) break;
                 const half8_t* gv = reinterpret_cast<const half8_t*>(own);
@@ -578,10 +620,34 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
                 if (lane == 0) my_values()[wave] = rnnt_bits(fmaxf(a + bias, 0.0f));
                 publish(hid_entry(pub, jb), step_tag(pub, version));
                 ++pub;
-                // the frame that comes next, while the symbol blocks work
-                if (frame + 1 < p.T) frame_sum(frame + 1);
+            }
+            // The next frames the ring does not hold yet are asked for now and summed behind the wait for the decisions (their
+            // columns travel while the symbol blocks work): up to four a round, as many as a round can publish.
+            constexpr int kAsk = 4;
+            static_assert(kRnntGreedyAhead + 1 + kAsk <= kRnntGreedyRing, "the ring holds what is asked for ahead");
+            const int f_first = af_hi;
+            int n_ask = 0;
+            half8_t col[kAsk][kRnntFC];
+#pragma unroll
+            for (int q = 0; q < kAsk; ++q) {
+                const int f = f_first + q;
+                const bool ask = f < p.T && f <= s.t + kRnntGreedyAhead + kAsk;
+                if (ask) n_ask = q + 1;
+#pragma unroll
+                for (int k = 0; k < kRnntFC; ++k)
+                    col[q][k] = (ask && lane + 64 * k < nfp) ? reinterpret_cast<const half8_t*>(p.enc + (long)f * p.F)[lane + 64 * k] : wf[k];
             }
             ok = wait_for_decisions();
+#pragma unroll
+            for (int q = 0; q < kAsk; ++q) {
+                if (q < n_ask) {
+                    float a = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < kRnntFC; ++k)
+                        if (lane + 64 * k < nfp) a = dot8(wf[k], col[q][k], a);
+                    frame_keep(f_first + q, a);
+                }
+            }
         }
     } else if (someone_gave_up == 0) {
         // ---- the joint network's second layer: row v of W2, for every hidden vector that arrives ----
@@ -620,21 +686,42 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
             }
             // the hidden vector of `step` itself is what everybody waits for (no decision can come before it): polled; one
             // of a later step is looked for once per round, between looks at the decisions
-            const int r = pass(hid_entry(pub, 0), want ? nwj : 0, step_tag(pub, version), buf0, pub == step, true, false);
+            // and the one behind it is taken along (to the LDS that the first layer's blocks use for the embedding rows)
+            const bool want2 = want && frame + 1 < p.T && pub + 1 <= step + kRnntGreedyAhead && pub + 1 - kRnntGreedyRing < min_seen;
+            const int r = pass(hid_entry(pub, 0), want ? nwj : 0, step_tag(pub, version), buf0, pub == step, true, false,
+                               hid_entry(pub + 1, 0), want2 ? nwj : 0, step_tag(pub + 1, version), emb);
             if (dead) {
                 ok = false;
                 break;
             }
             if (r & 1) {
-                const half8_t* in = reinterpret_cast<const half8_t*>(buf0);
-                float a = 0.0f;
+                const bool two = (r & (1 << 30)) != 0;
+                const half8_t* in0 = reinterpret_cast<const half8_t*>(buf0);
+                const half8_t* in1 = reinterpret_cast<const half8_t*>(emb);
+                float a0 = 0.0f, a1 = 0.0f;
 #pragma unroll
-                for (int k = 0; k < kRnntJC; ++k)
-                    if (lane + 64 * k < njp) a = dot8(wv[k], in[lane + 64 * k], a);
-                a = rnnt_sum(a);
-                if (lane == 0) my_values()[wave] = v < p.V ? rnnt_bits(a + bias) : (unsigned short)0xfc00u;  // (-inf past the last symbol)
-                publish(lg_entry(pub, vb), step_tag(pub, version));
-                ++pub;
+                for (int k = 0; k < kRnntJC; ++k) {
+                    if (lane + 64 * k < njp) {
+                        a0 = dot8(wv[k], in0[lane + 64 * k], a0);
+                        if (two) a1 = dot8(wv[k], in1[lane + 64 * k], a1);
+                    }
+                }
+                a0 = rnnt_sum(a0);
+                if (two) a1 = rnnt_sum(a1);
+                if (lane == 0) {
+                    mine[n_publish & 1u][wave] = v < p.V ? rnnt_bits(a0 + bias) : (unsigned short)0xfc00u;   // (-inf past the last symbol)
+                    if (two) mine[(n_publish + 1u) & 1u][wave] = v < p.V ? rnnt_bits(a1 + bias) : (unsigned short)0xfc00u;
+                }
+                // both go out behind one barrier, from two wavefronts
+                rnnt_barrier();
+                const int which = tid >> 6, part = tid & 63;
+                if (part < 3 && which < (two ? 2 : 1)) {
+                    const unsigned short* m = mine[(n_publish + which) & 1u] + 3 * part;
+                    const u64 w = (u64)m[0] | ((u64)m[1] << 16) | ((u64)m[2] << 32) | ((u64)step_tag(pub + which, version) << 48);
+                    __hip_atomic_store(lg_entry(pub + which, vb) + part, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                n_publish += two ? 2u : 1u;
+                pub += two ? 2 : 1;
             }
             const int taken = take_decisions(r);
             if ((r & 1) || taken > 0)

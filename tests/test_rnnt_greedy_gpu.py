@@ -74,6 +74,7 @@ CASES = [
     (2, 320, 320, 1024, 512, 29, 40, 28, 30, None, 0.3, True),       # mostly symbols: frames end at the per-frame limit
     (2, 320, 320, 1024, 512, 29, 50, 28, 2, 37, 0.4, True),          # ends at max_symbols
     (1, 64, 32, 128, 64, 5, 12, 0, 3, None, 0.3, True),
+    (2, 136, 344, 1000, 504, 64, 30, 1, 4, None, 0.3, True),         # widths that are no multiples of 64, the most symbols
     (3, 72, 136, 200, 1024, 8, 40, 3, 4, None, 0.2, False),
     (4, 1024, 256, 2048, 512, 64, 25, 63, 5, None, 0.5, True),       # widest x and f, embedding rows read from memory
     (1, 64, 32, 128, 64, 5, 0, 0, 3, None, 0.3, True),               # no frames
