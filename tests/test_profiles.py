@@ -72,5 +72,5 @@ def test_profile_summaries_name_the_kernels_the_library_builds():
             assert re.search(r"\b" + kernel + r"\b", src), (name, kernel)
     trace = open(os.path.join(ROOT, "profiles", "gemv_sweep_and_lstm_kernel_trace.md")).read()
     for kernel in ("lstm_seq_f16_kernel<2, true, 4, 16>", "decoder_step_f16_kernel<4, true>", "lstm_xcd_f16_kernel<true>", "moe_ffn_step_f16_kernel",
-                   "rnnt_step_f16_kernel"):
+                   "rnnt_step_f16_kernel", "rnnt_greedy_f16_kernel"):
         assert kernel in trace, kernel
