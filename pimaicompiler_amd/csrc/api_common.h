@@ -88,9 +88,12 @@ void launch_add_f16_vec(const half_t* a, const half_t* b, half_t* c, long total8
 // out_p[T, N] = x[T, K] . w_p[N, K]^T + bias_p for p < count (1, or 2 for the two directions of a bidirectional layer).
 int launch_input_projection(int count, float* const* out, const half_t* x, const half_t* const* w, const float* const* bias,
                             int64_t T, int64_t K, int64_t N, hipStream_t s, int64_t ldx = 0, int64_t ldw = 0);
-// The same with weights in fragment order (launch_pack_w_fragments); N, K checked by the caller.
+// The same with weights in fragment order (launch_pack_w_fragments); N, K checked by the caller.  `ones`: n_ones ranges that
+// the same launch sets to all-ones bytes with blocks of their own (a launch of their own where they are not whole
+// 16-byte words).
 int launch_input_projection_packed(int count, float* const* out, const half_t* x, const half_t* const* wp, const float* const* bias,
-                                   int64_t T, int64_t K, int64_t N, int ksteps, hipStream_t s);
+                                   int64_t T, int64_t K, int64_t N, int ksteps, hipStream_t s, const FillSegments* ones = nullptr,
+                                   int n_ones = 0);
 void packed_geometry(int64_t in_w, int64_t n_out, int* ntiles, int* ksteps);
 void launch_pack_w_fragments(const half_t* w, half_t* packed, int64_t n_out, int64_t in_w, int ntiles, int ksteps, hipStream_t s);
 // bsum[n] (fp32) = b_ih[n] + b_hh[n]; zeros for null biases.

@@ -562,16 +562,6 @@ int lstm_forward_impl(PimHipLstmPlan* plan, const void* x, const void* h0, const
             const int last = l + n - 1;
             half_t* group_out = (last == L - 1) ? (half_t*)y : plan->ybuf[last & 1];
             const PimHipLstmPlan::Cell& cf = plan->cells[(size_t)l];
-            float* outs1[1] = {plan->xproj};
-            const float* bs1[1] = {cf.bsum};
-            if (cf.w_ih_packed) {
-                const half_t* ws1[1] = {cf.w_ih_packed};
-                rc = launch_input_projection_packed(1, outs1, layer_in, ws1, bs1, T, cf.in_w, 4 * H, cf.ksteps, s);
-            } else {
-                const half_t* ws1[1] = {cf.w_ih};
-                rc = launch_input_projection(1, outs1, layer_in, ws1, bs1, T, cf.in_w, 4 * H, s);
-            }
-            if (rc != PIMHIP_OK) return rc;
             LstmXcdArgs a;
             memset(&a, 0, sizeof(a));
             FillSegments seg;
@@ -613,7 +603,18 @@ int lstm_forward_impl(PimHipLstmPlan* plan, const void* x, const void* h0, const
                     seg.words[2 * (j - 1) + 1] = (size_t)T * 4 * H;
                 }
             }
-            launch_fill_segments(seg, 2 * (n - 1), 0xffffffffu, s);
+            // the first layer's projection, and beside it (blocks of the same launch) the hand-over slots marked empty
+            float* outs1[1] = {plan->xproj};
+            const float* bs1[1] = {cf.bsum};
+            if (cf.w_ih_packed) {
+                const half_t* ws1[1] = {cf.w_ih_packed};
+                rc = launch_input_projection_packed(1, outs1, layer_in, ws1, bs1, T, cf.in_w, 4 * H, cf.ksteps, s, &seg, 2 * (n - 1));
+            } else {
+                const half_t* ws1[1] = {cf.w_ih};
+                rc = launch_input_projection(1, outs1, layer_in, ws1, bs1, T, cf.in_w, 4 * H, s);
+                launch_fill_segments(seg, 2 * (n - 1), 0xffffffffu, s);
+            }
+            if (rc != PIMHIP_OK) return rc;
             a.hx = plan->xcd_hx;
             a.g_counter = plan->xcd_g_counters;
             a.claims = plan->xcd_claims;

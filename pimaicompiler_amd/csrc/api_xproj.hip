@@ -43,9 +43,27 @@ int launch_input_projection(int count, float* const* out, const half_t* x, const
 
 // The same with weights in fragment order (pack_w_fragments_kernel); N, K checked by the caller (plan creation).
 int launch_input_projection_packed(int count, float* const* out, const half_t* x, const half_t* const* wp, const float* const* bias,
-                                   int64_t T, int64_t K, int64_t N, int ksteps, hipStream_t s)
+                                   int64_t T, int64_t K, int64_t N, int ksteps, hipStream_t s, const FillSegments* ones, int n_ones)
 {
-    if (T <= 0 || N <= 0) return PIMHIP_OK;
+    if (T <= 0 || N <= 0) {
+        if (ones && n_ones > 0) launch_fill_segments(*ones, n_ones, 0xffffffffu, s);
+        return PIMHIP_OK;
+    }
+    // ranges to set to all-ones bytes beside the projection (whole 16-byte words, or a launch of their own does it)
+    XprojFill fill;
+    memset(&fill, 0, sizeof(fill));
+    bool fill_here = ones && n_ones > 0 && n_ones <= 6;
+    for (int r = 0; fill_here && r < n_ones; ++r)
+        fill_here = (reinterpret_cast<uintptr_t>(ones->ptr[r]) & 15u) == 0 && (ones->words[r] & 3u) == 0 && ones->words[r] / 4 <= 0xffffffffull;
+    if (ones && n_ones > 0 && !fill_here) launch_fill_segments(*ones, n_ones, 0xffffffffu, s);
+    if (fill_here) {
+        for (int r = 0; r < n_ones; ++r) {
+            fill.ptr[r] = ones->ptr[r];
+            fill.words16[r] = (unsigned int)(ones->words[r] / 4);
+        }
+        fill.count = n_ones;
+        fill.blocks = 128;
+    }
     XprojPackedProblems pr;
     memset(&pr, 0, sizeof(pr));
     for (int p = 0; p < count; ++p) {
@@ -55,17 +73,28 @@ int launch_input_projection_packed(int count, float* const* out, const half_t* x
     }
     const unsigned row_blocks = (unsigned)((T + kXprojTile - 1) / kXprojTile);
     auto blocks = [&](int cols) { return (unsigned)(((N + cols - 1) / cols + 7) / 8 * 8) * row_blocks; };
+    // the projection's blocks first, the filling blocks behind them
+    auto launch_as = [&](unsigned proj_blocks, auto launch) {
+        fill.first_block = (int)proj_blocks;
+        launch(proj_blocks + (unsigned)(fill.count > 0 ? fill.blocks : 0));
+    };
     // Measured on MI355X (T = 50, 200, 800; K = 240, 1024, 2048; N = 4096): with one row block 16-column tiles and
     // eight wavefronts splitting K; with more, 32-column tiles, and eight wavefronts only for long rows and few row blocks.
     if (row_blocks >= 2) {
         pr.blocks_per_problem = (int)blocks(32);
         if (row_blocks <= 4 && K >= 2048)
-            input_projection_packed_f16_kernel<2, 8><<<blocks(32) * count, 512, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+            launch_as(blocks(32) * count, [&](unsigned grid) {
+                input_projection_packed_f16_kernel<2, 8><<<grid, 512, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks, fill);
+            });
         else
-            input_projection_packed_f16_kernel<2, 4><<<blocks(32) * count, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+            launch_as(blocks(32) * count, [&](unsigned grid) {
+                input_projection_packed_f16_kernel<2, 4><<<grid, 256, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks, fill);
+            });
     } else {
         pr.blocks_per_problem = (int)blocks(16);
-        input_projection_packed_f16_kernel<1, 8><<<blocks(16) * count, 512, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks);
+        launch_as(blocks(16) * count, [&](unsigned grid) {
+            input_projection_packed_f16_kernel<1, 8><<<grid, 512, 0, s>>>(x, pr, (int)T, (int)K, (int)N, (long)K, ksteps, (int)row_blocks, fill);
+        });
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(PIMHIP_ERR_HIP, "input projection launch failed: %s", hipGetErrorString(e));

@@ -197,12 +197,38 @@ struct XprojPackedProblems {
     int blocks_per_problem;
 };
 
+// Ranges of 16-byte words that the blocks behind the projection's own set to all-ones bytes: the hand-over slots of the
+// pipeline launch that follows (lstm_xcd_kernels.h), marked "not written yet" beside the projection instead of by a launch
+// of their own between the two.
+struct XprojFill {
+    unsigned int* ptr[6];
+    unsigned int words16[6];
+    int count;        // ranges; 0: the launch has no such blocks
+    int first_block;  // the first block that fills
+    int blocks;       // how many do
+};
+
+__device__ __forceinline__ void xproj_fill_ones(const XprojFill& f, int fb, int n_threads)
+{
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 ones = {~0u, ~0u, ~0u, ~0u};
+    for (int r = 0; r < f.count; ++r) {
+        u32x4* p = reinterpret_cast<u32x4*>(f.ptr[r]);
+        const size_t n = f.words16[r];
+        for (size_t i = (size_t)fb * n_threads + threadIdx.x; i < n; i += (size_t)f.blocks * n_threads) p[i] = ones;
+    }
+}
+
 // KS wavefronts per block, one 32-wide K step of a (32 * KS)-wide slab each.
 template <int NT, int KS = kXprojKSplit>
 __global__ __launch_bounds__(64 * KS) void input_projection_packed_f16_kernel(const half_t* __restrict__ x, XprojPackedProblems problems,
                                                                          int T, int K, int N, long ldx, int ksteps,
-                                                                         int row_blocks)
+                                                                         int row_blocks, XprojFill fill)
 {
+    if (fill.count > 0 && (int)blockIdx.x >= fill.first_block) {
+        xproj_fill_ones(fill, (int)blockIdx.x - fill.first_block, 64 * KS);
+        return;
+    }
     constexpr int SLAB = 32 * KS;                          // K values per slab
     constexpr int PITCH = SLAB + 8;                        // LDS row pitch in halves
     constexpr int CPR = SLAB / 8;                          // 16-byte pieces per x row and slab
