@@ -28,7 +28,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_scaled_f16_kernel(const ha
         float v = alpha * acc;
         if (beta != 0.0f) v += beta * (float)y[row];  // (as the reference: y is not read when beta is 0)
         if (bias) v += (float)bias[row];
-        if (relu) v = fmaxf(v, 0.0f);
+        if (relu) v = relu_f32(v);
         y[row] = (half_t)v;
     }
 }
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(64 * kVmScaledWaves) void gemv_vm_scaled_f16_kernel
         float v = alpha * s;
         if (beta != 0.0f) v += beta * (float)y[col];
         if (bias) v += (float)bias[col];
-        if (relu) v = fmaxf(v, 0.0f);
+        if (relu) v = relu_f32(v);
         y[col] = (half_t)v;
     }
 }

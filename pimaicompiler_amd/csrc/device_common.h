@@ -113,6 +113,10 @@ __device__ __forceinline__ void store16_device_scope(void* p, unsigned long long
     asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
 }
 
+// relu as at::relu computes it (the reference applies it to its GEMV's result, aten_ops.cpp:466, 704-705): below zero
+// becomes zero and a NaN stays a NaN; fmaxf would return its other operand for one.
+__device__ __forceinline__ float relu_f32(float v) { return v < 0.0f ? 0.0f : v; }
+
 __device__ __forceinline__ float sigmoid_f32(float v) { return 1.0f / (1.0f + __expf(-v)); }
 
 // Sigmoid on the hardware exp2 and reciprocal (about 1 ulp each): exact limits 0 and 1 at -+inf, absolute error

@@ -103,7 +103,7 @@ __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, c
             const long row = row0 + lane;
             if (row < N) {
                 if (bias) v += (float)bias[row];
-                if (relu) v = fmaxf(v, 0.0f);
+                if (relu) v = relu_f32(v);
                 y[row] = (half_t)v;
             }
         }
@@ -114,7 +114,7 @@ __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, c
             if (lane == r && row < N) {
                 float v = acc[r];
                 if (bias) v += (float)bias[row];
-                if (relu) v = fmaxf(v, 0.0f);
+                if (relu) v = relu_f32(v);
                 y[row] = (half_t)v;
             }
         }
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_generic_kernel(const h
     acc = wave_sum(acc);
     if (lane == 0) {
         if (bias) acc += (float)bias[row];
-        if (relu) acc = fmaxf(acc, 0.0f);
+        if (relu) acc = relu_f32(acc);
         y[row] = (half_t)acc;
     }
 }
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_vm_f16_kernel(const half_t* _
         for (int j = 0; j < 8; ++j) {
             float r = v[j];
             if (bias) r += (float)bias[col0 + j];
-            if (relu) r = fmaxf(r, 0.0f);
+            if (relu) r = relu_f32(r);
             out[j] = (half_t)r;
         }
         for (int o = 0; o < outs.count; ++o) *reinterpret_cast<half8_t*>(outs.y[o] + col0) = out;
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(64 * kVmGenericWaves) void gemv_vm_f16_generic_kern
 #pragma unroll
         for (int w = 1; w < kVmGenericWaves; ++w) v += red[w][lane];
         if (bias) v += (float)bias[col];
-        if (relu) v = fmaxf(v, 0.0f);
+        if (relu) v = relu_f32(v);
         for (int o = 0; o < outs.count; ++o) outs.y[o][col] = (half_t)v;
     }
 }

@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
     // One row of W1[e] times the token, bias and activation, as the bits `hidden` holds; a NaN in its canonical form.
     auto hidden_bits = [&](float a, int r) {
         if (b1) a += (float)b1[r];
-        if (p.act == 1) a = fmaxf(a, 0.0f);
+        if (p.act == 1) a = relu_f32(a);
         unsigned short bits = __builtin_bit_cast(unsigned short, (half_t)a);
         if (a != a) bits = 0x7e00u;
         return bits;

@@ -207,7 +207,7 @@ __device__ __forceinline__ void rnnt_greedy_solo(const RnntGreedyArgs& p, half_t
             float a = rnnt_row_dot(row, fv, nfp, lane, 0.0f);
             a = rnnt_row_dot(row + nfp, gv, nhp, lane, a);
             a = rnnt_sum(a);
-            if (lane == 0) tmp[r] = __builtin_bit_cast(half_t, rnnt_bits(fmaxf(a + (p.b1 ? (float)p.b1[r] : 0.0f), 0.0f)));
+            if (lane == 0) tmp[r] = __builtin_bit_cast(half_t, rnnt_bits(relu_f32(a + (p.b1 ? (float)p.b1[r] : 0.0f))));
         }
         __syncthreads();
         for (int v = wave; v < p.V; v += kRnntWaves) {
@@ -617,7 +617,7 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
                 for (int k = 0; k < kRnntHC; ++k)
                     if (lane + 64 * k < nhp) a = dot8(wg[k], gv[lane + 64 * k], a);
                 a = rnnt_sum(a);
-                if (lane == 0) my_values()[wave] = rnnt_bits(fmaxf(a + bias, 0.0f));
+                if (lane == 0) my_values()[wave] = rnnt_bits(relu_f32(a + bias));
                 publish(hid_entry(pub, jb), step_tag(pub, version));
                 ++pub;
             }

@@ -233,7 +233,7 @@ __device__ __forceinline__ const half_t* rnnt_solo(const RnntStepIo& io, const R
             a = rnnt_sum(a);
             if (lane == 0) {
                 if (p.b1) a += (float)p.b1[r];
-                nxt[r] = __builtin_bit_cast(half_t, rnnt_bits(fmaxf(a, 0.0f)));
+                nxt[r] = __builtin_bit_cast(half_t, rnnt_bits(relu_f32(a)));
             }
         }
         __syncthreads();
@@ -442,7 +442,7 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_step_f16_kernel(const half_
             if (lane + 64 * k < nhp) a = dot8(wg[k], gv[k], a);
         a = rnnt_sum(a);
         if (lane == 0) {
-            const unsigned short bits = rnnt_bits(fmaxf(a + bias, 0.0f));
+            const unsigned short bits = rnnt_bits(relu_f32(a + bias));
             mine[wave] = bits;
             if (p.joint_hidden) p.joint_hidden[r] = __builtin_bit_cast(half_t, bits);
         }

@@ -61,6 +61,26 @@ def test_gemv_both_orders_match_oracle(ops, n, k, bias, relu):
     assert maxabs(y, want) <= GEMV_TOL
 
 
+@pytest.mark.parametrize("n,k", [(7, 17), (512, 1344), (1024, 1024), (33, 8200), (4096, 4096)])
+def test_relu_keeps_a_nan_as_at_relu_does(ops, n, k):
+    """The reference applies at::relu to its GEMV's result (aten_ops.cpp:466, 704-705): a NaN stays a NaN, it does not
+    become 0.  One NaN weight poisons one row, one NaN bias another; the oracle and both weight orders agree on which."""
+    from pimaicompiler_amd import _lib as L
+    W, x, b = workloads.gemv_inputs(300 + n + k, n, k, bias=True)
+    W, b = W.clone(), b.clone()
+    W[n // 2, k // 3] = float("nan")
+    b[n - 1] = float("nan")
+    want = oracle.gemv_mv(W.numpy(), x.numpy().reshape(-1), b.numpy(), relu=True)
+    assert np.isnan(want[n // 2]) and np.isnan(want[n - 1]) and np.isnan(want).sum() == (1 if n // 2 == n - 1 else 2)
+    xd, bd = x.to(DEV).reshape(-1), b.to(DEV)
+    for weight, order in ((W.to(DEV), L.PIMHIP_W_X_I), (W.t().contiguous().to(DEV), L.PIMHIP_I_X_W)):
+        rc, y = raw_gemv(ops, weight, xd, bd, k, n, 0, L.PIMHIP_ACT_RELU, order)
+        assert rc == 0
+        y = y.cpu().numpy()
+        assert np.array_equal(np.isnan(y), np.isnan(want))
+        assert np.nanmax(np.abs(y.astype(np.float32) - want.astype(np.float32))) <= GEMV_TOL and np.nanmin(y) >= 0.0
+
+
 def test_gemv_result_is_correctly_rounded_almost_everywhere(ops):
     """fp32 accumulation then one rounding: the result is within one fp16 ulp of the exactly rounded value and
     equal to it for all but near-tie elements."""

@@ -190,6 +190,37 @@ def test_the_loop_recorded_into_a_graph_replays_like_the_eager_call(ops):
     assert plan.fallbacks() == (0, True)
 
 
+def test_ties_nans_and_an_empty_budget_are_decided_as_torch_argmax_decides_them(ops):
+    """Equal logits: the first index wins.  A NaN among them: it counts as the largest.  No symbols allowed: nothing runs."""
+    L, I, H, F, J, V, T = 1, 64, 32, 128, 64, 5, 6
+    g, params, joint = make(8181, L, I, H, F, J, V, True)
+    w1, b1, w2, b2 = joint
+    flat = (w1, b1, torch.zeros_like(w2), torch.full_like(b2, 0.25))        # every logit 0.25
+    enc = torch.randn(T, F, generator=g).half().to(DEV)
+    embedding = torch.randn(V, I, generator=g).half().to(DEV)
+    x0 = torch.zeros(I, dtype=torch.float16, device=DEV)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(flat)))
+    for blank, per_frame in ((0, 3), (1, 3), (4, 2)):
+        want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, per_frame, T * per_frame)
+        r = check(plan.greedy_decode(enc, embedding, x0, blank, per_frame), want)
+        assert r[0] == (0 if blank == 0 else T * per_frame)                  # index 0 every time: a blank, or a symbol
+    # a NaN in the embedding row of symbol 0 makes every later logit a NaN: index 0 again, by the other rule
+    nan_emb = embedding.clone()
+    nan_emb[0, 3] = float("nan")
+    plan2 = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    want = loop_driven_from_the_host(plan2, enc, nan_emb, nan_emb[0], 4, 2, T * 2)
+    symbols, result, hn, cn = plan2.greedy_decode(enc, nan_emb, nan_emb[0], 4, 2)
+    torch.cuda.synchronize()
+    r = result.cpu().tolist()
+    assert r[0] == len(want[0]) == T * 2 and symbols[: r[0]].cpu().tolist() == want[0] == [0] * (T * 2)
+    assert bool(torch.isnan(hn).all()) and bool(torch.isnan(want[3]).all())
+    # no budget
+    symbols, result, hn, cn = plan.greedy_decode(enc, embedding, x0, 1, 3, 0)
+    torch.cuda.synchronize()
+    assert result.cpu().tolist()[:3] == [0, 0, 0] and float(hn.abs().max()) == 0.0
+    assert plan.fallbacks() == (0, True) and plan2.fallbacks() == (0, True)
+
+
 def test_arguments_the_loop_refuses(ops):
     L, I, H, F, J, V, T = 2, 320, 320, 1024, 512, 29, 8
     params, joint, enc, embedding, x0 = model(7171, L, I, H, F, J, V, T, 28, 0.5)
