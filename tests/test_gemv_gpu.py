@@ -81,6 +81,29 @@ def test_relu_keeps_a_nan_as_at_relu_does(ops, n, k):
         assert np.nanmax(np.abs(y.astype(np.float32) - want.astype(np.float32))) <= GEMV_TOL and np.nanmin(y) >= 0.0
 
 
+@pytest.mark.parametrize("n,k", [(7, 17), (1024, 1024), (4096, 4096)])
+@pytest.mark.parametrize("x_scale", [256.0, 2.0 ** -6])
+def test_subnormal_operands_and_results_are_not_flushed(ops, n, k, x_scale):
+    """Weights and bias below the smallest normal fp16 (6.1e-5) are values like any other (LibTorch CPU does not flush
+    them either); with the small x the results are subnormal too.  Within one ulp of the oracle's exactly rounded value."""
+    torch.manual_seed(3)
+    W = (torch.randn(n, k) * 2.0 ** -18).half()
+    x = (torch.randn(k) * x_scale).half()
+    b = (torch.randn(n) * 2.0 ** -16).half()
+    assert float((W.abs() < 6.1e-5).float().mean()) > 0.99
+    want = oracle.gemv_mv(W.numpy(), x.numpy(), b.numpy())
+    assert np.abs(want.astype(np.float64)).max() > 0.0
+    if x_scale < 1.0:
+        assert np.mean(np.abs(want.astype(np.float64)) < 6.1e-5) > 0.9
+    for weight, order_is_vm in ((W.to(DEV), False), (W.t().contiguous().to(DEV), True)):
+        from pimaicompiler_amd import _lib as L
+        rc, y = raw_gemv(ops, weight, x.to(DEV), b.to(DEV), k, n, 0, L.PIMHIP_ACT_NONE, L.PIMHIP_I_X_W if order_is_vm else L.PIMHIP_W_X_I)
+        assert rc == 0
+        y = y.cpu().numpy()
+        assert np.all(np.abs(y.astype(np.float64) - want.astype(np.float64)) <= ulp_f16(want))
+        assert np.mean(y.view(np.uint16) == want.view(np.uint16)) > 0.95
+
+
 def test_gemv_result_is_correctly_rounded_almost_everywhere(ops):
     """fp32 accumulation then one rounding: the result is within one fp16 ulp of the exactly rounded value and
     equal to it for all but near-tie elements."""
