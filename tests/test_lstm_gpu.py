@@ -560,6 +560,28 @@ def test_persistent_kernel_survives_a_nan_input(ops, mode):
     assert bool(torch.isnan(want[7:]).all()) and bool(torch.isnan(y[7:]).all()) and bool(torch.isnan(cn).all())
 
 
+@pytest.mark.parametrize("mode", [1, 2, 3, 4])
+def test_saturated_gates_reach_their_limits_exactly(ops, mode):
+    """Weights forty times the usual size drive the gates far into saturation (pre-activations of tens to hundreds): the
+    sigmoid and tanh built on the hardware exp2 and reciprocal must give exactly 0, 1 and -1 there, as LibTorch's do, and
+    nothing may turn into a NaN (exp2 overflows to inf, whose reciprocal is 0).  Two steps only: with such a gain a
+    longer recurrence amplifies any last-bit difference into another trajectory, in LibTorch's own builds too."""
+    T = 2
+    params, x, h0, c0 = workloads.lstm_inputs(9, 64, 256, 2, False, T)
+    params = [(p.float() * 40).half() for p in params]
+    x = (x.float() * 8).half()
+    plan = ops.LstmPlan([p.to(DEV) for p in params], True, 2, False, T)
+    plan.set_mode(mode)
+    y, hn, cn = plan.forward(x.reshape(T, 64).to(DEV), h0.to(DEV), c0.to(DEV))
+    plan.status()
+    want_y, want_hn, want_cn = oracle.torch_lstm(x, h0, c0, params, True, 2, False)
+    assert not bool(torch.isnan(y).any()) and not bool(torch.isnan(cn).any())
+    # it does saturate: most gates of the last step are 0 or 1 to within fp16, so c moved by a whole unit or stayed
+    moved = (want_cn.float() - c0.float()).abs().reshape(-1)
+    assert float(((moved - moved.round()).abs() < 2e-3).float().mean()) > 0.3 and float(moved.max()) > 0.9
+    assert maxabs(y, want_y) <= 5e-3 and maxabs(hn, want_hn) <= 5e-3 and maxabs(cn, want_cn) <= 1e-2
+
+
 def test_a_nan_travels_through_the_pipeline_of_layers(ops):
     """Mode 4 hands h from layer to layer through slots whose "not written yet" mark is the all-ones pattern, itself a NaN:
     a NaN h is stored there in its canonical form, so it arrives, and nobody waits for a slot that looks empty."""
