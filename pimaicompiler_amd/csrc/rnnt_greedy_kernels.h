@@ -59,7 +59,7 @@ constexpr int kRnntGreedyRing = 16;                // hidden vectors and logits:
 constexpr int kRnntGreedyAhead = 8;                // steps the joint network runs ahead of the decisions
 constexpr int kRnntGreedyLook = 4;                 // steps whose logits one pass looks at
 static_assert(kRnntGreedyAhead < kRnntGreedyRing && (kRnntGreedyRing & (kRnntGreedyRing - 1)) == 0, "ring");
-constexpr int kRnntGreedyMaxVocab = 64;            // the argmax is one wavefront's ballot
+constexpr int kRnntGreedyMaxVocab = 64;            // the argmax is one maximum over one wavefront
 constexpr int kRnntGreedyEmbHalfs = 16384;         // embedding rows kept in LDS by the first layer's blocks (32 KB)
 constexpr int kRnntSeenStride = 16;                // 32-bit words between the blocks' `seen` counts
 
