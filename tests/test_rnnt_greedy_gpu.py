@@ -190,6 +190,28 @@ def test_the_loop_recorded_into_a_graph_replays_like_the_eager_call(ops):
     assert plan.fallbacks() == (0, True)
 
 
+def test_an_utterance_from_the_rnnt_feature_file_end_to_end(ops):
+    """The reference's own RNNT input (examples/runtime/resource/rnnt/inputs/feature.bin, 341 x 1 x 240 fp16, a fixture
+    here) through an encoder of the RNNT shape (two LSTM layers, 240 -> 1024, one pipeline launch) and then the whole
+    greedy loop in one launch: two launches of this library's per utterance where the reference interprets some thousand
+    operators.  The loop's symbols and state against the loop driven from the host on the same encoder output."""
+    import os
+    from pimaicompiler_amd import io, workloads
+    T, L, I, H, F, J, V, blank = 341, 2, 320, 320, 1024, 512, 29, 28
+    feat = io.load_tensor(os.path.join(os.path.dirname(__file__), "golden", "rnnt_feature_341x1x240_f16.bin"), [341, 1, 240], "FLOAT16")
+    enc_params, _, eh0, ec0 = workloads.lstm_inputs(3001, 240, F, 2, False, T)
+    eplan = ops.LstmPlan(dev(enc_params), True, 2, False, T)
+    enc, _, _ = eplan.forward(feat.reshape(T, 240).to(DEV), eh0.to(DEV), ec0.to(DEV))
+    eplan.status()
+    params, joint, _, embedding, x0 = model(777, L, I, H, F, J, V, 1, blank, 0.12)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    enc = enc.reshape(T, F).contiguous()
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, 30, T * 30)
+    r = check(plan.greedy_decode(enc, embedding, x0, blank), want)
+    assert r[1] == T and r[3] == 0 and plan.fallbacks() == (0, True)
+    assert 5 <= r[0] and r[2] >= T          # some frames emit, every frame is consumed
+
+
 def test_ties_nans_and_an_empty_budget_are_decided_as_torch_argmax_decides_them(ops):
     """Equal logits: the first index wins.  A NaN among them: it counts as the largest.  No symbols allowed: nothing runs."""
     L, I, H, F, J, V, T = 1, 64, 32, 128, 64, 5, 6
