@@ -1,11 +1,12 @@
 """The one-launch greedy decoding loop (pimhip_rnnt_greedy_decode) against the same loop driven from the host through
 pimhip_rnnt_step (which tests/test_rnnt_gpu.py holds against LibTorch CPU): symbols, counts and final state bit for bit, as
 both sum in the same order and round the state to fp16 between runs of the prediction network.  Integer outputs and fp16
-bits: no tolerance."""
+bits: no tolerance.  One test holds the loop against LibTorch CPU directly, on the decisions that the last bits of a logit
+cannot turn."""
 import pytest
 import torch
 
-from test_rnnt_gpu import DEV, dev, make
+from test_rnnt_gpu import DEV, dev, joint_cpu, libtorch_cpu_step, make
 
 pytestmark = pytest.mark.gpu
 
@@ -188,6 +189,45 @@ def test_the_loop_recorded_into_a_graph_replays_like_the_eager_call(ops):
         check((symbols, result, hn, cn), want)
         check(plan.greedy_decode(enc, embedding, x0, blank), want)      # eager calls between the replays
     assert plan.fallbacks() == (0, True)
+
+
+def test_the_loop_against_libtorch_cpu_where_the_decisions_are_clear(ops):
+    """The same loop on LibTorch CPU in fp16, operator by operator as the reference runs it (at::lstm at seq_len 1, the
+    joint network's products, argmax).  Its logits differ from the GPU's in the last bits, so only decisions whose two best
+    logits lie further apart than the tolerance can be held against it: the symbols must agree up to the first step where
+    they do not (seeded: that step, if any, is always the same one), and that has to be a good way into the utterance."""
+    L, I, H, F, J, V, T, blank, per_frame = 2, 320, 320, 1024, 512, 29, 40, 28, 3
+    params, joint, enc, embedding, x0 = model(9191, L, I, H, F, J, V, T, blank, 1.5, w2_scale=1.0)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    symbols, result, hn, cn = plan.greedy_decode(enc, embedding, x0, blank, per_frame)
+    torch.cuda.synchronize()
+    got = symbols[: int(result[0])].cpu().tolist()
+    enc_c, emb_c = enc.cpu(), embedding.cpu()
+    h, c = torch.zeros(L, H, dtype=torch.float16), torch.zeros(L, H, dtype=torch.float16)
+    t, want, in_frame, run_prediction, label, steps, clear = 0, [], 0, True, -1, 0, True
+    while t < T and clear:
+        if run_prediction:
+            h, c, _, logits = libtorch_cpu_step(params, joint, L, x0.cpu() if label < 0 else emb_c[label], h, c, enc_c[t])
+        else:
+            _, logits = joint_cpu(joint, enc_c[t], h[L - 1])
+        top2 = torch.topk(logits.float(), 2)
+        if float(top2.values[0] - top2.values[1]) <= 2e-2:
+            clear = False                       # a decision the last bits could turn: nothing behind it can be compared
+            break
+        k = int(top2.indices[0])
+        steps += 1
+        if k == blank:
+            t, in_frame, run_prediction = t + 1, 0, False
+        else:
+            want.append(k)
+            label, in_frame, run_prediction = k, in_frame + 1, True
+            if in_frame >= per_frame:
+                t, in_frame = t + 1, 0
+    assert steps >= 40 and len(want) >= 10 and len(set(want)) >= 3      # a real mix, a good way in
+    assert got[: len(want)] == want
+    if clear:
+        assert len(got) == len(want) and int(result[1]) == T
+        assert float((hn.cpu().float() - h.float()).abs().max()) <= 5e-3
 
 
 def test_an_utterance_from_the_rnnt_feature_file_end_to_end(ops):
