@@ -441,7 +441,7 @@ int pimhip_rnnt_step(PimHipRnntPlan* plan, const void* x, const void* h_prev, co
  *   shape or null, not overlapping h0 / c0; symbols [max_symbols] int32; result [8] int32: symbols emitted, frames
  *   consumed, steps taken, 1 if one workgroup had to decode alone, 1 if the last symbol has not been fed to the prediction
  *   network yet (hn / cn are the state before it), the last symbol (-1: none), 0, 0.  All device memory; fp16 tensors
- *   dense and 16-byte aligned.  vocab <= 64 (PIMHIP_ERR_UNSUPPORTED otherwise: drive pimhip_rnnt_step from the host).
+ *   dense and 16-byte aligned.  vocab <= 512 (PIMHIP_ERR_UNSUPPORTED otherwise: drive pimhip_rnnt_step from the host).
  * Symbols and final state equal, bit for bit, those of the same loop driven from the host through pimhip_rnnt_step.
  * Asynchronous; records three kernels, so it can be recorded into a HIP graph.  Residency, ordering and the plan's stream
  * as for pimhip_rnnt_step.  Every wait inside is bounded; when one gives up, one workgroup decodes the utterance again from

@@ -37,8 +37,9 @@
 // count that every block keeps of the decisions it has taken in (`seen`) before they reuse an entry.
 //
 // Waiting: a block looks at everything it waits for in one round ("pass"): the words of a vector by the first six
-// wavefronts, the logits of the next four steps by the last two.  What the block cannot go on without is polled until it
-// is there, the rest is looked at once; one barrier ends the round, and a pass can take several decisions at once.
+// wavefronts, the logits of the next four steps by the last two (of one step where there are more than 80 symbols).  What
+// the block cannot go on without is polled until it is there, the rest is looked at once; one barrier ends the round, and
+// a pass can take several decisions at once.
 //
 // Sums run in the order of the step kernel, c is rounded to fp16 after every run of the prediction network as it is when
 // the state travels between launches: symbols and final state equal, bit for bit, those of a loop of pimhip_rnnt_step
@@ -59,7 +60,8 @@ constexpr int kRnntGreedyRing = 16;                // hidden vectors and logits:
 constexpr int kRnntGreedyAhead = 8;                // steps the joint network runs ahead of the decisions
 constexpr int kRnntGreedyLook = 4;                 // steps whose logits one pass looks at
 static_assert(kRnntGreedyAhead < kRnntGreedyRing && (kRnntGreedyRing & (kRnntGreedyRing - 1)) == 0, "ring");
-constexpr int kRnntGreedyMaxVocab = 64;            // the argmax is one maximum over one wavefront
+constexpr int kRnntGreedyMaxVocab = 512;           // symbols (the logits of the steps a pass looks at lie in LDS)
+constexpr int kRnntGreedyWideVocab = 10;           // with more symbol blocks than this a pass looks at the logits of one step, not four
 constexpr int kRnntGreedyEmbHalfs = 16384;         // embedding rows kept in LDS by the first layer's blocks (32 KB)
 constexpr int kRnntSeenStride = 16;                // 32-bit words between the blocks' `seen` counts
 
@@ -142,23 +144,23 @@ __device__ __forceinline__ unsigned int rnnt_max_u32(unsigned int v)
     return v;
 }
 
-// torch.argmax over V <= 64 fp16 values: the first maximum, a NaN counting as the largest.  Every lane returns it.  One
-// integer maximum over keys: the value's bits made monotonic (-0 as +0, a NaN above everything) in front of the lane counted
-// from the top, so that of equal values the first wins.
+// torch.argmax over V fp16 values: the first maximum, a NaN counting as the largest.  Every lane returns it.  One integer
+// maximum over keys: the value's bits made monotonic (-0 as +0, a NaN above everything) in front of the index counted from
+// the top, so that of equal values the first wins.  A lane takes the values lane, lane + 64, ..
 __device__ __forceinline__ int rnnt_argmax(const half_t* lg, int V, int lane)
 {
     unsigned int key = 0u;
-    if (lane < V) {
-        unsigned int bits = __builtin_bit_cast(unsigned short, lg[lane]);
+    for (int i = lane; i < V; i += 64) {
+        unsigned int bits = __builtin_bit_cast(unsigned short, lg[i]);
         if (bits == 0x8000u) bits = 0u;
         unsigned int order = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
         if ((bits & 0x7fffu) > 0x7c00u) order = 0xffffu;
-        key = (order << 8) | (unsigned int)(255 - lane);
+        key = max(key, (order << 16) | (unsigned int)(0xffff - i));
     }
-    return 255 - (int)(rnnt_max_u32(key) & 0xffu);
+    return 0xffff - (int)(rnnt_max_u32(key) & 0xffffu);
 }
 
-// The whole loop by one workgroup.  LDS: hs [L * H] (h of every layer), cs [L * H], tmp [max(H, J)], lg [64].
+// The whole loop by one workgroup.  LDS: hs [L * H] (h of every layer), cs [L * H], tmp [max(H, J)], lg [V].
 __device__ __forceinline__ void rnnt_greedy_solo(const RnntGreedyArgs& p, half_t* hs, half_t* cs, half_t* tmp, half_t* lg)
 {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -360,8 +362,12 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
                 }
             }
         } else if (want_steps) {
-            const int j = (tid - 384) >> 5, i = (tid - 384) & 31;
-            if (i < 3 * nwv) {
+            // 32 threads per step for the logits of four steps, or (many symbols) all 128 for those of `step` alone
+            const bool wide = nwv > kRnntGreedyWideVocab;
+            const int per_step = wide ? 128 : 32;
+            const int j = (tid - 384) / per_step, i0 = (tid - 384) - j * per_step;
+            if (wide && tid - 384 < kRnntGreedyLook - 1) miss[2 + (tid - 384)] = 1;
+            for (int i = i0; i < 3 * nwv; i += per_step) {
                 const int prod = i / 3, part = i - 3 * prod;
                 if (fetch(lg_entry(step + j, prod) + part, step_tag(step + j, g_version()), step_blocks && j == 0, miss, w))
                     unpack(w, lgs[n_pass & 1u][j], prod, part);
@@ -736,7 +742,7 @@ __global__ __launch_bounds__(kRnntThreads) void rnnt_greedy_f16_kernel(const Rnn
     if (someone_gave_up != 0) {
         if (tid == 0) i_decode_alone = (p.alone || atomicCAS(p.solo_owner, 0u, 1u) == 0u) ? 1 : 0;
         __syncthreads();
-        if (i_decode_alone) rnnt_greedy_solo(p, solo_hs, solo_cs, buf0, lgs[0][0]);
+        if (i_decode_alone) rnnt_greedy_solo(p, solo_hs, solo_cs, buf0, &lgs[0][0][0]);
         return;
     }
     if (b == 0 && tid == 0) {

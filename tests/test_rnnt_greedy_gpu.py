@@ -79,6 +79,8 @@ CASES = [
     (3, 72, 136, 200, 1024, 8, 40, 3, 4, None, 0.2, False),
     (4, 1024, 256, 2048, 512, 64, 25, 63, 5, None, 0.5, True),       # widest x and f, embedding rows read from memory
     (1, 64, 32, 128, 64, 5, 0, 0, 3, None, 0.3, True),               # no frames
+    (1, 64, 32, 128, 64, 100, 30, 99, 3, None, 0.3, True),           # more symbols than a look at four steps takes
+    (2, 64, 64, 256, 128, 300, 25, 7, 4, None, 0.3, True),           # ... and an embedding too large for LDS
 ]
 
 
@@ -155,6 +157,17 @@ def test_a_loop_whose_waits_give_up_still_gives_the_right_result(ops):
     plan2 = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
     r = check(plan2.greedy_decode(enc, embedding, x0, blank), want)
     assert r[3] == 0 and plan2.fallbacks() == (0, True)
+
+
+def test_a_workgroup_decoding_alone_handles_many_symbols_too(ops):
+    L, I, H, F, J, V, T, blank = 1, 64, 32, 128, 64, 100, 20, 99
+    params, joint, enc, embedding, x0 = model(5252, L, I, H, F, J, V, T, blank, 0.05)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, 3, T * 3)
+    assert len(want[0]) >= 3
+    plan.set_spin_limit(0)
+    r = check(plan.greedy_decode(enc, embedding, x0, blank, 3), want)
+    assert r[3] == 1
 
 
 def test_the_loop_recorded_into_a_graph_replays_like_the_eager_call(ops):
@@ -297,9 +310,9 @@ def test_arguments_the_loop_refuses(ops):
         plan.greedy_decode(enc, embedding, None, 28)
     with pytest.raises(ops.NNRuntimeException, match=r"\[T, 1024\]"):
         plan.greedy_decode(enc[:, :512], embedding, x0, 28)
-    # more symbols than one wavefront's ballot takes
-    g2, params2, joint2 = make(7272, 1, 64, 32, 128, 64, 130, True)
+    # more symbols than the loop kernel keeps logits for
+    g2, params2, joint2 = make(7272, 1, 64, 32, 128, 64, 600, True)
     plan2 = ops.RnntPlan(dev(params2), True, 1, tuple(dev(joint2)))
     with pytest.raises(ops.NNRuntimeException, match="symbols"):
-        plan2.greedy_decode(torch.zeros(4, 128, dtype=torch.float16, device=DEV), torch.zeros(130, 64, dtype=torch.float16, device=DEV),
+        plan2.greedy_decode(torch.zeros(4, 128, dtype=torch.float16, device=DEV), torch.zeros(600, 64, dtype=torch.float16, device=DEV),
                             torch.zeros(64, dtype=torch.float16, device=DEV), 0)
