@@ -324,16 +324,28 @@ int pimhip_decoder_plan_set_encoder(PimHipDecoderPlan* plan, const void* enc, in
  * h_prev[k] / c_prev[k] were read from (a one-layer plan without a classifier excepted); no other output may alias an
  * input.  All blocks of the launch have to be resident at once, so the call is ordered like a sequence call of
  * pimhip_lstm_forward against the device's other such launches, and steps sharing a plan must be ordered on one stream.
- * Records one kernel.  Every wait inside is bounded: see pimhip_decoder_plan_status. */
+ * h_prev, c_prev and x 16-byte aligned.
+ * Records one kernel.  Every wait inside is bounded (a poll count and one second).  When one gives up because part of the
+ * grid was kept from running, the block that waited computes the missing values itself, in the order their owner would
+ * have (the step's results are bit for bit what they would have been), and a block that cannot know whether every other
+ * block has read the previous state yet keeps its new state in the plan's memory until the last block of the launch
+ * stores it to hn / cn: the in-place update stays safe.  Slower (milliseconds when most of the grid is missing), never
+ * undefined; pimhip_decoder_plan_fallbacks counts the events. */
 int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const void* att, const void* ctx_in,
                         const void* const* h_prev, const void* const* c_prev, void* const* hn,
                         void* const* cn, void* const* layer_outs, void* const* ctx_outs, int n_ctx_outs, void* logits,
                         void* stream);
 
-/* As pimhip_lstm_plan_status / pimhip_lstm_plan_set_spin_limit: a wait that gave up is reported exactly once, by the
- * status call (after the stream has been synchronised) or by the next pimhip_decoder_step, which then launches nothing. */
+/* Always PIMHIP_OK for a valid plan: no step of this plan leaves an undefined result (kept for callers of the earlier
+ * interface, where a wait that gave up was an error). */
 int pimhip_decoder_plan_status(PimHipDecoderPlan* plan);
+/* The poll limit of the waits inside a step (default 2^22; 0: a wait gives up at its first look, which tests use). */
 int pimhip_decoder_plan_set_spin_limit(PimHipDecoderPlan* plan, unsigned int spin_limit);
+/* No counterpart in the reference.  *events: how many times a wait inside a step of this plan has given up so far (as far
+ * as the host has seen: ask after synchronising the stream; counted per step that had one, when the next step is issued
+ * outside a graph capture or here); *patient (may be null): 1 while waits run to the plan's poll limit, 0 once, after
+ * the third event, every wait of the plan's steps gives up after 4096 polls. */
+int pimhip_decoder_plan_fallbacks(PimHipDecoderPlan* plan, uint64_t* events, int* patient);
 
 /* ---- mixture-of-experts feed-forward step ----------------------------------------------------- */
 

@@ -68,6 +68,7 @@ SIGNATURES = {
                                            ctypes.c_void_p, c_void_pp, c_void_pp, c_void_pp, c_void_pp, c_void_pp, c_void_pp,
                                            ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
     "pimhip_decoder_plan_status": (ctypes.c_int, [ctypes.c_void_p]),
+    "pimhip_decoder_plan_fallbacks": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_int)]),
     "pimhip_decoder_plan_set_spin_limit": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint]),
     "pimhip_moe_plan_create": (ctypes.c_int, [c_void_pp, ctypes.c_void_p, ctypes.c_void_p, c_void_pp, c_void_pp, c_void_pp,
                                               c_void_pp, ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,

@@ -3,6 +3,8 @@
 #include "api_common.h"
 #include "decoder_kernels.h"
 
+#include <algorithm>
+
 using namespace pimhip;
 
 struct PimHipDecoderPlan {
@@ -23,19 +25,23 @@ struct PimHipDecoderPlan {
     int64_t enc_cap = 0;              // encoder positions cx_proj has room for
     const half_t* enc = nullptr;      // the encoder outputs the projection was made from (read again only for ctx_outs)
     int64_t enc_len = 0;
-    unsigned int* hx = nullptr;       // [kDecStages][blocks][kDecEntryWords], zero when *g_counter == 1
-    unsigned int* g_counter = nullptr;
-    unsigned int* abort_flag = nullptr;
+    unsigned int* hx = nullptr;       // [kDecStages][blocks][kDecEntryWords], zeros before the first launch
+    // One allocation behind `notes`: the blocks' notes (kDecNoteWords 64-bit words each, and one word more; zeros before the
+    // first launch), then the parked h and c ([num_layers][H] fp16 each).
+    unsigned long long* notes = nullptr;
+    half_t* parked_h = nullptr;
+    half_t* parked_c = nullptr;
     unsigned int* abort_host = nullptr;
     unsigned int* abort_host_dev = nullptr;
     unsigned int spin_limit = 1u << 22;
+    unsigned long long gave_up_events = 0;  // waits that gave up, as far as the host has seen them (pimhip_decoder_plan_fallbacks)
     int blocks = 0;
-    bool reset_exchange = false;
 };
 
 namespace
 {
 std::vector<PimHipDecoderPlan*> g_decoder_plans;
+constexpr unsigned long long kDecEventsBeforeImpatient = 3;  // waits given up before every wait of a plan's steps is short
 
 int destroy_decoder_plan_locked(PimHipDecoderPlan* plan)
 {
@@ -47,8 +53,7 @@ int destroy_decoder_plan_locked(PimHipDecoderPlan* plan)
     if (plan->bsum) hipFree(plan->bsum);
     if (plan->cx_proj) hipFree(plan->cx_proj);
     if (plan->hx) hipFree(plan->hx);
-    if (plan->g_counter) hipFree(plan->g_counter);
-    if (plan->abort_flag) hipFree(plan->abort_flag);
+    if (plan->notes) hipFree(plan->notes);
     if (plan->abort_host) hipHostFree(plan->abort_host);
     if (prev >= 0) hipSetDevice(prev);
     for (size_t i = 0; i < g_decoder_plans.size(); ++i) {
@@ -149,10 +154,16 @@ extern "C" int pimhip_decoder_plan_create(PimHipDecoderPlan** plan_out, const vo
     const size_t words = (size_t)kDecStages * blocks * kDecEntryWords;
     DEC_HIP_CHECK(hipMalloc(&plan->hx, words * sizeof(unsigned int)));
     launch_fill_u32(plan->hx, words, 0u, s);
-    DEC_HIP_CHECK(hipMalloc(&plan->g_counter, sizeof(unsigned int)));
-    launch_fill_u32(plan->g_counter, 1, 1u, s);
-    DEC_HIP_CHECK(hipMalloc(&plan->abort_flag, sizeof(unsigned int)));
-    launch_fill_u32(plan->abort_flag, 1, 0u, s);
+    {
+        const size_t note_words = 2 * ((size_t)blocks * kDecNoteWords + 1);                  // 32-bit words
+        const size_t state_words = ((size_t)num_layers * H * sizeof(half_t) + 3) / 4;         // per parked array
+        const size_t aux_words = note_words + 2 * state_words;
+        DEC_HIP_CHECK(hipMalloc(&plan->notes, aux_words * sizeof(unsigned int)));
+        unsigned int* aux = reinterpret_cast<unsigned int*>(plan->notes);
+        plan->parked_h = reinterpret_cast<half_t*>(aux + note_words);
+        plan->parked_c = reinterpret_cast<half_t*>(aux + note_words + state_words);
+        launch_fill_u32(aux, aux_words, 0u, s);
+    }
     DEC_HIP_CHECK(hipGetLastError());
     DEC_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&plan->abort_host), sizeof(unsigned int), hipHostMallocMapped));
     *plan->abort_host = 0u;
@@ -229,11 +240,16 @@ extern "C" int pimhip_decoder_plan_set_spin_limit(PimHipDecoderPlan* plan, unsig
 extern "C" int pimhip_decoder_plan_status(PimHipDecoderPlan* plan)
 {
     if (!plan) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan is null");
-    if (*plan->abort_host != 0u) {
-        *plan->abort_host = 0u;
-        plan->reset_exchange = true;
-        return fail(PIMHIP_ERR_TIMEOUT, "a bounded wait of the decoder step kernel gave up: the results of that step are undefined");
-    }
+    // A wait that gives up is made good inside the same launch (the entries that did not come are computed where they are
+    // missed), so there is nothing to report as an error.  pimhip_decoder_plan_fallbacks counts the events.
+    return PIMHIP_OK;
+}
+
+extern "C" int pimhip_decoder_plan_fallbacks(PimHipDecoderPlan* plan, uint64_t* events, int* patient)
+{
+    if (!plan || !events) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "plan and events must be non-null");
+    *events = plan->gave_up_events + (*plan->abort_host != 0u ? 1u : 0u);
+    if (patient) *patient = *events >= kDecEventsBeforeImpatient ? 0 : 1;
     return PIMHIP_OK;
 }
 
@@ -270,33 +286,23 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     PIMHIP_HIP_CHECK(hipStreamIsCapturing(s, &capture));
     const bool capturing = capture != hipStreamCaptureStatusNone;
-    if (*plan->abort_host != 0u) {
-        if (capturing)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "an earlier step of this plan gave up a wait; recovering from that is not for a graph");
-        PIMHIP_HIP_CHECK(hipStreamSynchronize(s));
+    if (*plan->abort_host != 0u && !capturing) {
+        // A wait gave up in an earlier step; that step made the missing entries itself and its results stand.  The exchange
+        // buffer needs nothing (every block has written every entry of that launch by the time it ended).
         *plan->abort_host = 0u;
-        plan->reset_exchange = true;
-        return fail(PIMHIP_ERR_TIMEOUT, "an earlier step of this plan gave up a wait of the decoder step kernel: its results are undefined "
-                                        "(this call was not launched; the next one starts from a re-initialised exchange buffer)");
+        ++plan->gave_up_events;
     }
-    if (plan->reset_exchange) {
-        if (capturing)
-            return fail(PIMHIP_ERR_UNSUPPORTED, "the plan's exchange buffer has to be re-initialised after a time-out, which a graph must not "
-                                                "record: run one step outside the capture first");
-        const size_t words = (size_t)kDecStages * plan->blocks * kDecEntryWords;
-        launch_fill_u32(plan->hx, words, 0u, s);
-        launch_fill_u32(plan->g_counter, 1, 1u, s);
-        launch_fill_u32(plan->abort_flag, 1, 0u, s);
-        PIMHIP_HIP_CHECK(hipGetLastError());
-        plan->reset_exchange = false;
-    }
+    // A plan whose steps have had to do that kDecEventsBeforeImpatient times keeps every wait short: a step then costs a
+    // few milliseconds at worst when part of the grid is kept from running, instead of a second.
+    const unsigned int spin_limit = plan->gave_up_events >= kDecEventsBeforeImpatient ? std::min(plan->spin_limit, kDecImpatientPolls) : plan->spin_limit;
 
     DecoderStepArgs a;
     memset(&a, 0, sizeof(a));
     a.n_layers = L;
     for (int l = 0; l < L; ++l) {
         if (!h_prev[l] || !c_prev[l] || !hn[l] || !cn[l]) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "state pointers of layer %d are null", l);
-        if (!aligned16(h_prev[l])) return fail(PIMHIP_ERR_UNSUPPORTED, "h_prev of layer %d must be 16-byte aligned", l);
+        if (!aligned16(h_prev[l]) || !aligned16(c_prev[l]))
+            return fail(PIMHIP_ERR_UNSUPPORTED, "h_prev and c_prev of layer %d must be 16-byte aligned", l);
         DecoderLayerArgs& ly = a.layer[l];
         ly.w_ih = plan->w_ih[l];
         ly.w_hh = plan->w_hh[l];
@@ -329,10 +335,11 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
     a.logits = (half_t*)logits;
     a.vocab = (int)plan->vocab;
     a.hx = plan->hx;
-    a.g_counter = plan->g_counter;
-    a.abort_flag = plan->abort_flag;
+    a.notes = plan->notes;
+    a.parked_h = plan->parked_h;
+    a.parked_c = plan->parked_c;
     a.abort_host = plan->abort_host_dev;
-    a.spin_limit = plan->spin_limit;
+    a.spin_limit = spin_limit;
     a.H = (int)H;
     // All blocks have to be resident at once, like the sequence kernel's: ordered after it on other streams.
     if (!capturing) {
@@ -358,3 +365,4 @@ extern "C" int pimhip_decoder_step(PimHipDecoderPlan* plan, const void* x, const
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
 }
+

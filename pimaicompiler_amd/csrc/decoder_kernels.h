@@ -39,11 +39,18 @@
 // streaming wavefronts ask for after it (one group of classifier rows per layer) streams while the output travels.
 //
 // Exchange: hx[stage][NB] entries of 64 bytes: a block's four fp16 outputs of layer `stage` in the first 8 bytes.
-// |y| <= 1, so bit 14 of each fp16 carries a flag, the parity of the launch count g (a device word read at the start and
-// advanced by block 0 at the end): a slot written by launch g - 1 cannot pass for launch g, and the buffer starts as
-// zeros with g = 1.  A NaN (bit 14 set) travels as the otherwise unused pattern 0x3fff.  Every wait is bounded: after
-// `spin_limit` polls a lane raises the abort flags, all lanes stop waiting, the kernel runs to its end with undefined
-// results and the host reports a time-out.
+// |y| <= 1, so bit 14 of each fp16 carries a flag, the parity of the launch count g (kept per block in device memory: read at the
+// start, advanced at the end): a slot written by launch g - 1 cannot pass for launch g, and the buffer starts as
+// zeros with g = 1.  A NaN (bit 14 set) travels as the otherwise unused pattern 0x3fff.
+//
+// Every wait is bounded (`spin_limit` polls, one second of the constant clock), and a wait that gives up costs time, not
+// the result.  The polling wavefront computes the entries that have not come itself, with the very operations, in the very
+// order, of the block that owns them (dec_substitute): it holds every layer's previous state in LDS from the start of the
+// kernel, so the values, and everything made of them, are bit for bit what they would have been.  The block that is late
+// still does its own share when it runs.  The previous state may be the very buffers the new one goes to (hn == h_prev):
+// a block that went past layer 0's exchange without everybody's entry cannot know whether everybody has read its inputs
+// yet, so it parks its new state in the plan's memory instead; every block notes when it has read the inputs and when its
+// parked state is complete, and whichever of these notes comes last makes its writer store the parked state to hn / cn.
 #pragma once
 
 #include "device_common.h"
@@ -68,6 +75,8 @@ static constexpr int kDecEntryWords = 16;    // 32-bit words between the entries
 static constexpr int kDecStages = kDecMaxLayers;      // exchange stages: one per layer
 static constexpr int kDecMaxCtxOuts = 4;
 static constexpr unsigned short kDecNanCode = 0x3fffu;
+static constexpr int kDecNoteWords = 8;
+static constexpr unsigned int kDecImpatientPolls = 4096u;  // the poll limit of a wavefront's waits after its first one that gave up
 
 struct DecoderLayerArgs {
     const half_t* w_ih;    // [4H, in_w]
@@ -100,9 +109,15 @@ struct DecoderStepArgs {
     half_t* logits;        // [vocab]
     int vocab;
     unsigned int* hx;          // [kDecStages][NB][kDecEntryWords]
-    unsigned int* g_counter;   // launches this buffer has seen, plus 1
-    unsigned int* abort_flag;
-    unsigned int* abort_host;
+    // Per block b, kDecNoteWords 64-bit words (one 64-byte line) at notes + b * kDecNoteWords, written by that block only:
+    //   [0] the launches the block has run (every block runs once per launch, so all agree: this launch is number g = that + 1)
+    //   [1] the last launch in which the block has read all the inputs of the step
+    //   [2] the last launch in which the block parked its new state (written when all of it is in place)
+    // and after the blocks' lines one word: the last launch in which some block parked its new state.  All zero at first.
+    unsigned long long* notes;
+    half_t* parked_h;          // [n_layers][H] the parked h of such blocks
+    half_t* parked_c;          // [n_layers][H]
+    unsigned int* abort_host;  // pinned host word: raised when a wait gives up, for the host's count
     unsigned int spin_limit;
     int H;
 };
@@ -122,6 +137,134 @@ __device__ __forceinline__ float transpose_sum4(const float (&acc)[4], int lane)
 __device__ __forceinline__ unsigned int readlane_u32(unsigned int v, int l)
 {
     return (unsigned int)__builtin_amdgcn_readlane((int)v, l);
+}
+
+// The cell of one hidden unit from its four gate sums: lanes 4q .. 4q+3 of a quad hold the sums of the gates i, f, g, o
+// (`pg` = lane & 3), every lane of the quad returns the unit's h.  The owner of a unit and a block that stands in for it
+// both go through here; every operation is spelled out (no contraction left to the compiler) so that both get the same bits.
+__device__ __forceinline__ half_t dec_cell(float a, int pg, float cprev, float& c_new, bool& is_number)
+{
+    const bool is_g = pg == 2;
+    const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
+    const float act = is_g ? fmaf(2.0f, sg, -1.0f) : sg;
+    const float g_i = dpp_mov_f32<0x00>(act);
+    const float g_f = dpp_mov_f32<0x55>(act);
+    const float g_g = dpp_mov_f32<0xAA>(act);
+    const float g_o = dpp_mov_f32<0xFF>(act);
+    c_new = fmaf(g_f, cprev, g_i * g_g);
+    is_number = (c_new == c_new) && (g_o == g_o);
+    return round_f16(g_o * fmaf(2.0f, fast_sigmoid_f32(2.0f * c_new), -1.0f));
+}
+
+// How a streaming wavefront (unit `j`, half `hf` of the columns) splits a row of `nchunks` 16-byte pieces.
+struct DecPiece {
+    bool active;
+    int chunk;
+};
+__device__ __forceinline__ DecPiece dec_piece(int nchunks, int hf, int lane)
+{
+    const int n0 = (nchunks + 1) >> 1;
+    const int my_cnt = hf ? nchunks - n0 : n0;
+    DecPiece r;
+    r.active = lane < my_cnt;
+    r.chunk = r.active ? (hf ? n0 : 0) + lane : 0;
+    return r;
+}
+
+// The exchange entry of block `z` for layer `k` (first: k == 0), made by one wavefront from the step's inputs and the
+// layer's input: the same loads, products and sums, in the same order, as block z's own wavefronts make (two streaming
+// wavefronts per unit, then the cell), so the same bits.  hprev_k / cprev_k: the layer's previous state, all H values;
+// in_vec: the layer's input without the context part (k >= 1); ctx_vec: a given context.
+// (Inlined: as a function of its own it needs a stack, which costs the undisturbed step more than the cold code in its way.)
+struct DecSubstituteLayer {
+    const half_t* w_ih;
+    const half_t* w_hh;
+    const float* bsum;
+    const float* cx_proj;
+    int in_w;
+    int takes_ctx;
+};
+__device__ __forceinline__ unsigned long long dec_substitute(const DecSubstituteLayer ly, bool first, int z, int lane, int H,
+                                                                       const half_t* x, const half_t* att, int S, bool ctx_given,
+                                                                       const half_t* hprev_k, const half_t* cprev_k,
+                                                                       const half_t* in_vec, const half_t* ctx_vec, unsigned short flag)
+{
+    const int nchunks = H >> 3;
+    const int gate_of_slot[4] = {0, 2, 1, 3};
+    const int pg = lane & 3;
+    half8_t zero8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) zero8[e] = (half_t)0.0f;
+    unsigned long long word = 0ull;
+    for (int u = 0; u < kDecUnits; ++u) {
+        const int j = z * kDecUnits + u;
+        unsigned int bits = flag;
+        if (j < H) {
+            float half_sum[2];
+            for (int hf = 0; hf < 2; ++hf) {
+                const DecPiece pc = dec_piece(nchunks, hf, lane);
+                auto row_ptr = [&](const half_t* base, int v, long pitch, long col0) {
+                    return reinterpret_cast<const half8_t*>(base + ((long)gate_of_slot[v] * H + j) * pitch + col0);
+                };
+                float acc[4];
+                const half8_t hv = pc.active ? *reinterpret_cast<const half8_t*>(&hprev_k[pc.chunk * 8]) : zero8;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[v] = dot8(load_stream(row_ptr(ly.w_hh, v, H, 0) + pc.chunk), hv, 0.0f);
+                if (ly.takes_ctx) {
+                    if (ly.cx_proj) {
+                        const int e_mine = 64 * hf + lane;
+                        const float att_mine = (att && e_mine < S) ? (float)att[e_mine] : 0.0f;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            acc[v] = fmaf(att_mine, ly.cx_proj[((long)gate_of_slot[v] * H + j) * S + min(e_mine, S - 1)], acc[v]);
+                        for (int e = e_mine + 128; e < S; e += 128) {
+                            const float a = (float)att[e];
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) acc[v] = fmaf(a, ly.cx_proj[((long)gate_of_slot[v] * H + j) * S + e], acc[v]);
+                        }
+                    } else {
+                        const half8_t cvec = (ctx_given && pc.active) ? *reinterpret_cast<const half8_t*>(&ctx_vec[pc.chunk * 8]) : zero8;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) acc[v] = dot8(load_stream(row_ptr(ly.w_ih, v, ly.in_w, H) + pc.chunk), cvec, acc[v]);
+                    }
+                }
+                if (first) {
+                    const int xw = ly.takes_ctx ? H : ly.in_w;
+                    const int xchunks = xw >> 3;
+                    const int xn0 = (xchunks + 1) >> 1;
+                    const int x_begin = hf ? xn0 : 0, x_end = hf ? xchunks : xn0;
+                    const half8_t* xv = reinterpret_cast<const half8_t*>(x);
+                    if (x_end - x_begin <= 64) {
+                        const bool x_active = lane < x_end - x_begin;
+                        const int x_chunk = x_active ? x_begin + lane : 0;
+                        const half8_t xvec = x_active ? xv[x_chunk] : zero8;
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) acc[v] = dot8(load_stream(row_ptr(ly.w_ih, v, ly.in_w, 0) + x_chunk), xvec, acc[v]);
+                    } else {
+                        for (int c = x_begin + lane; c < x_end; c += 64) {
+                            const half8_t xr = xv[c];
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) acc[v] = dot8(load_stream(row_ptr(ly.w_ih, v, ly.in_w, 0) + c), xr, acc[v]);
+                        }
+                    }
+                } else {
+                    const half8_t pv = pc.active ? *reinterpret_cast<const half8_t*>(&in_vec[pc.chunk * 8]) : zero8;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[v] = dot8(load_stream(row_ptr(ly.w_ih, v, ly.in_w, 0) + pc.chunk), pv, acc[v]);
+                }
+                half_sum[hf] = transpose_sum4(acc, lane);  // gate (lane & 3) in every lane
+            }
+            const float a = half_sum[0] + half_sum[1] + ly.bsum[(long)pg * H + j];
+            float c_new;
+            bool is_number;
+            const half_t h_new = dec_cell(a, pg, (float)cprev_k[j], c_new, is_number);
+            // Lanes 0..3 hold what the owner's cell works on: the sums the streaming wavefronts hand over are those of their
+            // lanes 0..3, and the other quads of a wavefront add the same four partial sums in another order (wave_sum_mod4).
+            bits = readlane_u32((unsigned int)((is_number ? __builtin_bit_cast(unsigned short, h_new) : kDecNanCode) | flag), 0);
+        }
+        word |= (unsigned long long)bits << (16 * u);
+    }
+    return word;
 }
 
 // L = p.n_layers and CLS = "there is a classifier" are template parameters so that the order of loads and uses is fixed
@@ -145,9 +288,11 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
 {
     static_assert(L >= 1 && L <= kDecMaxLayers, "layers per step");
     static_assert(kDecPollWaves == 1 || kDecPollWaves == 2 || kDecPollWaves == 4, "entries per polling lane");
-    __shared__ __align__(16) half_t in_vec[kDecMaxH];                  // the current layer's input without the context part
+    __shared__ __align__(16) half_t in_vec[2][kDecMaxH];               // layer k's input without the context part in [k & 1], its output goes to the other
     __shared__ __align__(16) half_t ctx_vec[kDecMaxH];                 // a given context (ctx_in)
-    __shared__ __align__(16) half_t hprev[kDecMaxLayers][kDecMaxH];    // the previous hidden state of the layers after the first
+    __shared__ __align__(16) half_t hprev[kDecMaxLayers][kDecMaxH];    // every layer's previous hidden state (the streamers read layer 0's from memory)
+    __shared__ __align__(16) half_t cprev[kDecMaxLayers][kDecMaxH];    // every layer's previous cell state: for entries that have to be made here
+    __shared__ unsigned int parked_lds;                                // some wavefront went past layer 0's exchange without every entry
     __shared__ float part[kDecStreamWaves][4];                         // a layer's gate sums: [wavefront][gate]
 
     const int tid = threadIdx.x;
@@ -346,7 +491,7 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
         }
 #pragma unroll
         for (int k = 1; k < L; ++k) {
-            const half8_t pv = active ? *reinterpret_cast<const half8_t*>(&in_vec[chunk * 8]) : zero8;
+            const half8_t pv = active ? *reinterpret_cast<const half8_t*>(&in_vec[k & 1][chunk * 8]) : zero8;
 #pragma unroll
             for (int v = 0; v < 4; ++v) acc[k][v] = dot8(w_in[k][v], pv, acc[k][v]);
             deliver(k);
@@ -362,7 +507,7 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
         if (has_cls) {
             half8_t vv[CH];
 #pragma unroll
-            for (int c = 0; c < CH; ++c) vv[c] = (c * 64 + lane < nchunks) ? *reinterpret_cast<const half8_t*>(&in_vec[(c * 64 + lane) * 8]) : zero8;
+            for (int c = 0; c < CH; ++c) vv[c] = (c * 64 + lane < nchunks) ? *reinterpret_cast<const half8_t*>(&in_vec[L & 1][(c * 64 + lane) * 8]) : zero8;
             auto cls_finish = [&](const half8_t (&src)[4][CH], int it, float bias, bool bias_given) __attribute__((always_inline)) {
                 const long r0 = cls_row0(it);
                 float s[4];
@@ -397,7 +542,11 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
         // ========================= the wavefronts that activate, publish and poll (no weights) =========================
         const int pw = wave - kDecStreamWaves;         // 0: also activates and publishes
         constexpr int QP = 4 / kDecPollWaves;          // entries polled per lane: blocks lane + 64 (pw * QP + q)
-        const unsigned int g = __hip_atomic_load(p.g_counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the number of this launch, kept per block: a block that runs late must not find it advanced by one that is done
+        unsigned long long* const my_notes = p.notes + (long)blockIdx.x * kDecNoteWords;
+        unsigned long long* const parked_any = p.notes + (long)nb * kDecNoteWords;
+        const unsigned long long g = __hip_atomic_load(my_notes, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1ull;
+        if (tid == kDecStreamWaves * 64) parked_lds = 0u;
         // lanes 4u .. 4u+3 are the gates i, f, g, o of unit u of this block (lanes 16.. repeat them)
         const int pu = (lane >> 2) & 3, pg = lane & 3;
         const int pj = blockIdx.x * kDecUnits + pu;
@@ -413,30 +562,55 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                 cprev_r[k] = (float)p.layer[k].c_prev[pjc];
             }
         }
-        // the later layers' h_prev, layer 0's input (for its residual sum, when it is H wide) and a given context into LDS
+        // every layer's previous state, layer 0's input (for its residual sum, when it is H wide) and a given context into LDS
         for (int c = pw * 64 + lane; c < nchunks; c += 64 * kDecPollWaves) {
 #pragma unroll
-            for (int k = 1; k < L; ++k) *reinterpret_cast<half8_t*>(&hprev[k][c * 8]) = reinterpret_cast<const half8_t*>(p.layer[k].h_prev)[c];
-            if (p.x_w == H) *reinterpret_cast<half8_t*>(&in_vec[c * 8]) = reinterpret_cast<const half8_t*>(p.x)[c];
+            for (int k = 0; k < L; ++k) {
+                *reinterpret_cast<half8_t*>(&hprev[k][c * 8]) = reinterpret_cast<const half8_t*>(p.layer[k].h_prev)[c];
+                *reinterpret_cast<half8_t*>(&cprev[k][c * 8]) = reinterpret_cast<const half8_t*>(p.layer[k].c_prev)[c];
+            }
+            if (p.x_w == H) *reinterpret_cast<half8_t*>(&in_vec[0][c * 8]) = reinterpret_cast<const half8_t*>(p.x)[c];
             if (p.ctx_in) *reinterpret_cast<half8_t*>(&ctx_vec[c * 8]) = reinterpret_cast<const half8_t*>(p.ctx_in)[c];
         }
         const unsigned short flag = (unsigned short)((g & 1u) << 14);
-        bool gave_up = false;
+        bool gave_up = false;  // a wait of this wavefront has given up: its later waits are short
         // one step of a bounded wait: true when the caller should stop waiting
         unsigned long long t_first = 0ull;
         auto give_up_check = [&](unsigned int& spins) {
             ++spins;
-            if ((spins & 255u) == 0u) {
-                if (__hip_atomic_load(p.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) gave_up = true;
-                if (wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
-            }
-            if (spins >= p.spin_limit) {
-                __hip_atomic_store(p.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                gave_up = true;
-            }
-            return gave_up;
+            if ((spins & 255u) == 0u && wait_clock_expired(spins, t_first)) spins = 0xffffffffu;  // gives up below
+            const unsigned int limit = gave_up ? min(p.spin_limit, kDecImpatientPolls) : p.spin_limit;
+            if (spins < limit) return false;
+            __hip_atomic_store(p.abort_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            gave_up = true;
+            return true;
         };
+        // Parked state goes to hn / cn once every block has read the step's inputs (every block notes that, after layer 0's
+        // gate sums) and the state is all there (its block notes that, at its end).  Each side writes its note, then looks
+        // at the other's: whichever comes last sees both and does the stores (twice the same values if both do).
+        auto store_parked = [&]() {
+            __threadfence();
+            bool all_read = true;
+            for (int z = lane; z < nb; z += 64)
+                all_read = all_read && __hip_atomic_load(p.notes + (long)z * kDecNoteWords + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g;
+            if (__ballot(!all_read) != 0ull) return;
+            for (int z = lane; z < nb; z += 64) {
+                if (__hip_atomic_load(p.notes + (long)z * kDecNoteWords + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != g) continue;
+                __threadfence();
+                for (int k = 0; k < L; ++k) {
+                    for (int u = 0; u < kDecUnits; ++u) {
+                        const int j = z * kDecUnits + u;
+                        if (j < H) {
+                            p.layer[k].hn[j] = p.parked_h[(long)k * H + j];
+                            p.layer[k].cn[j] = p.parked_c[(long)k * H + j];
+                        }
+                    }
+                }
+            }
+        };
+        constexpr int kLastExchange = has_cls ? L - 1 : L - 2;  // the last exchange of the step
+        bool parked = false;  // this block keeps its new state in the plan's memory instead of hn / cn
+        unsigned long long parked_seen = 0ull;
 
         // ---- where the caller wants the attention context stored, this block stores its own four columns ----
         if (pw == 0 && p.n_ctx_out > 0 && blockIdx.x * kDecUnits + kDecUnits <= H) {
@@ -476,32 +650,32 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
             const DecoderLayerArgs& ly = p.layer[k];
             dec_barrier();  // B1: the gate sums of layer k are in LDS
             const bool exchange = k + 1 < L || has_cls;
+            if (k == 0 && kLastExchange >= 0 && tid == kDecThreads - 64) {
+                // every wavefront of the block is past its reads of the step's inputs (the streamers have used h_prev of
+                // layer 0, the others have filled LDS): noted for whoever has parked state to store
+                __hip_atomic_store(my_notes + 1, g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             if (pw == 0) {
                 // (the streamers leave gate k in lane k, i.e. in part[.][k])
                 const float a = part[2 * pu][pg] + part[2 * pu + 1][pg] + bias_r[k];
-                const bool is_g = pg == 2;
-                const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
-                const float act = is_g ? 2.0f * sg - 1.0f : sg;
-                const float g_i = dpp_mov_f32<0x00>(act);
-                const float g_f = dpp_mov_f32<0x55>(act);
-                const float g_g = dpp_mov_f32<0xAA>(act);
-                const float g_o = dpp_mov_f32<0xFF>(act);
-                const float c_new = g_f * cprev_r[k] + g_i * g_g;
-                const half_t h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
-                const bool is_number = (c_new == c_new) && (g_o == g_o);
+                float c_new;
+                bool is_number;
+                const half_t h_new = dec_cell(a, pg, cprev_r[k], c_new, is_number);
+                half_t* const dst_h = parked ? p.parked_h + (long)k * H : ly.hn;
+                half_t* const dst_c = parked ? p.parked_c + (long)k * H : ly.cn;
                 const unsigned int hbits = p_ok ? (unsigned int)((is_number ? __builtin_bit_cast(unsigned short, h_new) : kDecNanCode) | flag)
                                                 : (unsigned int)flag;
                 if (owner) {
                     if (k == 0 && exchange) {
                         keep_h = h_new;
-                        keep_c = (half_t)c_new;
+                        keep_c = round_f16(c_new);
                     } else {
-                        ly.hn[pj] = h_new;
-                        ly.cn[pj] = (half_t)c_new;
+                        dst_h[pj] = h_new;
+                        dst_c[pj] = round_f16(c_new);
                     }
                     if (ly.out) {
                         half_t o = h_new;
-                        if (ly.residual) o = (half_t)((float)h_new + (float)in_vec[pj]);
+                        if (ly.residual) o = (half_t)((float)h_new + (float)in_vec[k & 1][pj]);
                         ly.out[pj] = o;
                     }
                 }
@@ -532,15 +706,29 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                     }
 #pragma unroll
                     for (int q = 0; q < QP; ++q) ok = ok && (got[q] & 0x4000400040004000ull) == want;
-                    if (ok || gave_up) break;
-                    if (give_up_check(spins)) break;
+                    if (ok || give_up_check(spins)) break;
+                }
+                // Entries that have not come: made here, bit for bit as their owners make them.
+#pragma unroll
+                for (int q = 0; q < QP; ++q) {
+                    const int blk = lane + 64 * (pw * QP + q);
+                    unsigned long long missing = __ballot(blk < nb && (got[q] & 0x4000400040004000ull) != want);
+                    if (missing != 0ull && k == 0 && lane == 0) parked_lds = 1u;
+                    while (__builtin_expect(missing != 0ull, 0)) {  // (said to be unlikely: 0.3 us of the undisturbed step)
+                        const int src = __builtin_ctzll(missing);
+                        missing &= missing - 1ull;
+                        const DecSubstituteLayer sl = {ly.w_ih, ly.w_hh, ly.bsum, ly.cx_proj, ly.in_w, ly.takes_ctx};
+                        const unsigned long long word = dec_substitute(sl, k == 0, src + 64 * (pw * QP + q), lane, H, p.x, p.att, p.enc_len, p.ctx_in != nullptr,
+                                                                       hprev[k], cprev[k], in_vec[k & 1], ctx_vec, flag);
+                        if (lane == src) got[q] = word;
+                    }
                 }
                 // the outputs of this lane's blocks; with a residual connection the next input is y + in
 #pragma unroll
                 for (int q = 0; q < QP; ++q) {
                     const int blk = lane + 64 * (pw * QP + q);
                     if (blk < nb) {
-                        const half4_t old = *reinterpret_cast<const half4_t*>(&in_vec[blk * 4]);
+                        const half4_t old = *reinterpret_cast<const half4_t*>(&in_vec[k & 1][blk * 4]);
                         half4_t nv;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
@@ -549,19 +737,39 @@ __global__ __launch_bounds__(kDecThreads) void decoder_step_f16_kernel(DecoderSt
                             if ((bits & 0x7fffu) == kDecNanCode) yv = __builtin_bit_cast(half_t, (unsigned short)0x7e00u);
                             nv[e] = ly.residual ? (half_t)((float)yv + (float)old[e]) : yv;
                         }
-                        *reinterpret_cast<half4_t*>(&in_vec[blk * 4]) = nv;
+                        *reinterpret_cast<half4_t*>(&in_vec[(k + 1) & 1][blk * 4]) = nv;
                     }
                 }
                 dec_barrier();  // B3: the next input is in LDS
-                if (k == 0 && owner) {
-                    // every block has published layer 0's output, so every block is past its reads of h_prev:
-                    // hn / cn may be the very buffers h_prev / c_prev were read from
-                    ly.hn[pj] = keep_h;
-                    ly.cn[pj] = keep_c;
+                if (k == 0) {
+                    // With every block's entry seen here, every block is past its reads of h_prev and c_prev, which hn / cn may
+                    // be.  Without (a wait gave up, the entries were made here), nobody knows that: the new state is parked.
+                    parked = parked_lds != 0u;
+                    if (owner) {
+                        (parked ? p.parked_h : ly.hn)[pj] = keep_h;
+                        (parked ? p.parked_c : ly.cn)[pj] = keep_c;
+                    }
+                }
+                if (k == 0 && pw == kDecPollWaves - 1) {
+                    // The look for parked state may come any time after this block's own note (a device-scope store, before the
+                    // polls that have just ended) has arrived: here the answer travels while the next layer is at work.
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    parked_seen = __hip_atomic_load(parked_any, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                if (k == kLastExchange && pw == kDecPollWaves - 1) {
+                    if (parked_seen == g) store_parked();
+                    if (lane == 0) __hip_atomic_store(my_notes, g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
         }
-        if (blockIdx.x == 0 && pw == 0 && lane == 0) __hip_atomic_store(p.g_counter, g + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (kLastExchange >= 0 && parked && pw == 0) {
+            __threadfence();  // the parked state is in place
+            if (lane == 0) {
+                __hip_atomic_store(parked_any, g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(my_notes + 2, g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            store_parked();
+        }
     }
 }
 

@@ -117,6 +117,15 @@ __device__ __forceinline__ void store16_device_scope(void* p, unsigned long long
 // becomes zero and a NaN stays a NaN; fmaxf would return its other operand for one.
 __device__ __forceinline__ float relu_f32(float v) { return v < 0.0f ? 0.0f : v; }
 
+// fp32 -> fp16 with the fp32 value made first.  Without the empty statement in between, hipcc folds a product or an fma
+// whose only use is the conversion into v_fma_mixlo_f16, which rounds once from the exact result; the same expression with a
+// second use rounds twice (fp32, then fp16).  Code paths that must agree bit for bit convert through this.
+__device__ __forceinline__ half_t round_f16(float v)
+{
+    asm volatile("" : "+v"(v));
+    return (half_t)v;
+}
+
 __device__ __forceinline__ float sigmoid_f32(float v) { return 1.0f / (1.0f + __expf(-v)); }
 
 // Sigmoid on the hardware exp2 and reciprocal (about 1 ulp each): exact limits 0 and 1 at -+inf, absolute error

@@ -711,9 +711,19 @@ class DecoderPlan:
         _check(L.load().pimhip_decoder_plan_set_spin_limit(self._handle, limit))
 
     def status(self):
-        """Raises NNRuntimeException if a step's kernel gave up a wait since the last report.  Synchronises."""
+        """Synchronises.  No step of this plan leaves an undefined result (a wait that gives up is made good inside the same
+        launch), so there is nothing to raise; fallbacks() counts such events."""
         torch.cuda.synchronize(self.device)
         _check(L.load().pimhip_decoder_plan_status(self._handle))
+
+    def fallbacks(self):
+        """(events, patient): steps of this plan in which a wait has given up so far, and whether waits still run to the
+        plan's poll limit (False once, after the third event, they are kept short).  Synchronises
+        (pimhip_decoder_plan_fallbacks)."""
+        torch.cuda.synchronize(self.device)
+        events, patient = ctypes.c_uint64(0), ctypes.c_int(0)
+        _check(L.load().pimhip_decoder_plan_fallbacks(self._handle, ctypes.byref(events), ctypes.byref(patient)))
+        return int(events.value), bool(patient.value)
 
     def bind(self, x, h_prev, c_prev, att=None, enc=None, ctx=None, hn=None, cn=None, outs=None, ctx_outs=(), logits=None):
         """Fixes the buffers of a step (lists of [H] tensors per layer; hn / cn default to h_prev / c_prev, i.e. the state is
