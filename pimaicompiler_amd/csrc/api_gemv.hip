@@ -62,7 +62,12 @@ void launch_mv(const half_t* W, const half_t* x, const half_t* b, half_t* y, int
 {
     constexpr int rows_per_block = (WAVES / KS) * R;
     const int grid = (N + rows_per_block - 1) / rows_per_block;
-    gemv_mv_f16_kernel<R, U, WAVES, KS><<<grid, WAVES * 64, 0, s>>>(W, x, b, y, N, K, ldw, relu);
+    // a matrix that fits the L2s is read with plain loads: the next launch on it finds its rows there (load_weight)
+    const int keep = (unsigned long long)N * (unsigned long long)K * sizeof(half_t) <= kKeepInL2Bytes;
+    if (keep)
+        gemv_mv_keep_f16_kernel<R, U, WAVES, KS><<<grid, WAVES * 64, 0, s>>>(W, x, b, y, N, K, ldw, relu);
+    else
+        gemv_mv_f16_kernel<R, U, WAVES, KS><<<grid, WAVES * 64, 0, s>>>(W, x, b, y, N, K, ldw, relu);
 }
 
 int gemv_mv(const half_t* W, const half_t* x, const half_t* bias, half_t* y, int64_t N, int64_t K, int64_t ldw,
@@ -258,20 +263,21 @@ extern "C" int pimhip_execute_gemv_cat2(void* out, const void* in1, int64_t in1_
     const int relu = act == PIMHIP_ACT_RELU;
     const int N = (int)out_w;
     const int split = (int)(in1_w >> 3);
+    const int keep = (unsigned long long)out_w * (unsigned long long)K * sizeof(half_t) <= kKeepInL2Bytes;
     // (the launch shapes of gemv_mv)
+    auto launch = [&](auto kernel, unsigned grid) {
+        kernel<<<grid, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split, (const half_t*)bias, (half_t*)out, N,
+                                    (int)K, (long)ldw, relu);
+    };
     if (out_w < 1024) {
         if (K >= 2048)
-            gemv_mv_cat2_f16_kernel<1, 4, 4, 4><<<N, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
-                                                                    (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+            keep ? launch(gemv_mv_cat2_f16_kernel<1, 4, 4, 4, true>, (unsigned)N) : launch(gemv_mv_cat2_f16_kernel<1, 4, 4, 4, false>, (unsigned)N);
         else
-            gemv_mv_cat2_f16_kernel<1, 2, 4, 4><<<N, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
-                                                                    (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+            keep ? launch(gemv_mv_cat2_f16_kernel<1, 2, 4, 4, true>, (unsigned)N) : launch(gemv_mv_cat2_f16_kernel<1, 2, 4, 4, false>, (unsigned)N);
     } else if (K >= 4096) {
-        gemv_mv_cat2_f16_kernel<2, 4, 4, 4><<<(N + 1) / 2, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
-                                                                          (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+        keep ? launch(gemv_mv_cat2_f16_kernel<2, 4, 4, 4, true>, (unsigned)(N + 1) / 2) : launch(gemv_mv_cat2_f16_kernel<2, 4, 4, 4, false>, (unsigned)(N + 1) / 2);
     } else {
-        gemv_mv_cat2_f16_kernel<2, 2, 4, 2><<<(N + 3) / 4, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split,
-                                                                          (const half_t*)bias, (half_t*)out, N, (int)K, (long)ldw, relu);
+        keep ? launch(gemv_mv_cat2_f16_kernel<2, 2, 4, 2, true>, (unsigned)(N + 3) / 4) : launch(gemv_mv_cat2_f16_kernel<2, 2, 4, 2, false>, (unsigned)(N + 3) / 4);
     }
     PIMHIP_HIP_CHECK(hipGetLastError());
     return PIMHIP_OK;
@@ -413,6 +419,7 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
         GemvGroupArgs g;
         memset(&g, 0, sizeof(g));
         int n = 0, blocks = 0;
+        unsigned long long weight_bytes = 0;
         for (; done + n < count && n < kGemvGroupMax; ++n) {
             const int i = done + n;
             if (!outs[i] || !ins[i] || !weights[i]) return fail(PIMHIP_ERR_INVALID_ARGUMENT, "entry %d has a null pointer", i);
@@ -430,12 +437,16 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
             g.K[n] = (int)in_ws[i];
             g.relu[n] = a == PIMHIP_ACT_RELU;
             g.block_begin[n] = blocks;
+            weight_bytes += (unsigned long long)out_ws[i] * (unsigned long long)in_ws[i] * sizeof(half_t);
             const int rows_per_block = gemv_group_rows_per_block((int)in_ws[i]);
             blocks += ((int)out_ws[i] + rows_per_block - 1) / rows_per_block;
         }
         g.block_begin[n] = blocks;
         g.count = n;
-        gemv_mv_f16_group_kernel<<<blocks, kGemvGroupThreads, 0, s>>>(g);
+        if (weight_bytes <= kKeepInL2Bytes)
+            gemv_mv_f16_group_kernel<true><<<blocks, kGemvGroupThreads, 0, s>>>(g);
+        else
+            gemv_mv_f16_group_kernel<false><<<blocks, kGemvGroupThreads, 0, s>>>(g);
         PIMHIP_HIP_CHECK(hipGetLastError());
         done += n;
     }

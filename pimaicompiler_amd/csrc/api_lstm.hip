@@ -792,12 +792,14 @@ int lstm_forward_impl(PimHipLstmPlan* plan, const void* x, const void* h0, const
                 }
                 float* cst = plan->c_state + (size_t)d * H;
                 const unsigned grid = (unsigned)((H + 3) / 4);
+                // what a step's launch reads: W_hh, and W_ih when the projection is made in the same kernel
+                const int keep = (unsigned long long)(4 * H) * (unsigned long long)(H + (fuse_xproj ? in_w : 0)) * sizeof(half_t) <= kKeepInL2Bytes;
                 for (int64_t step = 0; step < T; ++step) {
                     const int64_t t = d ? (T - 1 - step) : step;
                     const int64_t tp = d ? (t + 1) : (t - 1);
                     const half_t* h_prev = (step == 0) ? h0c : (yd + tp * y_stride);
                     const bool last = step == T - 1;
-                    lstm_step_f16_kernel<4><<<grid, 256, 0, s>>>(
+                    (keep ? lstm_step_f16_kernel<4, true> : lstm_step_f16_kernel<4, false>)<<<grid, 256, 0, s>>>(
                         c.w_ih, c.w_hh, c.bsum, fuse_xproj ? nullptr : (xp + t * 4 * H), layer_in + t * in_w, h_prev,
                         (step == 0) ? c0c : nullptr, cst, yd + t * y_stride, last ? hnc : nullptr, last ? cnc : nullptr,
                         (int)in_w, (int)H);

@@ -39,6 +39,22 @@ __device__ __forceinline__ float dot4(const half4_t w, const half4_t x, float ac
 // 16-byte streaming load of weight data that is read exactly once per launch.
 __device__ __forceinline__ half8_t load_stream(const half8_t* p) { return __builtin_nontemporal_load(p); }
 
+// The same with the choice of the cache policy.  A non-temporal load leaves nothing behind in the XCD's L2, which is what a
+// matrix far larger than the L2s wants (the GEMV sweep's 134 MB shapes lose 7 % with plain loads: the lines they leave
+// push out what other wavefronts still need).  A matrix that fits the eight L2s (32 MB together) and is used again by the
+// next launch, as in a decoding loop, wants the opposite: blocks land on the same XCDs launch after launch, and plain
+// loads find the rows in the L2 (a warm 1024 x 1024 product 2.52 -> 2.26 us, an LSTM step launch with 8 MB of W_hh
+// 3.9 -> 3.2 us, measured on MI355X).
+static constexpr unsigned long long kKeepInL2Bytes = 16ull << 20;  // weights of a launch up to this size use plain loads
+template <bool KEEP>
+__device__ __forceinline__ half8_t load_weight(const half8_t* p)
+{
+    if constexpr (KEEP)
+        return *p;
+    else
+        return __builtin_nontemporal_load(p);
+}
+
 // DPP controls (gfx9 encoding).
 static constexpr int kDppQuadXor1 = 0xB1;     // quad_perm:[1,0,3,2]
 static constexpr int kDppQuadXor2 = 0x4E;     // quad_perm:[2,3,0,1]

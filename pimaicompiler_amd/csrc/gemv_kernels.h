@@ -27,8 +27,8 @@ namespace pimhip
 // keeps U chunks per row in flight: R*U independent 16-byte weight loads per lane per iteration.
 // ---------------------------------------------------------------------------------------------
 // SPLIT: x is the concatenation of two vectors that lie apart (x: the first split_chunks 16-byte pieces, x2: the rest);
-// compiled out of every other instance.
-template <int R, int U, int WAVES, int KS, bool SPLIT = false>
+// compiled out of every other instance.  KEEP: the weight is read with plain loads (load_weight).
+template <int R, int U, int WAVES, int KS, bool SPLIT = false, bool KEEP = false>
 __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, const half_t* __restrict__ x,
                                                  const half_t* __restrict__ bias, half_t* __restrict__ y, int N,
                                                  int K, long ldw, int relu, int block,
@@ -67,7 +67,7 @@ __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, c
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) wr[r][u] = load_stream(wrow[r] + c + u * STEP);
+            for (int r = 0; r < R; ++r) wr[r][u] = load_weight<KEEP>(wrow[r] + c + u * STEP);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) xr[u] = x_at(c + u * STEP);
@@ -81,7 +81,7 @@ __device__ __forceinline__ void gemv_mv_f16_body(const half_t* __restrict__ W, c
     for (; c < nchunks; c += STEP) {
         half8_t wr[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) wr[r] = load_stream(wrow[r] + c);
+        for (int r = 0; r < R; ++r) wr[r] = load_weight<KEEP>(wrow[r] + c);
         const half8_t xr = x_at(c);
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[r] = dot8(wr[r], xr, acc[r]);
@@ -131,10 +131,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_kernel(const half_t* _
     gemv_mv_f16_body<R, U, WAVES, KS>(W, x, bias, y, N, K, ldw, relu, blockIdx.x);
 }
 
+// The same for a matrix that fits the L2s and is used launch after launch: plain loads (load_weight).  A kernel of its
+// own, chosen on the host, so that the streaming kernel stays as it is.
+template <int R, int U, int WAVES, int KS>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mv_keep_f16_kernel(const half_t* __restrict__ W,
+                                                                      const half_t* __restrict__ x,
+                                                                      const half_t* __restrict__ bias,
+                                                                      half_t* __restrict__ y, int N, int K, long ldw,
+                                                                      int relu)
+{
+    gemv_mv_f16_body<R, U, WAVES, KS, false, true>(W, x, bias, y, N, K, ldw, relu, blockIdx.x);
+}
+
 // y = act(W . cat(x1, x2) + bias) without the concatenation: the second operand of the RNNT joint network's first layer
 // is cat(encoder frame, prediction), which the reference either materialises or splits the product over
 // (compiler/source/frontend/optimizer/remove_cat_for_addmm.cpp:46-191: two dependent launches).
-template <int R, int U, int WAVES, int KS>
+template <int R, int U, int WAVES, int KS, bool KEEP>
 __global__ __launch_bounds__(WAVES * 64) void gemv_mv_cat2_f16_kernel(const half_t* __restrict__ W,
                                                                       const half_t* __restrict__ x1,
                                                                       const half_t* __restrict__ x2, int split_chunks,
@@ -142,7 +154,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_cat2_f16_kernel(const half
                                                                       half_t* __restrict__ y, int N, int K, long ldw,
                                                                       int relu)
 {
-    gemv_mv_f16_body<R, U, WAVES, KS, true>(W, x1, bias, y, N, K, ldw, relu, blockIdx.x, x2, split_chunks);
+    gemv_mv_f16_body<R, U, WAVES, KS, true, KEEP>(W, x1, bias, y, N, K, ldw, relu, blockIdx.x, x2, split_chunks);
 }
 
 // Several independent MV GEMVs in one launch (sibling projections that the reference issues on separate
@@ -167,15 +179,16 @@ static constexpr int kGemvGroupThreads = 256;
 static constexpr int kGemvGroupLongRow = 4096;
 __host__ __device__ inline int gemv_group_rows_per_block(int K) { return K >= kGemvGroupLongRow ? 2 : 4; }
 
+template <bool KEEP>  // the group's weights together fit the L2s: plain loads
 __global__ __launch_bounds__(kGemvGroupThreads) void gemv_mv_f16_group_kernel(GemvGroupArgs g)
 {
     int i = 0;
     while (i + 1 < g.count && (int)blockIdx.x >= g.block_begin[i + 1]) ++i;
     const int block = (int)blockIdx.x - g.block_begin[i];
     if (g.K[i] >= kGemvGroupLongRow)
-        gemv_mv_f16_body<2, 4, 4, 4>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i], block);
+        gemv_mv_f16_body<2, 4, 4, 4, false, KEEP>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i], block);
     else
-        gemv_mv_f16_body<2, 2, 4, 2>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i], block);
+        gemv_mv_f16_body<2, 2, 4, 2, false, KEEP>(g.W[i], g.x[i], g.bias[i], g.y[i], g.N[i], g.K[i], (long)g.K[i], g.relu[i], block);
 }
 
 // MV order, any K / leading dimension / alignment: one wavefront per row, 2-byte loads.

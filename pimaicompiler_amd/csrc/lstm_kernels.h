@@ -57,18 +57,12 @@ __device__ __forceinline__ float wave_sum_mod4(float v)
 // c_in_f16 (fp16) is read when non-null, else c_state (fp32); c_state is always written; h_out, and
 // hn_f16 / cn_f16 when non-null, receive the new state.
 // ---------------------------------------------------------------------------------------------
-template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
-    const half_t* __restrict__ w_ih, const half_t* __restrict__ w_hh, const float* __restrict__ bsum,
-    const float* __restrict__ xproj, const half_t* __restrict__ x, const half_t* __restrict__ h_prev,
-    const half_t* __restrict__ c_in_f16, float* __restrict__ c_state, half_t* __restrict__ h_out,
-    half_t* __restrict__ hn_f16, half_t* __restrict__ cn_f16, int I, int H)
+// The four gate sums of unit j, this lane's share: W_hh[rows of j] . h_prev, and W_ih[rows of j] . x when there is no xproj.
+template <bool KEEP>
+__device__ __forceinline__ void lstm_step_sums(float (&acc)[4], const half_t* __restrict__ w_ih, const half_t* __restrict__ w_hh,
+                                               const float* __restrict__ xproj, const half_t* __restrict__ x,
+                                               const half_t* __restrict__ h_prev, int I, int H, int j, int lane)
 {
-    const int lane = threadIdx.x & 63;
-    const int j = blockIdx.x * WAVES + (threadIdx.x >> 6);
-    if (j >= H) return;
-
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     {
         const half8_t* hv = reinterpret_cast<const half8_t*>(h_prev);
         const half8_t* w0 = reinterpret_cast<const half8_t*>(w_hh + (long)j * H);
@@ -79,8 +73,8 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
             half8_t wr[4][2];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                wr[g][0] = load_stream(w0 + g * gstride + c);
-                wr[g][1] = load_stream(w0 + g * gstride + c + 64);
+                wr[g][0] = load_weight<KEEP>(w0 + g * gstride + c);
+                wr[g][1] = load_weight<KEEP>(w0 + g * gstride + c + 64);
             }
             const half8_t h0 = hv[c], h1 = hv[c + 64];
 #pragma unroll
@@ -89,7 +83,7 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
         for (; c < nchunks; c += 64) {
             half8_t wr[4];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) wr[g] = load_stream(w0 + g * gstride + c);
+            for (int g = 0; g < 4; ++g) wr[g] = load_weight<KEEP>(w0 + g * gstride + c);
             const half8_t h0 = hv[c];
 #pragma unroll
             for (int g = 0; g < 4; ++g) acc[g] = dot8(wr[g], h0, acc[g]);
@@ -105,8 +99,8 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
             half8_t wr[4][2];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                wr[g][0] = load_stream(w0 + g * gstride + c);
-                wr[g][1] = load_stream(w0 + g * gstride + c + 64);
+                wr[g][0] = load_weight<KEEP>(w0 + g * gstride + c);
+                wr[g][1] = load_weight<KEEP>(w0 + g * gstride + c + 64);
             }
             const half8_t x0 = xv[c], x1 = xv[c + 64];
 #pragma unroll
@@ -115,12 +109,28 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
         for (; c < nchunks; c += 64) {
             half8_t wr[4];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) wr[g] = load_stream(w0 + g * gstride + c);
+            for (int g = 0; g < 4; ++g) wr[g] = load_weight<KEEP>(w0 + g * gstride + c);
             const half8_t x0 = xv[c];
 #pragma unroll
             for (int g = 0; g < 4; ++g) acc[g] = dot8(wr[g], x0, acc[g]);
         }
     }
+}
+
+// KEEP: the weights this launch reads fit the L2s and the next step's launch reads them again: plain loads (load_weight).
+template <int WAVES, bool KEEP>
+__global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
+    const half_t* __restrict__ w_ih, const half_t* __restrict__ w_hh, const float* __restrict__ bsum,
+    const float* __restrict__ xproj, const half_t* __restrict__ x, const half_t* __restrict__ h_prev,
+    const half_t* __restrict__ c_in_f16, float* __restrict__ c_state, half_t* __restrict__ h_out,
+    half_t* __restrict__ hn_f16, half_t* __restrict__ cn_f16, int I, int H)
+{
+    const int lane = threadIdx.x & 63;
+    const int j = blockIdx.x * WAVES + (threadIdx.x >> 6);
+    if (j >= H) return;
+
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    lstm_step_sums<KEEP>(acc, w_ih, w_hh, xproj, x, h_prev, I, H, j, lane);
     // The four gate sums are folded into one reduction: two halving exchanges leave gate l & 3 (i, f, g, o), summed over
     // its quad, in lane l, and the rest of the tree adds the sixteen quads.  Lanes 0..3 of every quad then activate one gate
     // each (sigmoid, and tanh(a) = 2 sigmoid(2a) - 1, on the hardware exp2 and reciprocal: absolute error below 1e-6) and

@@ -199,7 +199,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
 #pragma unroll
         for (int k = 0; k < kMoeFC; ++k) {
             if (64 * k >= nf) break;  // (uniform) pieces past the row for every lane
-            w2r[k] = load_stream(src + min(lane + 64 * k, nf - 1));
+            w2r[k] = load_weight<true>(src + min(lane + 64 * k, nf - 1));
         }
     };
 
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_ffn_step_f16_kernel(const hal
 #pragma unroll
         for (int k = 0; k < kMoeXC; ++k) {
             if (64 * k >= nx) break;
-            w1r[s][k] = load_stream(w1 + (long)r * nx + min(lane + 64 * k, nx - 1));
+            w1r[s][k] = load_weight<true>(w1 + (long)r * nx + min(lane + 64 * k, nx - 1));
         }
     }
 #pragma unroll
