@@ -31,7 +31,7 @@ POOL_BYTES_PER_SHAPE = 512 << 20
 # shape and one counter per run (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch, factors from --calibration-copy);
 # the per-shape figures and the commands are in profiles/gemv_sweep_pmc.md, and tests/test_profiles.py recomputes this
 # number from that file.  A counter reading, not something this script can measure itself.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 101093035
+DOMINANT_KERNEL_TRAFFIC_BYTES = 101094400
 
 
 def gemv_bytes(n, k, bias=True):
