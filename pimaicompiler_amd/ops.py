@@ -966,6 +966,9 @@ def aten_lstm2(data, batch_sizes, hx, params, has_biases, num_layers, dropout, t
     return y, hn.view(num_layers * D, 1, H), cn.view(num_layers * D, 1, H)
 
 
+RNNT_GREEDY_MAX_VOCAB = 512  # symbols the one-launch greedy loop keeps logits for (kRnntGreedyMaxVocab in csrc/rnnt_greedy_kernels.h)
+
+
 class RnntPlan:
     """One launch per (t, u) step of an RNN-transducer's greedy decoding loop (pimhip_rnnt_step): the prediction network's
     LSTM cells at seq_len 1 and the joint network relu(W1 . cat(f, g) + b1) -> W2 . + b2.  The reference runs
@@ -1059,7 +1062,8 @@ class RnntPlan:
         """The greedy decoding loop over the frames enc [T, F] in one launch (pimhip_rnnt_greedy_decode): returns
         (symbols int32 [max_symbols], result int32 [8], hn, cn [L, H]), all on the device and not synchronised; result[0] is
         the number of symbols.  embedding [rows >= V, I]: row k is the prediction network's input after symbol k; x0 [I] its
-        input before any symbol."""
+        input before any symbol.  A vocabulary of more than RNNT_GREEDY_MAX_VOCAB symbols runs the same loop driven from the
+        host (one step launch and one read of the argmax per iteration): the same outputs, several times slower."""
         lib = L.load()
         enc, embedding = enc.contiguous(), embedding.contiguous()
         given = [t for t in (enc, embedding, x0, h0, c0) if t is not None]
@@ -1077,6 +1081,9 @@ class RnntPlan:
             max_symbols = n_frames * max_symbols_per_frame
         symbols = torch.empty(max(int(max_symbols), 1), dtype=torch.int32, device=self.device)
         result = torch.zeros(8, dtype=torch.int32, device=self.device)
+        if self.vocab > RNNT_GREEDY_MAX_VOCAB:
+            return self._greedy_decode_from_the_host(enc, embedding, x0, int(blank), int(max_symbols_per_frame), int(max_symbols), h0, c0,
+                                                     bool(run_prediction_first), stream, symbols, result)
         hn = torch.empty(self.num_layers, self.hidden, dtype=torch.float16, device=self.device)
         cn = torch.empty_like(hn)
         ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
@@ -1085,6 +1092,44 @@ class RnntPlan:
                                              int(max_symbols), symbols.data_ptr(), result.data_ptr(), hn.data_ptr(), cn.data_ptr(),
                                              _stream_handle(stream)))
         return symbols[:int(max_symbols)], result, hn, cn
+
+    def _greedy_decode_from_the_host(self, enc, embedding, x0, blank, per_frame, max_symbols, h0, c0, run_prediction, stream, symbols,
+                                     result):
+        """The same loop for a vocabulary the loop kernel does not take (more than RNNT_GREEDY_MAX_VOCAB symbols): one
+        pimhip_rnnt_step and one argmax read back per iteration, as the reference's interpreter drives it
+        (examples/runtime/source/pipeline_manager.cpp:105).  Same outputs; synchronises every step."""
+        if not 0 <= blank < self.vocab:
+            raise NNRuntimeException(f"blank={blank} is not a symbol of the vocabulary of {self.vocab}")
+        if embedding.size(0) < self.vocab:
+            raise NNRuntimeException(f"embedding has {embedding.size(0)} rows for {self.vocab} symbols")
+        if per_frame < 1:
+            raise NNRuntimeException("max_symbols_per_frame must be at least 1")
+        if x0 is None and run_prediction:
+            raise NNRuntimeException("x0 (the prediction network's input before any symbol) is missing")
+        shape = (self.num_layers, self.hidden)
+        h = torch.zeros(shape, dtype=torch.float16, device=self.device) if h0 is None else h0.reshape(shape).clone()
+        c = torch.zeros(shape, dtype=torch.float16, device=self.device) if c0 is None else c0.reshape(shape).clone()
+        t, emitted, in_frame, label, steps = 0, [], 0, -1, 0
+        while t < enc.size(0) and len(emitted) < max_symbols:
+            if run_prediction:
+                logits, h, c = self.forward(x0 if label < 0 else embedding[label], h, c, enc[t], True, stream)
+            else:
+                logits, _, _ = self.forward(None, h, None, enc[t], False, stream)
+            # torch.argmax's choice: the first maximum, a NaN counting as the largest
+            nan = torch.isnan(logits)
+            k = int(nan.float().argmax()) if bool(nan.any()) else int(torch.argmax(logits.float()))
+            steps += 1
+            if k == blank:
+                t, in_frame, run_prediction = t + 1, 0, False
+            else:
+                emitted.append(k)
+                label, in_frame, run_prediction = k, in_frame + 1, True
+                if in_frame >= per_frame:
+                    t, in_frame = t + 1, 0
+        if emitted:
+            symbols[:len(emitted)] = torch.tensor(emitted, dtype=torch.int32, device=self.device)
+        result.copy_(torch.tensor([len(emitted), t, steps, 0, int(run_prediction), label, 0, 0], dtype=torch.int32))
+        return symbols[:max_symbols], result, h, c
 
     def forward(self, x, h_prev, c_prev, f, run_prediction=True, stream=None):
         """logits [V], hn, cn [L, H] for one step (new tensors; with run_prediction False hn, cn are h_prev, c_prev)."""

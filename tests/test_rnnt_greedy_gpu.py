@@ -310,9 +310,31 @@ def test_arguments_the_loop_refuses(ops):
         plan.greedy_decode(enc, embedding, None, 28)
     with pytest.raises(ops.NNRuntimeException, match=r"\[T, 1024\]"):
         plan.greedy_decode(enc[:, :512], embedding, x0, 28)
-    # more symbols than the loop kernel keeps logits for
+    # more symbols than the loop kernel keeps logits for: the C ABI says so (the Python layer then drives the loop itself, below)
     g2, params2, joint2 = make(7272, 1, 64, 32, 128, 64, 600, True)
     plan2 = ops.RnntPlan(dev(params2), True, 1, tuple(dev(joint2)))
-    with pytest.raises(ops.NNRuntimeException, match="symbols"):
-        plan2.greedy_decode(torch.zeros(4, 128, dtype=torch.float16, device=DEV), torch.zeros(600, 64, dtype=torch.float16, device=DEV),
-                            torch.zeros(64, dtype=torch.float16, device=DEV), 0)
+    import ctypes
+    from pimaicompiler_amd import _lib
+    z = lambda *shape: torch.zeros(*shape, dtype=torch.float16, device=DEV)  # noqa: E731
+    e4, emb, x64, st = z(4, 128), z(600, 64), z(64), z(1, 32)
+    sym, res = torch.zeros(8, dtype=torch.int32, device=DEV), torch.zeros(8, dtype=torch.int32, device=DEV)
+    rc = _lib.load().pimhip_rnnt_greedy_decode(plan2._handle, e4.data_ptr(), 4, emb.data_ptr(), 600, x64.data_ptr(), None, None, 1, 0, 30, 8,
+                                               sym.data_ptr(), res.data_ptr(), st.data_ptr(), st.clone().data_ptr(), None)
+    assert rc == _lib.PIMHIP_ERR_UNSUPPORTED
+    with pytest.raises(ops.NNRuntimeException, match="blank"):
+        plan2.greedy_decode(e4, emb, x64, 600)
+
+
+def test_a_vocabulary_the_loop_kernel_does_not_take_is_decoded_from_the_host(ops):
+    """600 symbols: ops.RnntPlan.greedy_decode drives pimhip_rnnt_step itself and returns what the one-launch loop returns
+    (same fields, same meaning); checked against this file's own host loop and, for the first steps, LibTorch CPU."""
+    L, I, H, F, J, V, T, blank = 1, 64, 32, 128, 64, 600, 20, 599
+    params, joint, enc, embedding, x0 = model(7373, L, I, H, F, J, V, T, blank, 0.35)
+    plan = ops.RnntPlan(dev(params), True, L, tuple(dev(joint)))
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, 3, T * 3)
+    r = check(plan.greedy_decode(enc, embedding, x0, blank, 3), want)
+    print(f"600 symbols from the host: {r[0]} symbols over {r[1]} frames in {r[2]} steps", flush=True)
+    assert r[1] == T and r[0] > 0 and r[3] == 0
+    # a budget of symbols ends the loop as it ends the kernel's
+    want = loop_driven_from_the_host(plan, enc, embedding, x0, blank, 3, 4)
+    check(plan.greedy_decode(enc, embedding, x0, blank, 3, 4), want)
