@@ -757,7 +757,8 @@ def main():
             "read_only_kernel_us": round(probe_us, 2),
             "bytes": dec_step_bytes,
             "max_abs_diff_of_logits_to_the_8_launch_step": round(fused_err, 6),
-            "set_encoder_once_per_sentence_us": round(timed_us(reproject, 20), 2)}
+            "set_encoder_once_per_sentence_us": round(timed_us(reproject, 20), 2),
+            "waits_that_gave_up": fplan.fallbacks()[0]}
         progress("other: the reference's own GEMV kernel")
         # the reference's own HIP GEMV (custom_ops.h addmv_kernel_Axy, compiled from its tree) on the same cold weights
         from oracle import oracle  # the loader of the reference's own kernels, nothing else of the oracle
