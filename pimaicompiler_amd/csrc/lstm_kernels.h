@@ -129,6 +129,16 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
     const int j = blockIdx.x * WAVES + (threadIdx.x >> 6);
     if (j >= H) return;
 
+    // what the cell needs besides the sums, asked for before the weights: it arrives behind them at no cost, where a load
+    // after the reduction is a trip to the L2 of its own at the end of a short kernel
+    const int gate = lane & 3;
+    float addend = 0.0f;
+    if (xproj)
+        addend = xproj[(long)gate * H + j];
+    else if (bsum)
+        addend = bsum[(long)gate * H + j];
+    const float c_prev = c_in_f16 ? (float)c_in_f16[j] : c_state[j];
+
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     lstm_step_sums<KEEP>(acc, w_ih, w_hh, xproj, x, h_prev, I, H, j, lane);
     // The four gate sums are folded into one reduction: two halving exchanges leave gate l & 3 (i, f, g, o), summed over
@@ -141,11 +151,7 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
     const float a1 = (b0 ? acc[3] : acc[2]) + dpp_mov_f32<kDppQuadXor1>(b0 ? acc[2] : acc[3]);
     float a = (b1 ? a1 : a0) + dpp_mov_f32<kDppQuadXor2>(b1 ? a0 : a1);
     a = wave_sum_mod4(a);
-    const int gate = lane & 3;
-    if (xproj)
-        a += xproj[(long)gate * H + j];
-    else if (bsum)
-        a += bsum[(long)gate * H + j];
+    a += addend;
     const bool is_g = gate == 2;
     const float sg = fast_sigmoid_f32(is_g ? 2.0f * a : a);
     const float act = is_g ? 2.0f * sg - 1.0f : sg;
@@ -153,7 +159,6 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
     const float g_f = dpp_mov_f32<0x55>(act);
     const float g_g = dpp_mov_f32<0xAA>(act);
     const float g_o = dpp_mov_f32<0xFF>(act);
-    const float c_prev = c_in_f16 ? (float)c_in_f16[j] : c_state[j];
     const float c_new = g_f * c_prev + g_i * g_g;
     const half_t h_new = (half_t)(g_o * (2.0f * fast_sigmoid_f32(2.0f * c_new) - 1.0f));
     if (lane == 0) {
