@@ -62,8 +62,8 @@ void launch_mv(const half_t* W, const half_t* x, const half_t* b, half_t* y, int
 {
     constexpr int rows_per_block = (WAVES / KS) * R;
     const int grid = (N + rows_per_block - 1) / rows_per_block;
-    // a matrix that fits the L2s is read with plain loads: the next launch on it finds its rows there (load_weight)
-    const int keep = (unsigned long long)N * (unsigned long long)K * sizeof(half_t) <= kKeepInL2Bytes;
+    // a small matrix is read with plain loads: its rows are still cached when its turn comes again (load_weight)
+    const int keep = (unsigned long long)N * (unsigned long long)K * sizeof(half_t) <= kKeepCachedBytes;
     if (keep)
         gemv_mv_keep_f16_kernel<R, U, WAVES, KS><<<grid, WAVES * 64, 0, s>>>(W, x, b, y, N, K, ldw, relu);
     else
@@ -263,7 +263,7 @@ extern "C" int pimhip_execute_gemv_cat2(void* out, const void* in1, int64_t in1_
     const int relu = act == PIMHIP_ACT_RELU;
     const int N = (int)out_w;
     const int split = (int)(in1_w >> 3);
-    const int keep = (unsigned long long)out_w * (unsigned long long)K * sizeof(half_t) <= kKeepInL2Bytes;
+    const int keep = (unsigned long long)out_w * (unsigned long long)K * sizeof(half_t) <= kKeepCachedBytes;
     // (the launch shapes of gemv_mv)
     auto launch = [&](auto kernel, unsigned grid) {
         kernel<<<grid, 256, 0, s>>>((const half_t*)weight, (const half_t*)in1, (const half_t*)in2, split, (const half_t*)bias, (half_t*)out, N,
@@ -443,7 +443,7 @@ extern "C" int pimhip_execute_gemv_group(int count, void* const* outs, const voi
         }
         g.block_begin[n] = blocks;
         g.count = n;
-        if (weight_bytes <= kKeepInL2Bytes)
+        if (weight_bytes <= kKeepCachedBytes)
             gemv_mv_f16_group_kernel<true><<<blocks, kGemvGroupThreads, 0, s>>>(g);
         else
             gemv_mv_f16_group_kernel<false><<<blocks, kGemvGroupThreads, 0, s>>>(g);

@@ -793,7 +793,7 @@ int lstm_forward_impl(PimHipLstmPlan* plan, const void* x, const void* h0, const
                 float* cst = plan->c_state + (size_t)d * H;
                 const unsigned grid = (unsigned)((H + 3) / 4);
                 // what a step's launch reads: W_hh, and W_ih when the projection is made in the same kernel
-                const int keep = (unsigned long long)(4 * H) * (unsigned long long)(H + (fuse_xproj ? in_w : 0)) * sizeof(half_t) <= kKeepInL2Bytes;
+                const int keep = (unsigned long long)(4 * H) * (unsigned long long)(H + (fuse_xproj ? in_w : 0)) * sizeof(half_t) <= kKeepCachedBytes;
                 for (int64_t step = 0; step < T; ++step) {
                     const int64_t t = d ? (T - 1 - step) : step;
                     const int64_t tp = d ? (t + 1) : (t - 1);

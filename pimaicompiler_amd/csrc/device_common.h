@@ -39,13 +39,14 @@ __device__ __forceinline__ float dot4(const half4_t w, const half4_t x, float ac
 // 16-byte streaming load of weight data that is read exactly once per launch.
 __device__ __forceinline__ half8_t load_stream(const half8_t* p) { return __builtin_nontemporal_load(p); }
 
-// The same with the choice of the cache policy.  A non-temporal load leaves nothing behind in the XCD's L2, which is what a
-// matrix far larger than the L2s wants (the GEMV sweep's 134 MB shapes lose 7 % with plain loads: the lines they leave
-// push out what other wavefronts still need).  A matrix that fits the eight L2s (32 MB together) and is used again by the
-// next launch, as in a decoding loop, wants the opposite: blocks land on the same XCDs launch after launch, and plain
-// loads find the rows in the L2 (a warm 1024 x 1024 product 2.52 -> 2.26 us, an LSTM step launch with 8 MB of W_hh
-// 3.9 -> 3.2 us, measured on MI355X).
-static constexpr unsigned long long kKeepInL2Bytes = 16ull << 20;  // weights of a launch up to this size use plain loads
+// The same with the choice of the cache policy.  Lines read with non-temporal loads are the first the caches drop, which
+// is what a matrix far larger than the caches wants (the GEMV sweep's 134 MB shapes lose 7 % with plain loads: the lines
+// they leave push out what other wavefronts still need).  The weights of a decoding loop are small and come round again
+// every token, with other weights read in between: read with plain loads they stay in the caches (the XCDs' L2s and the
+// 256 MB Infinity Cache behind them) until then.  Measured on MI355X, graph replays: one 1024 x 1024 matrix multiplied
+// over and over 2.0 us either way; 64 such matrices in turn (134 MB) 2.43 us non-temporal, 2.19 us plain; 512 in turn
+// (1 GB, more than the caches hold) 2.45 us either way; the three products of the mixture-of-experts step 7.3 -> 6.3 us.
+static constexpr unsigned long long kKeepCachedBytes = 16ull << 20;  // the weights of a launch up to this size are read with plain loads
 template <bool KEEP>
 __device__ __forceinline__ half8_t load_weight(const half8_t* p)
 {

@@ -131,7 +131,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mv_f16_kernel(const half_t* _
     gemv_mv_f16_body<R, U, WAVES, KS>(W, x, bias, y, N, K, ldw, relu, blockIdx.x);
 }
 
-// The same for a matrix that fits the L2s and is used launch after launch: plain loads (load_weight).  A kernel of its
+// The same for a small matrix that is used again and again between other work: plain loads (load_weight).  A kernel of its
 // own, chosen on the host, so that the streaming kernel stays as it is.
 template <int R, int U, int WAVES, int KS>
 __global__ __launch_bounds__(WAVES * 64) void gemv_mv_keep_f16_kernel(const half_t* __restrict__ W,
@@ -179,7 +179,7 @@ static constexpr int kGemvGroupThreads = 256;
 static constexpr int kGemvGroupLongRow = 4096;
 __host__ __device__ inline int gemv_group_rows_per_block(int K) { return K >= kGemvGroupLongRow ? 2 : 4; }
 
-template <bool KEEP>  // the group's weights together fit the L2s: plain loads
+template <bool KEEP>  // the group's weights together are small: plain loads (load_weight)
 __global__ __launch_bounds__(kGemvGroupThreads) void gemv_mv_f16_group_kernel(GemvGroupArgs g)
 {
     int i = 0;

@@ -117,7 +117,7 @@ __device__ __forceinline__ void lstm_step_sums(float (&acc)[4], const half_t* __
     }
 }
 
-// KEEP: the weights this launch reads fit the L2s and the next step's launch reads them again: plain loads (load_weight).
+// KEEP: the weights this launch reads are small and the next step's launch reads them again: plain loads (load_weight).
 template <int WAVES, bool KEEP>
 __global__ __launch_bounds__(WAVES * 64) void lstm_step_f16_kernel(
     const half_t* __restrict__ w_ih, const half_t* __restrict__ w_hh, const float* __restrict__ bsum,
